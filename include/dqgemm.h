@@ -1,0 +1,75 @@
+/* C-ABI of libdqgemm.so: hand-written gfx950 kernels for the dequantize-GEMM path.
+ *
+ * Convention (the one the reference's kernel adapter generates for every JIT kernel,
+ * tilelang/jit/adapter/wrapper.py:59-85,719-736): plain device pointers, explicit sizes,
+ * the HIP stream as the last argument, return 0 on success and -1 on error with the
+ * message available from get_last_error().  Launches are asynchronous on `stream`; no
+ * entry point allocates, frees or synchronises.  The caller owns every buffer.
+ *
+ * All matrices are row-major and contiguous.  Packed weights keep the examples' layout:
+ * B[N, K*bits/8] bytes, low field = lowest k.
+ */
+#ifndef DQGEMM_H_
+#define DQGEMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* dq_stream_t; /* hipStream_t */
+
+/* ---- library ------------------------------------------------------------------------ */
+
+/* Replaces `int init()` of the generated host stub (tilelang/jit/adapter/wrapper.py:75-85,
+ * :33-57): clears the error buffer, checks a gfx950 device is current and that the
+ * largest dynamic-LDS request of any kernel fits the device limit. */
+int init(void);
+
+/* Replaces `const char* get_last_error()` (tilelang/jit/adapter/wrapper.py:71-73):
+ * static 1024-byte buffer, not thread safe. */
+const char* get_last_error(void);
+
+/* ---- enums (int arguments below) ------------------------------------------------------ */
+
+/* file names below are under examples/dequantize_gemm/quantize/ */
+enum dq_w4_mode {
+  DQ_W4_UNSIGNED = 0,       /* w = q                      quantization.py:310-318, lop3.py:35-39 (i4u) */
+  DQ_W4_SIGNED = 1,         /* w = sext4(q)               quantization.py:333-343                      */
+  DQ_W4_OFFSET8 = 2,        /* w = q - 8                  quantization.py:298-307, lop3.py:29-33 (i4s) */
+  DQ_W4_SCALE = 3,          /* w = rne16((q-8)*s)         lop3.py:41-75 (i4s_scale)                    */
+  DQ_W4_USCALE = 4,         /* w = rne16(q*s)             lop3.py:77-81 (i4u_scale)                    */
+  DQ_W4_ZEROS_ORIGINAL = 5, /* w = rne16(rne16(q-z)*s)    lop3.py:136-176, quantization.py:321-330     */
+  DQ_W4_ZEROS_RESCALE = 6   /* w = rne16(fma(q,s,-z))     lop3.py:233-271                              */
+};
+
+enum dq_w4_layout {
+  DQ_LAYOUT_PLAIN = 0,      /* nibble e of each 32-bit word is element e                         */
+  DQ_LAYOUT_INTERLEAVED = 1 /* words pre-permuted by interleave_weight(.., 4, "float16"),
+                               examples/dequantize_gemm/quantize/utils.py:71-125              */
+};
+
+/* ---- W4A16 ---------------------------------------------------------------------------- */
+
+/* C[M,N] fp16 = A[M,K] fp16 . dequant(B[N,K/2], Scale[N,K/group], Zeros[N,K/group])^T,
+ * fp32 accumulation.  Replaces `call(A, B, C, stream)` of the kernel generated from
+ * examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:83-153 (M = 1) and its
+ * batched use (M up to 64 per pass; larger M loops over blocks of 64 rows).
+ * Requires K % 128 == 0, group % 32 == 0, K % group == 0 (group = K when there is one
+ * scale per row).  Scale / Zeros may be NULL for modes that do not read them.
+ * `variant` < 0 selects the kernel configuration heuristically. */
+int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M,
+                               int N, int K, int group, int mode, int layout, int variant, dq_stream_t stream);
+
+/* W[N,K] fp16 = dequant(B, Scale, Zeros): the dequantised weight tile with the same
+ * device decoder the GEMV/GEMM kernels use.  Replaces the `_convert_test`-style kernels
+ * of the examples (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:36-65). */
+int call_dequantize_w4(const void* B, const void* Scale, const void* Zeros, void* W, int N, int K, int group,
+                       int mode, int layout, dq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DQGEMM_H_ */

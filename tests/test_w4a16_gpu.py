@@ -1,0 +1,200 @@
+"""GPU parity of the W4A16 path (through the C-ABI) against the CPU oracle.
+
+Bars: dequantised tiles bit-exact; fp16 GEMV/GEMM outputs within rtol=1e-2, atol=1e-2 of
+``A.float() @ W_deq.float().T -> fp16`` with no allowance for mismatching elements.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from tilelang_amd import workloads
+from oracle import dq_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2
+
+
+def _dev(x, cuda):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(cuda)
+
+
+def _mode_kwargs(mode):
+    return {
+        "unsigned": dict(source_format="uint", fast_decoding=True, with_scaling=False),
+        "signed": dict(source_format="uint", fast_decoding=False, with_scaling=False),
+        "offset8": dict(source_format="int", fast_decoding=True, with_scaling=False),
+        "scale": dict(source_format="int", with_scaling=True),
+        "uscale": dict(source_format="uint", with_scaling=True),
+        "original": dict(source_format="uint", with_scaling=True, with_zeros=True, zeros_mode="original"),
+        "rescale": dict(source_format="uint", with_scaling=True, with_zeros=True, zeros_mode="rescale"),
+    }[mode]
+
+
+def _oracle_tile(mode, B, S, Z, group):
+    if mode == "unsigned":
+        return orc.dequant_u4_plain(B, signed=False)
+    if mode == "signed":
+        return orc.dequant_u4_plain(B, signed=True)
+    if mode == "offset8":
+        return (orc.unpack_u4(B).astype(np.float32) - 8).astype(np.float16)
+    if mode == "scale":
+        return orc.dequant_u4_scale(B, S, group)
+    if mode == "uscale":
+        q = orc.unpack_u4(B).astype(np.float32)
+        s = np.repeat(S, group, axis=1).astype(np.float32)
+        return (q * s + np.float32(0)).astype(np.float16)
+    return orc.dequant_u4_scale_zeros(B, S, Z, group, mode)
+
+
+@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_dequant_tile_bit_exact(cuda, mode, interleaved):
+    N, K, group = 96, 512, 128
+    d = workloads.w4a16(1, N, K, group, seed=3, scale_range=(0.002, 0.02), zeros_range=(6, 10))
+    B, S, Z = d["B"], d["Scale"], d["Zeros"]
+    # every nibble value next to every other, extreme scales, non-integer and negative zeros
+    B[0, :128] = np.arange(256, dtype=np.uint8)[::2] | 0
+    B[1, :] = np.arange(K // 2, dtype=np.uint8)
+    S[2, :] = np.array([6.1e-5, 1.0, -0.013, 655.0], dtype=np.float16)
+    Z[3, :] = np.array([7.5, -3.25, 0.0, 15.0], dtype=np.float16)
+    expected = _oracle_tile(mode, B, S, Z, group)
+
+    kw = _mode_kwargs(mode)
+    fast = kw.pop("fast_decoding", False)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = tl.quantize.interleave_weight(Bdev, 4, "float16")
+    # the tile kernel takes the layout from fast_decoding; the decode formula from the rest
+    kern = tl.dequantize_w4(N, K, group, fast_decoding=interleaved, _formula_fast=fast, **kw)
+    args = [Bdev]
+    if kw.get("with_scaling"):
+        args.append(_dev(S, cuda))
+    if kw.get("with_zeros"):
+        args.append(_dev(Z, cuda))
+    W = kern(*args)
+    torch.cuda.synchronize()
+    got = W.cpu().numpy()
+    assert got.dtype == np.float16 and got.shape == (N, K)
+    np.testing.assert_array_equal(got.view(np.uint16), expected.view(np.uint16))
+
+
+def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False, scale_range=(0.005, 0.02)):
+    d = workloads.w4a16(M, N, K, group, seed=seed, scale_range=scale_range, zeros_range=(6, 10))
+    kw = _mode_kwargs(mode)
+    fast = kw.pop("fast_decoding", False)
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, fast_decoding=interleaved,
+                              _formula_fast=fast, variant=variant, **kw)
+    Bdev = _dev(d["B"], cuda).view(torch.int8)
+    if interleaved:
+        Bdev = tl.quantize.interleave_weight(Bdev, 4, "float16")
+    args = [_dev(d["A"], cuda), Bdev]
+    if kw.get("with_scaling"):
+        args.append(_dev(d["Scale"], cuda))
+    if kw.get("with_zeros"):
+        args.append(_dev(d["Zeros"], cuda))
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(*args, C)
+    torch.cuda.synchronize()
+    W = _oracle_tile(mode, d["B"], d["Scale"], d["Zeros"], group)
+    ref = (d["A"].astype(np.float32) @ W.astype(np.float32).T).astype(np.float16)
+    got = C.cpu().numpy()
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+    return got
+
+
+@pytest.mark.parametrize("N,K", [(1024, 1024), (4096, 4096), (11008, 4096), (4096, 11008)])
+def test_gemv_m1_configs(cuda, N, K):
+    """Benchmark configurations 1 and 2: M=1, w=(q-8)*s, group 128."""
+    _run_gemv(cuda, 1, N, K, 128, "scale")
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 7, 16, 17, 33, 64, 65, 130])
+def test_small_batch_zeros(cuda, M):
+    """Configuration 3's decode ((q-z)*s, zeros 6..10) at a size the oracle finishes quickly."""
+    _run_gemv(cuda, M, 1536, 1024, 128, "original", scale_range=(0.002, 0.01))
+
+
+@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "uscale", "rescale"])
+def test_gemv_other_modes(cuda, mode):
+    _run_gemv(cuda, 2, 512, 512, 128, mode, scale_range=(0.002, 0.01))
+
+
+@pytest.mark.parametrize("interleaved", [True])
+def test_gemv_interleaved_layout(cuda, interleaved):
+    _run_gemv(cuda, 1, 512, 1024, 128, "scale", interleaved=interleaved)
+    _run_gemv(cuda, 5, 512, 1024, 128, "original", interleaved=interleaved)
+
+
+@pytest.mark.parametrize("N", [1, 3, 15, 16, 17, 63, 65, 130])
+def test_ragged_n(cuda, N):
+    _run_gemv(cuda, 1, N, 256, 128, "scale")
+    _run_gemv(cuda, 3, N, 384, 128, "original")
+
+
+@pytest.mark.parametrize("group", [32, 64, 128, 256, -1])
+def test_group_sizes(cuda, group):
+    K = 1280 if group == -1 else 1024
+    _run_gemv(cuda, 1, 256, K, K if group == -1 else group, "scale")
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
+def test_kernel_variants(cuda, variant):
+    _run_gemv(cuda, 4, 1000, 2048, 128, "scale", variant=variant)
+    _run_gemv(cuda, 1, 1000, 2048 + 128, 128, "original", variant=variant)
+
+
+def test_multi_tile_k(cuda):
+    """K large enough that the activations are staged in several LDS tiles."""
+    _run_gemv(cuda, 16, 256, 8192, 128, "scale")
+    _run_gemv(cuda, 64, 128, 4096, 128, "original")
+
+
+def test_deterministic(cuda):
+    a = _run_gemv(cuda, 1, 4096, 4096, 128, "scale", seed=5)
+    b = _run_gemv(cuda, 1, 4096, 4096, 128, "scale", seed=5)
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+
+
+def test_full_size_linearity(cuda):
+    """North-star shape (N=28672, K=8192), checked without the oracle: with every scale equal to s and every
+    nibble equal to q the output is (q-8)*s*sum(A), and the kernel is linear in A."""
+    M, N, K, group = 1, 28672, 8192, 128
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    q = 11
+    B = torch.full((N, K // 2), q | (q << 4), dtype=torch.uint8, device=cuda).view(torch.int8)
+    S = torch.full((N, K // group), 0.0078125, dtype=torch.float16, device=cuda)
+    C = torch.empty((M, N), dtype=torch.float16, device=cuda)
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, source_format="int", with_scaling=True)
+    kern(_dev(A, cuda), B, S, C)
+    torch.cuda.synchronize()
+    expect = np.float32((q - 8) * 0.0078125) * A.astype(np.float32).sum()
+    np.testing.assert_allclose(C.cpu().numpy().astype(np.float32), np.full((M, N), expect, np.float32), rtol=RTOL, atol=ATOL)
+    # random weights: C(A1 + A2) == C(A1) + C(A2) up to fp16 rounding of the outputs
+    d = workloads.w4a16(1, N, K, group, seed=1)
+    A2 = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    Bd, Sd = _dev(d["B"], cuda).view(torch.int8), _dev(d["Scale"], cuda)
+    outs = []
+    for a in (d["A"], A2, (d["A"].astype(np.float32) + A2.astype(np.float32)).astype(np.float16)):
+        Ci = torch.empty((M, N), dtype=torch.float16, device=cuda)
+        kern(_dev(a, cuda), Bd, Sd, Ci)
+        outs.append(Ci.float().cpu().numpy())
+    np.testing.assert_allclose(outs[2], outs[0] + outs[1], rtol=2e-2, atol=5e-2)
+    # a sample of rows against the oracle
+    rows = rng.choice(N, 64, replace=False)
+    W = orc.dequant_u4_scale(d["B"][rows], d["Scale"][rows], group)
+    ref = (d["A"].astype(np.float32) @ W.astype(np.float32).T).astype(np.float16)
+    np.testing.assert_allclose(outs[0][:, rows], ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+
+
+def test_null_pointer_and_bad_args(cuda):
+    kern = tl.dequantize_gemv(1, 64, 256, group_size=128, source_format="int", with_scaling=True)
+    A = torch.zeros((1, 256), dtype=torch.float16, device=cuda)
+    B = torch.zeros((64, 128), dtype=torch.int8, device=cuda)
+    C = torch.zeros((1, 64), dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError, match="Kernel call failed: .*Scale is expected to have non-NULL data pointer"):
+        kern(A, B, None, C)

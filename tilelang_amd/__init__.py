@@ -1,0 +1,13 @@
+"""MI355X-native dequantize-GEMM kernels behind the call surface of TileLang's examples.
+
+Hand-written gfx950 HIP kernels in ``libdqgemm.so`` (C-ABI: ``include/dqgemm.h``), a thin
+ctypes adapter with the reference adapter's call contract, and factories named after the
+examples' kernels.  PyTorch is used for tensors and streams only.
+"""
+
+from . import quantize  # noqa: F401
+from .adapter import KernelAdapter, KernelParam  # noqa: F401
+from .kernels import dequantize_gemv, dequantize_w4  # noqa: F401
+from .profiler import Profiler, TensorSupplyType, do_bench  # noqa: F401
+
+__version__ = "0.1.0"

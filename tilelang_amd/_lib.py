@@ -1,0 +1,83 @@
+"""ctypes loader for ``libdqgemm.so`` (the C-ABI declared in ``include/dqgemm.h``).
+
+The reference loads each JIT-built kernel library with ``ctypes.CDLL`` and calls ``init()``
+once (tilelang/jit/adapter/libgen.py:52-57, tilelang/jit/adapter/cython/adapter.py:131-140).
+Here there is one ahead-of-time library.  There is no fallback: if it is missing or fails
+to load, every kernel call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+import threading
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libdqgemm.so")
+CSRC_DIR = os.path.join(_PKG_DIR, "csrc")
+
+_lock = threading.Lock()
+_lib = None
+_initialised = False
+
+_vp, _i = ctypes.c_void_p, ctypes.c_int
+
+#: name -> argtypes; every entry point returns int (0 ok / -1 error) except get_last_error
+SIGNATURES = {
+    "init": [],
+    "call_dequantize_gemv_w4a16": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "call_dequantize_w4": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+}
+
+
+class LibraryNotBuiltError(RuntimeError):
+    pass
+
+
+def build_library(jobs: int = 8, clean: bool = False) -> str:
+    """Compile every HIP source for gfx950 into ``libdqgemm.so`` (hipcc cross-compiles without a GPU)."""
+    if clean:
+        subprocess.run(["make", "-C", CSRC_DIR, "clean"], check=True, capture_output=True)
+    proc = subprocess.run(["make", "-C", CSRC_DIR, f"-j{jobs}"], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building libdqgemm.so failed:\n{proc.stdout[-4000:]}\n{proc.stderr[-4000:]}")
+    return LIB_PATH
+
+
+def load_library() -> ctypes.CDLL:
+    """Load the library and bind the signatures (no GPU call is made)."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise LibraryNotBuiltError(
+                    f"{LIB_PATH} is missing: build it with `make -C {CSRC_DIR}` "
+                    "(or `python -c 'import __graft_entry__ as g; g.build()'`). There is no fallback path."
+                )
+            lib = ctypes.CDLL(LIB_PATH)
+            lib.get_last_error.restype = ctypes.c_char_p
+            lib.get_last_error.argtypes = []
+            for name, argtypes in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = ctypes.c_int
+                fn.argtypes = argtypes
+            _lib = lib
+    return _lib
+
+
+def get_library() -> ctypes.CDLL:
+    """Library ready for kernel calls: loaded and ``init()`` run once on the current device."""
+    global _initialised
+    lib = load_library()
+    if not _initialised:
+        with _lock:
+            if not _initialised:
+                if lib.init() != 0:
+                    raise RuntimeError(f"libdqgemm init failed: {lib.get_last_error().decode()}")
+                _initialised = True
+    return lib
+
+
+def last_error() -> str:
+    return load_library().get_last_error().decode("utf-8", "replace")

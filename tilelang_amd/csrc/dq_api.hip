@@ -1,0 +1,82 @@
+// extern "C" entry points of libdqgemm.so (declared in include/dqgemm.h).
+//
+// Same shape as the host stub the reference's adapter generates around every JIT kernel
+// (tilelang/jit/adapter/wrapper.py:59-85): init / get_last_error / call, raw pointers and
+// sizes in, 0 or -1 out, message in a static buffer.  Argument checks run before any
+// launch so a bad call never reaches the GPU.
+#include "../../include/dqgemm.h"
+#include "dq_common.h"
+
+namespace dq {
+
+static char g_error_buf[kErrorBufSize];
+char* error_buf() { return g_error_buf; }
+
+// kernels (defined in the .hip files next to this one)
+int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                 int mode, int layout, int variant, hipStream_t stream);
+int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
+               hipStream_t stream);
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static int check_w4_args(const char* fn, const void* B, const void* S, const void* Z, int N, int K, int group, int mode,
+                         int layout) {
+  if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
+  if (N <= 0 || K <= 0) DQ_FAIL("%s: N and K must be positive (got N=%d K=%d)", fn, N, K);
+  if (mode < W4_UNSIGNED || mode >= W4_MODE_COUNT) DQ_FAIL("%s: unknown mode %d", fn, mode);
+  if (layout != LAYOUT_PLAIN && layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown layout %d", fn, layout);
+  if (group <= 0 || group % 32 != 0) DQ_FAIL("%s: group must be a positive multiple of 32 (got %d)", fn, group);
+  if (K % group != 0) DQ_FAIL("%s: K=%d is not a multiple of group=%d", fn, K, group);
+  if (group != K && (group & (group - 1)) != 0)
+    DQ_FAIL("%s: group=%d must be a power of two or equal to K", fn, group);
+  if (mode >= W4_SCALE && !S) DQ_FAIL("%s: Scale is expected to have non-NULL data pointer for mode %d", fn, mode);
+  if (mode >= W4_ZEROS_ORIGINAL && !Z) DQ_FAIL("%s: Zeros is expected to have non-NULL data pointer for mode %d", fn, mode);
+  if (!aligned16(B)) DQ_FAIL("%s: B must be 16-byte aligned", fn);
+  return 0;
+}
+
+}  // namespace dq
+
+using namespace dq;
+
+extern "C" const char* get_last_error(void) { return g_error_buf; }
+
+extern "C" int init(void) {
+  g_error_buf[0] = '\0';
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  hipDeviceProp_t prop;
+  DQ_CHECK_HIP(hipGetDeviceProperties(&prop, device));
+  if (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    DQ_FAIL("init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+  int max_lds = 0;
+  DQ_CHECK_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
+  const int kLargestLdsRequest = 144 * 1024;
+  if (kLargestLdsRequest > max_lds)
+    DQ_FAIL("Requested dynamic shared memory %d exceeds device limit %d", kLargestLdsRequest, max_lds);
+  return 0;
+}
+
+extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
+                                          int M, int N, int K, int group, int mode, int layout, int variant,
+                                          dq_stream_t stream) {
+  const char* fn = "call_dequantize_gemv_w4a16";
+  if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
+  if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
+  if (M <= 0) DQ_FAIL("%s: M must be positive (got %d)", fn, M);
+  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
+  if (K % 128 != 0) DQ_FAIL("%s: K=%d must be a multiple of 128", fn, K);
+  if (!aligned16(A) || !aligned16(C)) DQ_FAIL("%s: A and C must be 16-byte aligned", fn);
+  return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
+}
+
+extern "C" int call_dequantize_w4(const void* B, const void* Scale, const void* Zeros, void* W, int N, int K, int group,
+                                  int mode, int layout, dq_stream_t stream) {
+  const char* fn = "call_dequantize_w4";
+  if (!W) DQ_FAIL("%s: W is expected to have non-NULL data pointer", fn);
+  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
+  if (K % 8 != 0) DQ_FAIL("%s: K=%d must be a multiple of 8", fn, K);
+  if (!aligned16(W)) DQ_FAIL("%s: W must be 16-byte aligned", fn);
+  return w4_dequant(B, Scale, Zeros, W, N, K, group, mode, layout, (hipStream_t)stream);
+}

@@ -1,0 +1,153 @@
+// Shared device helpers for the gfx950 dequantize-GEMM kernels: vector types,
+// bit-exact weight decoders, and the host-side error buffer of the C-ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+namespace dq {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+typedef int int16_t_ __attribute__((ext_vector_type(16)));
+typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+
+// ---- host side: error reporting shared by every entry point ----------------------
+constexpr int kErrorBufSize = 1024;
+char* error_buf();  // static 1024-byte buffer, as in the reference adapter's generated host stub
+
+#define DQ_FAIL(...)                                        \
+  do {                                                      \
+    snprintf(::dq::error_buf(), ::dq::kErrorBufSize, __VA_ARGS__); \
+    return -1;                                              \
+  } while (0)
+
+#define DQ_CHECK_HIP(expr)                                                        \
+  do {                                                                            \
+    hipError_t e__ = (expr);                                                      \
+    if (e__ != hipSuccess) DQ_FAIL("%s failed: %s", #expr, hipGetErrorString(e__)); \
+  } while (0)
+
+// ---- weight formats / modes (values are part of the C-ABI, see include/dqgemm.h) --
+enum W4Mode : int {
+  W4_UNSIGNED = 0,        // w = q
+  W4_SIGNED = 1,          // w = sext4(q)  (two's complement)
+  W4_OFFSET8 = 2,         // w = q - 8
+  W4_SCALE = 3,           // w = RNE16((q - 8) * s)
+  W4_USCALE = 4,          // w = RNE16(q * s)
+  W4_ZEROS_ORIGINAL = 5,  // w = RNE16(RNE16(q - z) * s)
+  W4_ZEROS_RESCALE = 6,   // w = RNE16(fma(q, s, -z))
+  W4_MODE_COUNT = 7,
+};
+
+enum W4Layout : int {
+  LAYOUT_PLAIN = 0,        // nibble e of a 32-bit word is element e
+  LAYOUT_INTERLEAVED = 1,  // word already permuted for the fast 16-bit decoder (elements 0,2,4,6,1,3,5,7)
+};
+
+enum Fp4Format : int {
+  FP4_E2M1 = 0,       // OCP e2m1, plain low-first nibbles
+  FP4_SIMPLE = 1,     // 2^(E-1) * (1 + m/2) for every E (no zero, no subnormal)
+  FP4_TWIDDLING = 2,  // e2m1 in the 16-bit "twiddled" bit layout
+};
+
+enum I2Convention : int {
+  I2_UNSIGNED = 0,  // w = c
+  I2_OFFSET = 1,    // w = c - 2
+  I2_TWOS = 2,      // w = sext2(c)
+};
+
+// ---- device decoders ---------------------------------------------------------------
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+// One 32-bit word of eight 4-bit fields -> four half2 holding the raw integer values
+// plus a bias: out[i] = (bias_i + n_i, bias_i + n_{i+4}) where n_e is nibble e and
+// bias_0 = bias_2 = 1024, bias_1 = bias_3 = 64.  (0x6400 | n) is the fp16 1024 + n,
+// (0x5400 | n << 4) is the fp16 64 + n; both are exact.
+__device__ __forceinline__ void u4x8_to_biased_half(uint32_t w, uint32_t out[4]) {
+  // The two masks live in VGPRs (opaque to the optimiser) so that each (w & mask) | magic
+  // is a single v_and_or_b32: a VOP3 on gfx9 may read only one SGPR and no literal.
+  uint32_t mlo = 0x000F000Fu, mhi = 0x00F000F0u;
+  asm("" : "+v"(mlo));
+  asm("" : "+v"(mhi));
+  const uint32_t w2 = w >> 8;
+  out[0] = (w & mlo) | 0x64006400u;
+  out[1] = (w & mhi) | 0x54005400u;
+  out[2] = (w2 & mlo) | 0x64006400u;
+  out[3] = (w2 & mhi) | 0x54005400u;
+}
+
+// Decode one word of eight uint4 weights into fp16 with the rounding order of the
+// reference's device snippets.  Result order: element pair i is (n_i, n_{i+4}), i.e.
+// fragment element e holds nibble {0,4,1,5,2,6,3,7}[e].  For an interleaved word that
+// is the natural element order.
+template <int MODE>
+__device__ __forceinline__ half8_t decode_w4(uint32_t w, half_t s, half_t z) {
+  uint32_t t[4];
+  u4x8_to_biased_half(w, t);
+  half2_t r[4];
+  const half2_t s2 = {s, s};
+  const half2_t zero2 = {(half_t)0.f, (half_t)0.f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const half_t bias = (i & 1) ? (half_t)64.f : (half_t)1024.f;
+    half2_t x = as_half2(t[i]);
+    if constexpr (MODE == W4_UNSIGNED) {
+      const half2_t b2 = {bias, bias};
+      r[i] = x - b2;
+    } else if constexpr (MODE == W4_SIGNED) {
+      // sext4(q) = ((q ^ 8) - 8): flip bit 3 of the nibble inside the mantissa, then
+      // subtract bias + 8; all steps exact.
+      const uint32_t flip = (i & 1) ? 0x00800080u : 0x00080008u;
+      x = as_half2(t[i] ^ flip);
+      const half2_t b2 = {(half_t)(bias + (half_t)8.f), (half_t)(bias + (half_t)8.f)};
+      r[i] = x - b2;
+    } else if constexpr (MODE == W4_OFFSET8) {
+      const half2_t b2 = {(half_t)(bias + (half_t)8.f), (half_t)(bias + (half_t)8.f)};
+      r[i] = x - b2;
+    } else if constexpr (MODE == W4_SCALE) {
+      const half2_t b2 = {(half_t)(bias + (half_t)8.f), (half_t)(bias + (half_t)8.f)};
+      r[i] = __builtin_elementwise_fma(x - b2, s2, zero2);
+    } else if constexpr (MODE == W4_USCALE) {
+      const half2_t b2 = {bias, bias};
+      r[i] = __builtin_elementwise_fma(x - b2, s2, zero2);
+    } else if constexpr (MODE == W4_ZEROS_ORIGINAL) {
+      const half2_t b2 = {bias, bias};
+      const half2_t z2 = {z, z};
+      r[i] = __builtin_elementwise_fma((x - b2) - z2, s2, zero2);
+    } else {  // W4_ZEROS_RESCALE
+      const half2_t b2 = {bias, bias};
+      const half2_t nz2 = {(half_t)(-z), (half_t)(-z)};
+      r[i] = __builtin_elementwise_fma(x - b2, s2, nz2);
+    }
+  }
+  half8_t o;
+  o[0] = r[0][0]; o[1] = r[0][1]; o[2] = r[1][0]; o[3] = r[1][1];
+  o[4] = r[2][0]; o[5] = r[2][1]; o[6] = r[3][0]; o[7] = r[3][1];
+  return o;
+}
+
+// Permute eight consecutive 16-bit activations a0..a7 (two per register) into the
+// order the plain-layout decoder produces: (a0,a4) (a1,a5) (a2,a6) (a3,a7).
+__device__ __forceinline__ uint4_t permute_k8_16bit(uint4_t d) {
+  uint4_t o;
+  // __builtin_amdgcn_perm(hi_src, lo_src, sel): byte i of the result is byte sel[i] of {hi_src:lo_src}
+  o[0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100u);  // (d0.lo, d2.lo)
+  o[1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302u);  // (d0.hi, d2.hi)
+  o[2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100u);  // (d1.lo, d3.lo)
+  o[3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302u);  // (d1.hi, d3.hi)
+  return o;
+}
+
+}  // namespace dq

@@ -1,0 +1,173 @@
+"""Kernel factories with the call surface of the reference's examples.
+
+Each factory takes the example's arguments (shapes, dtype names, decode options) and
+returns a :class:`~tilelang_amd.adapter.KernelAdapter` whose call signature is the
+example kernel's: ``kernel(A, B_packed[, Scale[, Zeros]], C)`` on torch device tensors.
+Nothing is compiled at call time: every factory binds an ahead-of-time entry point of
+``libdqgemm.so``.  Tile-size / thread / stage arguments of the examples are accepted and
+ignored (the kernels carry their own gfx950 tiling).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .adapter import KernelAdapter, KernelParam
+
+# ---- enums of include/dqgemm.h -------------------------------------------------------------
+W4_UNSIGNED, W4_SIGNED, W4_OFFSET8, W4_SCALE, W4_USCALE, W4_ZEROS_ORIGINAL, W4_ZEROS_RESCALE = range(7)
+LAYOUT_PLAIN, LAYOUT_INTERLEAVED = 0, 1
+
+_DTYPES = {
+    "float16": torch.float16,
+    "bfloat16": torch.bfloat16,
+    "float32": torch.float32,
+    "int8": torch.int8,
+    "uint8": torch.uint8,
+    "int32": torch.int32,
+}
+
+
+def _dtype(d) -> torch.dtype:
+    if isinstance(d, torch.dtype):
+        return d
+    try:
+        return _DTYPES[str(d)]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {d!r}") from None
+
+
+def _w4_mode(source_format: str, fast_decoding: bool, with_scaling: bool, with_zeros: bool, zeros_mode: str) -> int:
+    if with_zeros:
+        if not with_scaling:
+            raise ValueError("with_zeros requires with_scaling")
+        if zeros_mode in ("original", "quantized"):
+            # "quantized" zeros are integers: (q - qz) is exact either way
+            return W4_ZEROS_ORIGINAL
+        if zeros_mode == "rescale":
+            return W4_ZEROS_RESCALE
+        raise ValueError(f"unknown zeros_mode {zeros_mode!r}")
+    if with_scaling:
+        return W4_SCALE if source_format == "int" else W4_USCALE
+    if fast_decoding:
+        return W4_OFFSET8 if source_format == "int" else W4_UNSIGNED
+    # the example's slow path sign-extends the nibble whatever source_format says
+    # (examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124)
+    return W4_SIGNED
+
+
+def dequantize_gemv(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="float16",
+    out_dtype="float16",
+    accum_dtype="float32",
+    num_bits: int = 4,
+    storage_dtype="int8",
+    source_format: str = "uint",
+    n_partition: int = 4,
+    reduce_thread: int = 32,
+    fast_decoding: bool = False,
+    trans_A: bool = False,
+    trans_B: bool = True,
+    group_size: int = -1,
+    with_scaling: bool = False,
+    with_zeros: bool = False,
+    zeros_mode: str = "original",
+    variant: int = -1,
+    _formula_fast: bool | None = None,
+) -> KernelAdapter:
+    """W4A16 decode GEMV / small-batch GEMM: ``C[M,N] = A[M,K] @ dequant(B[N,K/2]).T``.
+
+    Same positional arguments as ``dequantize_gemv`` of
+    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:11-29.  Call surface:
+    ``kernel(A, B, C)``; with ``with_scaling`` ``kernel(A, B, Scale, C)``; with
+    ``with_zeros`` ``kernel(A, B, Scale, Zeros, C)``, ``Scale``/``Zeros`` fp16
+    ``[N, K // group_size]``.
+
+    ``fast_decoding=True`` means, as in the example, that B was passed through
+    ``interleave_weight(B, 4, "float16")``; otherwise B is the plain low-nibble-first
+    layout.  Accumulation is always fp32.  ``source_format="int"`` with scaling is the
+    zero-point-8 decode ``w = (q - 8) * s``.
+    """
+    assert trans_A is False, "Dequantize only implement for trans_A=False currently"
+    assert trans_B is True, "Dequantize only implement for trans_B=TRue currently"
+    if num_bits != 4:
+        raise ValueError("dequantize_gemv: only num_bits=4 is built")
+    if _dtype(in_dtype) != torch.float16 or _dtype(out_dtype) != torch.float16:
+        raise ValueError("dequantize_gemv: in_dtype and out_dtype must be float16 (int8 x int2: bitnet_158_int8xint2_decode)")
+    if _dtype(storage_dtype) not in (torch.int8, torch.uint8):
+        raise ValueError("dequantize_gemv: storage_dtype must be int8 or uint8")
+    if group_size == -1:
+        group_size = K
+    if K % 128 != 0:
+        raise ValueError(f"dequantize_gemv: K={K} must be a multiple of 128")
+    if K % group_size != 0 or group_size % 32 != 0:
+        raise ValueError(f"dequantize_gemv: group_size={group_size} must divide K={K} and be a multiple of 32")
+    # _formula_fast (tests): pick the decode formula of the fast / slow path independently of the layout
+    formula_fast = fast_decoding if _formula_fast is None else _formula_fast
+    mode = _w4_mode(source_format, formula_fast, with_scaling, with_zeros, zeros_mode)
+    layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
+    groups = K // group_size
+
+    params = [
+        KernelParam("A", torch.float16, (M, K)),
+        KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True),
+    ]
+    if with_scaling:
+        params.append(KernelParam("Scale", torch.float16, (N, groups)))
+    if with_zeros:
+        params.append(KernelParam("Zeros", torch.float16, (N, groups)))
+    params.append(KernelParam("C", torch.float16, (M, N)))
+
+    def launch(ptrs, stream):
+        lib = _lib.get_library()
+        a, b = ptrs[0], ptrs[1]
+        s = ptrs[2] if with_scaling else None
+        z = ptrs[3] if with_zeros else None
+        c = ptrs[-1]
+        return lib.call_dequantize_gemv_w4a16(a, b, s, z, c, M, N, K, group_size, mode, layout, variant, stream)
+
+    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
+
+
+def dequantize_w4(
+    N: int,
+    K: int,
+    group_size: int = -1,
+    source_format: str = "int",
+    fast_decoding: bool = False,
+    with_scaling: bool = True,
+    with_zeros: bool = False,
+    zeros_mode: str = "original",
+    storage_dtype="int8",
+    _formula_fast: bool | None = None,
+) -> KernelAdapter:
+    """Dequantised weight tile ``W[N,K] fp16 = decode(B[N,K/2][, Scale[, Zeros]])``.
+
+    The decode-only kernel the examples use to test a converter
+    (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:36-65), here for the 4-bit
+    integer decoders.  ``W = kernel(B[, Scale[, Zeros]])``.
+    """
+    if group_size == -1:
+        group_size = K
+    formula_fast = fast_decoding if _formula_fast is None else _formula_fast
+    mode = _w4_mode(source_format, formula_fast, with_scaling, with_zeros, zeros_mode)
+    layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
+    groups = K // group_size
+    params = [KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True)]
+    if with_scaling:
+        params.append(KernelParam("Scale", torch.float16, (N, groups)))
+    if with_zeros:
+        params.append(KernelParam("Zeros", torch.float16, (N, groups)))
+    params.append(KernelParam("W", torch.float16, (N, K)))
+
+    def launch(ptrs, stream):
+        lib = _lib.get_library()
+        s = ptrs[1] if with_scaling else None
+        z = ptrs[2] if with_zeros else None
+        return lib.call_dequantize_w4(ptrs[0], s, z, ptrs[-1], N, K, group_size, mode, layout, stream)
+
+    return KernelAdapter("dequantize_w4", params, [-1], launch, _lib.last_error)

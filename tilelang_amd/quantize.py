@@ -1,0 +1,114 @@
+"""Host-side weight packing and layout helpers (one-off, torch ops, any device).
+
+Same names and argument meaning as the helpers the reference's examples import:
+``general_compress`` / ``interleave_weight`` (examples/dequantize_gemm/quantize/utils.py:50-125),
+``pack_int4`` (examples/gemm_int4/example_tilelang_gemm_int4.py:59-67), and the e2m1
+helpers of examples/dequantize_gemm/quantize/nvfp4.py:120-177.
+"""
+
+from __future__ import annotations
+
+import torch
+
+FP4_E2M1_VALUES = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0)
+
+
+def general_compress(lowprecision_weight: torch.Tensor, source_bits: int = 4, storage_dtype=None) -> torch.Tensor:
+    """Pack ``8 // source_bits`` fields per byte, field ``k`` of a byte at bit ``source_bits * k``."""
+    if storage_dtype is None:
+        storage_dtype = torch.int8
+    epb = 8 // source_bits
+    w = lowprecision_weight
+    if w.dtype == torch.float16:
+        w = w.to(torch.int8)
+    if w.shape[-1] % epb:
+        raise ValueError(f"last dimension {w.shape[-1]} is not a multiple of {epb}")
+    fields = w.to(torch.int32).reshape(*w.shape[:-1], w.shape[-1] // epb, epb)
+    packed = torch.zeros(fields.shape[:-1], dtype=torch.int32, device=w.device)
+    for k in range(epb):  # OR without masking the field, as the reference does for signed inputs
+        packed |= (fields[..., k] << (source_bits * k)) & 0xFF
+    return packed.to(torch.uint8).view(torch.int8).to(storage_dtype)
+
+
+def interleave_weight(qweight: torch.Tensor, nbits: int = 4, target_dtype: str = "float16") -> torch.Tensor:
+    """Permute every 32-bit word so the fast 16-bit / 8-bit decoders emit natural element order.
+
+    Element ``e`` of a word moves to bit ``(e % G) * stride + (e // G) * nbits`` (stride 16, G 2 for a
+    float16 target; stride 8, G 4 for int8), plus the extra byte shuffles of the 1-bit and
+    (2-bit, float16) cases.
+    """
+    if target_dtype not in ("float16", "int8"):
+        raise ValueError(target_dtype)
+    orig_shape, orig_dtype = qweight.shape, qweight.dtype
+    q = qweight.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    stride = 8 if target_dtype == "int8" else 16
+    groups = 32 // stride
+    mask = (1 << nbits) - 1
+    out = torch.zeros_like(q)
+    for e in range(32 // nbits):
+        dst = (e % groups) * stride + (e // groups) * nbits
+        out |= ((q >> (nbits * e)) & mask) << dst
+
+    def move(x, src_mask, right, left):
+        return ((x & src_mask) >> right) << left
+
+    if nbits == 1 and target_dtype == "int8":
+        out = (out & 0xF0F00F0F) | move(out, 0x000000F0, 4, 16) | move(out, 0x0000F000, 12, 24) \
+            | move(out, 0x000F0000, 16, 4) | move(out, 0x0F000000, 24, 12)
+    elif nbits == 2 and target_dtype == "float16":
+        out = (out & 0xFF0000FF) | move(out, 0x0000FF00, 8, 16) | move(out, 0x00FF0000, 16, 8)
+    elif nbits == 1 and target_dtype == "float16":
+        out = (out & 0xF000000F) | move(out, 0x000000F0, 4, 8) | move(out, 0x00000F00, 8, 16) \
+            | move(out, 0x0000F000, 12, 24) | move(out, 0x000F0000, 16, 4) | move(out, 0x00F00000, 20, 12) \
+            | move(out, 0x0F000000, 24, 20)
+    out = out & 0xFFFFFFFF
+    out = torch.where(out >= 2**31, out - 2**32, out).to(torch.int32)
+    return out.view(orig_dtype).reshape(orig_shape)
+
+
+def pack_int4(tensor: torch.Tensor) -> torch.Tensor:
+    """Logical signed int4 held in int8 -> two per byte, even index in the low nibble."""
+    if tensor.dtype != torch.int8:
+        raise TypeError(f"Expected torch.int8 logical int4 tensor, but got {tensor.dtype}.")
+    if tensor.ndim == 0 or tensor.shape[-1] % 2 != 0:
+        raise ValueError("The last dimension of a logical int4 tensor must be even for int8 packing.")
+    t = tensor.to(torch.int16)
+    return ((t[..., ::2] & 0x0F) | ((t[..., 1::2] & 0x0F) << 4)).to(torch.uint8).view(torch.int8).contiguous()
+
+
+def encode_fp4_e2m1_values(values: torch.Tensor) -> torch.Tensor:
+    """float -> raw e2m1 nibble codes (uint8)."""
+    if not isinstance(values, torch.Tensor):
+        raise TypeError(f"values must be a torch.Tensor, got {type(values)!r}")
+    x = torch.nan_to_num(values.to(torch.float32), nan=0.0, posinf=6.0, neginf=-6.0)
+    bounds = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], device=x.device)
+    mag = torch.bucketize(x.abs(), bounds, right=True).to(torch.int32)
+    sign = ((x < 0) & (mag != 0)).to(torch.int32) << 3
+    return (mag | sign).to(torch.uint8)
+
+
+def pack_fp4_e2m1_codes(codes: torch.Tensor) -> torch.Tensor:
+    """e2m1 codes [N, K] uint8 -> int8 storage [N, K/2], low nibble first."""
+    if not isinstance(codes, torch.Tensor):
+        raise TypeError(f"codes must be a torch.Tensor, got {type(codes)!r}")
+    if codes.dtype != torch.uint8:
+        raise TypeError(f"codes must have dtype torch.uint8, got {codes.dtype}")
+    if codes.ndim != 2:
+        raise ValueError(f"codes must be a 2D tensor, got shape {tuple(codes.shape)}")
+    if codes.shape[1] % 2 != 0:
+        raise ValueError(f"FP4 packing requires an even K dimension, got {tuple(codes.shape)}")
+    return ((codes[:, 0::2] & 0x0F) | ((codes[:, 1::2] & 0x0F) << 4)).contiguous().view(torch.int8)
+
+
+def decode_packed_fp4_e2m1(packed: torch.Tensor, cols: int | None = None) -> torch.Tensor:
+    """Packed e2m1 -> float32 values."""
+    if packed.ndim != 2:
+        raise ValueError(f"packed must be a 2D tensor, got shape {tuple(packed.shape)}")
+    if cols is None:
+        cols = packed.shape[1] * 2
+    if cols != packed.shape[1] * 2:
+        raise ValueError(f"cols must equal packed.shape[1] * 2, got cols={cols}, packed shape={tuple(packed.shape)}")
+    u = packed.contiguous().view(torch.uint8)
+    lut = torch.tensor(FP4_E2M1_VALUES, device=packed.device, dtype=torch.float32)
+    nib = torch.stack((u & 0x0F, u >> 4), dim=-1).reshape(packed.shape[0], cols)
+    return lut[nib.long()]
