@@ -17,6 +17,8 @@ int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, voi
                  int mode, int layout, int variant, hipStream_t stream);
 int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
                hipStream_t stream);
+int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                    int mode, int layout, int rows_hint, hipStream_t stream);
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -68,6 +70,14 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
   if (K % 128 != 0) DQ_FAIL("%s: K=%d must be a multiple of 128", fn, K);
   if (!aligned16(A) || !aligned16(C)) DQ_FAIL("%s: A and C must be 16-byte aligned", fn);
+  // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread
+  // (r = 0: its own choice).  0..99: a configuration of the MFMA kernel.
+  if (variant < 0 || variant >= 100) {
+    const int rc = w4a16_gemv_dot2(A, B, Scale, Zeros, C, M, N, K, group, mode, layout,
+                                   variant >= 100 ? variant - 100 : 0, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+    if (variant >= 100) DQ_FAIL("%s: the dot2 GEMV kernel does not cover M=%d K=%d", fn, M, K);
+  }
   return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
 }
 

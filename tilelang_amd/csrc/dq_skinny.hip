@@ -44,7 +44,10 @@ __device__ __forceinline__ void stage_a_tile(const half_t* __restrict__ A, half_
   }
 }
 
-template <int MB, int RB, int WAVES, int U, int MODE, bool APERM>
+// Workgroup = WAVES waves sharing RB row blocks of 16 weight rows; the 128-k chunks of every K
+// tile are split evenly between the waves (split-K inside the workgroup), partial 16x16 tiles are
+// summed through LDS in a fixed order at the end.  G128: group size 128 (one scale per chunk).
+template <int MB, int RB, int WAVES, int U, int MODE, bool APERM, bool G128>
 __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* __restrict__ A,
                                                                    const uint8_t* __restrict__ B,
                                                                    const half_t* __restrict__ S,
@@ -55,6 +58,8 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* 
   half_t* lds = reinterpret_cast<half_t*>(smem_raw);
 
   constexpr int THREADS = WAVES * 64;
+  constexpr bool kScale = ModeTraits<MODE>::kHasScale;
+  constexpr bool kZeros = ModeTraits<MODE>::kHasZeros;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -63,8 +68,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* 
 
   const int m0 = blockIdx.y * (16 * MB);
   const int mrows = min(M - m0, 16 * MB);
-  const int n_wg0 = blockIdx.x * (WAVES * RB * 16);
-  const int n_wave0 = n_wg0 + wave * (RB * 16);
+  const int n0 = blockIdx.x * (RB * 16);
 
   const int lds_stride = KT + 8;
   const int groups_per_row = K / group;
@@ -78,10 +82,10 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* 
   const half_t* zrow[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const int row = min(n_wave0 + rb * 16 + r, N - 1);
+    const int row = min(n0 + rb * 16 + r, N - 1);
     brow[rb] = B + (size_t)row * row_bytes + g * 16;
-    srow[rb] = ModeTraits<MODE>::kHasScale ? S + (size_t)row * groups_per_row : nullptr;
-    zrow[rb] = ModeTraits<MODE>::kHasZeros ? Z + (size_t)row * groups_per_row : nullptr;
+    srow[rb] = kScale ? S + (size_t)row * groups_per_row : nullptr;
+    zrow[rb] = kZeros ? Z + (size_t)row * groups_per_row : nullptr;
   }
 
   float4_t acc[RB][MB];
@@ -90,7 +94,6 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  const bool wave_active = n_wave0 < N;  // wave-uniform
   int a_row_off[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) a_row_off[mb] = min(mb * 16 + r, mrows - 1) * lds_stride;
@@ -101,80 +104,118 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* 
     stage_a_tile<THREADS, APERM>(A, lds, mrows, m0, k0, kt, K, lds_stride, tid);
     __syncthreads();
 
-    if (wave_active) {
-      const int nch = kt / kChunkK;
-      // Two register sets: the loads of batch b+1 are in flight while batch b is decoded
-      // and multiplied.
-      uint4_t bq0[RB][U], bq1[RB][U];
-      half_t sc0[RB][U], sc1[RB][U], zp0[RB][U], zp1[RB][U];
-      auto load_set = [&](uint4_t (&bq)[RB][U], half_t (&sc)[RB][U], half_t (&zp)[RB][U], int c) {
+    const int nch = kt / kChunkK;
+    const int cpw = (nch + WAVES - 1) / WAVES;
+    const int c_begin = wave * cpw;
+    const int c_end = min(nch, c_begin + cpw);
+
+    // Two register sets: the loads of batch b+1 are in flight while batch b is decoded and
+    // multiplied.  All offsets inside a batch are compile-time constants.
+    uint4_t bq0[RB][U], bq1[RB][U];
+    half_t sc0[RB][U], sc1[RB][U], zp0[RB][U], zp1[RB][U];
+    auto load_set = [&](uint4_t (&bq)[RB][U], half_t (&sc)[RB][U], half_t (&zp)[RB][U], int c) {
+      const int nvalid = c_end - c;  // wave-uniform
+      const int kk = k0 + c * kChunkK;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int cc = min(c + u, nch - 1);  // clamped: stays in bounds, unused past nch
-          const int kk = k0 + cc * kChunkK;
-          const int gi = (kk + g * 32) >> gshift;
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb) {
-            bq[rb][u] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(brow[rb] + (kk >> 1)));
-            if constexpr (ModeTraits<MODE>::kHasScale) sc[rb][u] = srow[rb][gi];
-            else sc[rb][u] = (half_t)1.f;
-            if constexpr (ModeTraits<MODE>::kHasZeros) zp[rb][u] = zrow[rb][gi];
-            else zp[rb][u] = (half_t)0.f;
-          }
+      for (int rb = 0; rb < RB; ++rb) {
+        const uint8_t* bp = brow[rb] + (kk >> 1);
+        const half_t* sp = nullptr;
+        const half_t* zp_ = nullptr;
+        if constexpr (G128) {
+          if constexpr (kScale) sp = srow[rb] + (kk >> 7);
+          if constexpr (kZeros) zp_ = zrow[rb] + (kk >> 7);
         }
-      };
-      auto compute_set = [&](uint4_t (&bq)[RB][U], half_t (&sc)[RB][U], half_t (&zp)[RB][U], int c) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          if (c + u < nch) {  // wave-uniform
-            const half_t* a_chunk = lds + (c + u) * kChunkK + g * 32;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              // Lanes whose activation row is past M re-read the last valid row: column m of
-              // the 32x16 operand only feeds output column m, which is never stored.
-              half8_t y[MB];
-#pragma unroll
-              for (int mb = 0; mb < MB; ++mb)
-                y[mb] = *reinterpret_cast<const half8_t*>(a_chunk + a_row_off[mb] + j * 8);
-#pragma unroll
-              for (int rb = 0; rb < RB; ++rb) {
-                const half8_t x = decode_w4<MODE>(bq[rb][u][j], sc[rb][u], zp[rb][u]);
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                  acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y[mb], acc[rb][mb], 0, 0, 0);
-              }
+          if (u < nvalid) {
+            bq[rb][u] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(bp + u * (kChunkK / 2)));
+            if constexpr (G128) {
+              if constexpr (kScale) sc[rb][u] = sp[u];
+              if constexpr (kZeros) zp[rb][u] = zp_[u];
+            } else {
+              const int gi = (kk + u * kChunkK + g * 32) >> gshift;
+              if constexpr (kScale) sc[rb][u] = srow[rb][gi];
+              if constexpr (kZeros) zp[rb][u] = zrow[rb][gi];
             }
           }
         }
-      };
-      load_set(bq0, sc0, zp0, 0);
-      for (int c = 0; c < nch; c += 2 * U) {
-        if (c + U < nch) load_set(bq1, sc1, zp1, c + U);
+      }
+    };
+    auto compute_set = [&](uint4_t (&bq)[RB][U], half_t (&sc)[RB][U], half_t (&zp)[RB][U], int c) {
+      const int nvalid = c_end - c;
+      const half_t* a_base = lds + c * kChunkK + g * 32;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (u < nvalid) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            // Lanes whose activation row is past M re-read the last valid row: column m of the
+            // 32x16 operand only feeds output column m, which is never stored.
+            half8_t y[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+              y[mb] = *reinterpret_cast<const half8_t*>(a_base + a_row_off[mb] + u * kChunkK + j * 8);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+              const half8_t x = decode_w4<MODE>(bq[rb][u][j], kScale ? sc[rb][u] : (half_t)1.f,
+                                                kZeros ? zp[rb][u] : (half_t)0.f);
+#pragma unroll
+              for (int mb = 0; mb < MB; ++mb)
+                acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y[mb], acc[rb][mb], 0, 0, 0);
+            }
+          }
+        }
+      }
+    };
+    if (c_begin < c_end) {
+      load_set(bq0, sc0, zp0, c_begin);
+      for (int c = c_begin; c < c_end; c += 2 * U) {
+        if (c + U < c_end) load_set(bq1, sc1, zp1, c + U);
         compute_set(bq0, sc0, zp0, c);
-        if (c + 2 * U < nch) load_set(bq0, sc0, zp0, c + 2 * U);
-        if (c + U < nch) compute_set(bq1, sc1, zp1, c + U);
+        if (c + 2 * U < c_end) load_set(bq0, sc0, zp0, c + 2 * U);
+        if (c + U < c_end) compute_set(bq1, sc1, zp1, c + U);
       }
     }
   }
 
-  if (!wave_active) return;
-  // acc[rb][mb][i] = C[m0 + mb*16 + r][n_wave0 + rb*16 + g*4 + i]
+  // Cross-wave reduction in a fixed order (deterministic), then the fp16 store.
+  // acc[rb][mb][i] = partial C[m0 + mb*16 + r][n0 + rb*16 + g*4 + i]
+  float4_t* red = reinterpret_cast<float4_t*>(smem_raw);
+  if constexpr (WAVES > 1) {
+    __syncthreads();  // every wave is done reading activations from LDS
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) red[((rb * MB + mb) * WAVES + wave) * 64 + lane] = acc[rb][mb];
+    __syncthreads();
+  }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
+      constexpr int kPairs = RB * MB;
+      const int pair = rb * MB + mb;
+      float4_t v = acc[rb][mb];
+      if constexpr (WAVES > 1) {
+        // output tile `pair` is finished by wave pair % WAVES
+        if ((pair % WAVES) != wave && kPairs > 1) continue;
+        if (kPairs == 1 && wave != 0) continue;
+        v = red[(pair * WAVES + 0) * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) v += red[(pair * WAVES + w) * 64 + lane];
+      }
       const int m = mb * 16 + r;
-      if (m >= mrows) continue;
-      const int n = n_wave0 + rb * 16 + g * 4;
+      const int n = n0 + rb * 16 + g * 4;
+      if (m >= mrows || n >= N) continue;
       half_t* dst = C + (size_t)(m0 + m) * N + n;
       if (((N & 3) == 0) && n + 3 < N) {
         typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-        half4_t o = {(half_t)acc[rb][mb][0], (half_t)acc[rb][mb][1], (half_t)acc[rb][mb][2], (half_t)acc[rb][mb][3]};
+        half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
         *reinterpret_cast<half4_t*>(dst) = o;
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (n + i < N) dst[i] = (half_t)acc[rb][mb][i];
+          if (n + i < N) dst[i] = (half_t)v[i];
       }
     }
   }
@@ -208,26 +249,29 @@ __global__ void w4_dequant_kernel(const uint8_t* __restrict__ B, const half_t* _
   }
 }
 
-struct SkinnyPlan {
-  int mb, rb, waves, u, kt;
-  size_t lds_bytes;
-};
-
 template <int MB, int RB, int WAVES, int U, bool ALL_MODES>
 int launch_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                   int mode, int layout, int KT, hipStream_t stream) {
-  const dim3 grid((N + WAVES * RB * 16 - 1) / (WAVES * RB * 16), (M + 16 * MB - 1) / (16 * MB));
+  const dim3 grid((N + RB * 16 - 1) / (RB * 16), (M + 16 * MB - 1) / (16 * MB));
   const dim3 block(WAVES * 64);
   const int mrows = M < 16 * MB ? M : 16 * MB;
-  const size_t lds_bytes = (size_t)mrows * (KT + 8) * sizeof(half_t);
-#define DQ_LAUNCH(MODE_, APERM_)                                                                                     \
+  size_t lds_bytes = (size_t)mrows * (KT + 8) * sizeof(half_t);
+  const size_t red_bytes = WAVES > 1 ? (size_t)RB * MB * WAVES * 64 * sizeof(float4_t) : 0;
+  if (red_bytes > lds_bytes) lds_bytes = red_bytes;
+  const bool g128 = group == 128;
+#define DQ_LAUNCH2(MODE_, APERM_, G128_)                                                                             \
   do {                                                                                                               \
-    auto kern = w4a16_skinny_kernel<MB, RB, WAVES, U, MODE_, APERM_>;                                                \
+    auto kern = w4a16_skinny_kernel<MB, RB, WAVES, U, MODE_, APERM_, G128_>;                                         \
     if (lds_bytes > 48 * 1024)                                                                                       \
       DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                          \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));                 \
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,  \
                        (const half_t*)Z, (half_t*)C, M, N, K, group, KT);                                            \
+  } while (0)
+#define DQ_LAUNCH(MODE_, APERM_)                  \
+  do {                                            \
+    if (g128) DQ_LAUNCH2(MODE_, APERM_, true);    \
+    else DQ_LAUNCH2(MODE_, APERM_, false);        \
   } while (0)
 #define DQ_LAUNCH_MODE(MODE_)                 \
   do {                                        \
@@ -256,18 +300,23 @@ int launch_skinny(const void* A, const void* B, const void* S, const void* Z, vo
   }
 #undef DQ_LAUNCH_MODE
 #undef DQ_LAUNCH
+#undef DQ_LAUNCH2
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }
 
 }  // namespace
 
-// Largest K tile (multiple of 128) whose staged activations fit the LDS budget.
+// K tile (multiple of 128) for staging `mrows` activation rows in LDS: the fewest equal tiles
+// that fit the budget.
 static int pick_kt(int mrows, int K, size_t lds_budget) {
-  long kt = (long)(lds_budget / (mrows * sizeof(half_t))) - 8;
-  kt = (kt / kChunkK) * kChunkK;
-  if (kt > K) kt = K;
-  if (kt < kChunkK) kt = kChunkK;
+  long kt_max = (long)(lds_budget / (mrows * sizeof(half_t))) - 8;
+  kt_max = (kt_max / kChunkK) * kChunkK;
+  if (kt_max < kChunkK) kt_max = kChunkK;
+  if (kt_max >= K) return K;
+  const long tiles = (K + kt_max - 1) / kt_max;
+  long kt = (K + tiles - 1) / tiles;
+  kt = ((kt + kChunkK - 1) / kChunkK) * kChunkK;
   return (int)kt;
 }
 
@@ -275,20 +324,31 @@ int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, voi
                  int mode, int layout, int variant, hipStream_t stream) {
   // variant < 0: heuristic.  Otherwise an explicit (benchmarking) choice, see switch below.
   if (variant < 0) {
-    if (M <= 16) variant = (N >= 8192) ? 0 : 1;
+    if (M <= 16) variant = 0;
     else if (M <= 32) variant = 4;
     else variant = 5;
   }
-  const size_t budget = 64 * 1024;
+  const size_t budget = 72 * 1024;
   switch (variant) {
-    case 0: return launch_skinny<1, 1, 4, 8, true>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 16 ? M : 16, K, budget), stream);
-    case 1: return launch_skinny<1, 1, 1, 8, true>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 16 ? M : 16, K, budget), stream);
-    case 2: return launch_skinny<1, 1, 2, 8, false>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 16 ? M : 16, K, budget), stream);
-    case 3: return launch_skinny<1, 2, 4, 4, false>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 16 ? M : 16, K, budget), stream);
-    case 4: return launch_skinny<2, 2, 4, 4, true>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 32 ? M : 32, K, budget), stream);
-    case 5: return launch_skinny<4, 4, 4, 2, true>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 64 ? M : 64, K, budget), stream);
-    case 6: return launch_skinny<1, 1, 4, 4, false>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 16 ? M : 16, K, budget), stream);
-    case 7: return launch_skinny<1, 1, 8, 8, false>(A, B, S, Z, C, M, N, K, group, mode, layout, pick_kt(M < 16 ? M : 16, K, budget), stream);
+#define DQ_V(ID, MB_, RB_, W_, U_, ALL_)                                                                  \
+  case ID:                                                                                                \
+    return launch_skinny<MB_, RB_, W_, U_, ALL_>(A, B, S, Z, C, M, N, K, group, mode, layout,             \
+                                                 pick_kt(M < 16 * MB_ ? M : 16 * MB_, K, budget), stream)
+    //   id  MB RB  W  U  all-modes
+    DQ_V(0, 1, 1, 4, 8, true);
+    DQ_V(1, 1, 1, 1, 8, false);
+    DQ_V(2, 1, 1, 2, 8, false);
+    DQ_V(3, 1, 2, 4, 4, false);
+    DQ_V(4, 2, 2, 4, 4, true);
+    DQ_V(5, 4, 4, 4, 2, true);
+    DQ_V(6, 1, 1, 4, 4, false);
+    DQ_V(7, 1, 1, 8, 8, false);
+    DQ_V(8, 1, 1, 8, 4, false);
+    DQ_V(9, 1, 2, 8, 4, false);
+    DQ_V(10, 1, 4, 4, 2, false);
+    DQ_V(11, 1, 1, 16, 4, false);
+    DQ_V(12, 1, 1, 8, 2, false);
+#undef DQ_V
     default: DQ_FAIL("w4a16: unknown kernel variant %d", variant);
   }
 }
