@@ -69,6 +69,24 @@ int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, 
 int call_dequantize_w4(const void* B, const void* Scale, const void* Zeros, void* W, int N, int K, int group,
                        int mode, int layout, dq_stream_t stream);
 
+/* ---- MXFP4 x bf16 ------------------------------------------------------------------------ */
+
+enum dq_fp4_format {
+  DQ_FP4_E2M1 = 0,     /* OCP e2m1, plain low-first nibbles: examples/dequantize_gemm/quantize/nvfp4.py:17-34,
+                          quantize/mxfp.py:136-157, src/tl_templates/hip/hip_fp4.h:18-57                         */
+  DQ_FP4_SIMPLE = 1,   /* bf16 bits (s<<15)|((E+126)<<7)|(m<<6) for every E: examples/dequantize_gemm/
+                          dequantize_utils.py:57-84, example_dequant_gemm_bf16_mxfp4_cdna4.py:26-41             */
+  DQ_FP4_TWIDDLING = 2 /* e2m1 in the 16-bit twiddled layout: dequantize_utils.py:4-54, quantize/mxfp.py:67-131  */
+};
+
+/* C[M,N] bf16 = A[M,K] bf16 . (fp4(B[N,K/2]) * 2^(Scale[N,K/32] - scale_bias))^T (+ Bias[M,N] bf16),
+ * fp32 accumulation.  Replaces `call(A, B, Scale, Bias, C, stream)` of the kernel generated from
+ * examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:201-244.  The reference
+ * multiplies by 2^Scale with the raw byte (:254-267): scale_bias = 0; an E8M0 scale is
+ * scale_bias = 127.  Bias may be NULL.  Requires K % 64 == 0, scale_size == 32. */
+int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale, const void* Bias, void* C, int M,
+                                 int N, int K, int scale_size, int fp4_format, int scale_bias, dq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

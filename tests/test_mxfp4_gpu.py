@@ -1,0 +1,113 @@
+"""GPU parity of the MXFP4 x bf16 GEMM (through the C-ABI) against the CPU oracle.
+
+bf16 outputs within rtol=1e-2, atol=1e-2 of ``A.float() @ (decode(B) * 2**(Scale - bias)).float().T -> bf16``
+(the dequantised operand is exact in bf16, the only rounding is the fp32 accumulation and the final cast).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from tilelang_amd import workloads
+from oracle import dq_oracle as orc
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def _dev(x, cuda):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(cuda)
+
+
+def _check(cuda, M, N, K, fmt, scale_bias, seed=0, with_bias=False, exp_range=(-8, 0)):
+    d = workloads.mxfp4(M, N, K, seed=seed, scale_exp_range=exp_range, scale_bias=scale_bias)
+    B = d["B"]
+    if fmt == "twiddling":
+        B = orc.twiddle_pack_fp4(orc.unpack_u4(B))
+    kern = tl.matmul_bf16_mxfp4(M, N, K, weight_format=fmt, scale_bias=scale_bias, with_bias=with_bias)
+    A = _dev(d["A"], cuda).view(torch.bfloat16)
+    rng = np.random.default_rng(seed + 1)
+    bias_bits = orc.f32_to_bf16_bits(rng.standard_normal((M, N), dtype=np.float32) * 4)
+    Bias = _dev(bias_bits, cuda).view(torch.bfloat16)
+    C = kern(A, _dev(B, cuda), _dev(d["Scale"], cuda), Bias)
+    torch.cuda.synchronize()
+    ref_bits = orc.ref_mxfp4(d["A"], B, d["Scale"], bias_bits if with_bias else None, fmt=fmt, scale_bias=scale_bias)
+    ref = orc.bf16_bits_to_f32(ref_bits)
+    got = C.float().cpu().numpy()
+    assert got.shape == (M, N) and np.isfinite(got).all()
+    np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
+    return got
+
+
+@pytest.mark.parametrize("fmt", ["e2m1", "twiddling", "simple"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (64, 64, 64), (128, 512, 128)])
+def test_reference_test_shapes(cuda, fmt, M, N, K):
+    """Shapes of testing/python/amd/test_tilelang_mxfp4_gfx950.py:111-222, but over all 16 codes
+    and, like the reference programs, the raw unbiased exponent (2**Scale, Scale in 0..2)."""
+    _check(cuda, M, N, K, fmt, scale_bias=0, exp_range=(0, 2))
+
+
+@pytest.mark.parametrize("fmt", ["e2m1", "twiddling", "simple"])
+def test_e8m0_scales(cuda, fmt):
+    _check(cuda, 512, 768, 512, fmt, scale_bias=127)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 64), (100, 300, 192), (257, 255, 128), (300, 520, 320)])
+def test_ragged_shapes(cuda, M, N, K):
+    _check(cuda, M, N, K, "e2m1", scale_bias=127)
+
+
+@pytest.mark.parametrize("fmt", ["e2m1", "simple"])
+def test_bias(cuda, fmt):
+    _check(cuda, 384, 512, 256, fmt, scale_bias=127, with_bias=True)
+
+
+def test_weight_values_exact(cuda):
+    """A = identity picks single weights: C[i, n] must equal decode(B)[n, i] * 2**e exactly (bf16)."""
+    N, K = 512, 256
+    for fmt in ("e2m1", "twiddling", "simple"):
+        d = workloads.mxfp4(K, N, K, seed=7, scale_bias=127)
+        B = d["B"]
+        # every byte value appears
+        B[0, :] = np.arange(K // 2, dtype=np.uint8)
+        B[1, :] = np.arange(K // 2, dtype=np.uint8)[::-1] + 128
+        Bp = orc.twiddle_pack_fp4(orc.unpack_u4(B)) if fmt == "twiddling" else B
+        eye = orc.f32_to_bf16_bits(np.eye(K, dtype=np.float32))
+        kern = tl.matmul_bf16_mxfp4(K, N, K, weight_format=fmt, scale_bias=127)
+        C = kern(_dev(eye, cuda).view(torch.bfloat16), _dev(Bp, cuda), _dev(d["Scale"], cuda),
+                 torch.empty((K, N), dtype=torch.bfloat16, device=cuda))
+        torch.cuda.synchronize()
+        W = orc.mxfp4_dequant(Bp, d["Scale"], fmt, 32, 127)  # [N, K] float32, exact
+        got = C.float().cpu().numpy()
+        np.testing.assert_array_equal(got, W.T + np.float32(0.0))
+
+
+def test_full_size_properties(cuda):
+    """Benchmark configuration 4 (M=4096, N=K=8192), checked without a full CPU matmul: a sample of
+    rows and columns against the oracle, and linearity in A."""
+    M, N, K = 4096, 8192, 8192
+    d = workloads.mxfp4(M, N, K, seed=0, scale_bias=127)
+    kern = tl.matmul_bf16_mxfp4(M, N, K, weight_format="e2m1", scale_bias=127)
+    A = _dev(d["A"], cuda).view(torch.bfloat16)
+    B, S = _dev(d["B"], cuda), _dev(d["Scale"], cuda)
+    bias = torch.empty((M, N), dtype=torch.bfloat16, device=cuda)
+    C = kern(A, B, S, bias)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(1)
+    rows = rng.choice(M, 48, replace=False)
+    cols = rng.choice(N, 64, replace=False)
+    Af = orc.bf16_bits_to_f32(d["A"][rows])
+    W = orc.mxfp4_dequant(d["B"][cols], d["Scale"][cols], "e2m1", 32, 127)
+    ref = orc.bf16_bits_to_f32(orc.f32_to_bf16_bits(Af @ W.T))
+    got = C[torch.from_numpy(rows).to(cuda)][:, torch.from_numpy(cols).to(cuda)].float().cpu().numpy()
+    np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
+    # whole-matrix check against the row sample: rows of C computed by an independent call on A[rows]
+    kern_small = tl.matmul_bf16_mxfp4(len(rows), N, K, weight_format="e2m1", scale_bias=127)
+    C_rows = kern_small(A[torch.from_numpy(rows).to(cuda)].contiguous(), B, S, bias[: len(rows)].contiguous())
+    torch.cuda.synchronize()
+    assert torch.equal(C_rows, C[torch.from_numpy(rows).to(cuda)])
+    # linearity: C(2A) == 2 C(A) exactly (power-of-two scaling commutes with every rounding)
+    C2 = kern((A.float() * 2).to(torch.bfloat16), B, S, bias)
+    torch.cuda.synchronize()
+    assert torch.equal(C2.float(), C.float() * 2)

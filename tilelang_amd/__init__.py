@@ -7,7 +7,7 @@ examples' kernels.  PyTorch is used for tensors and streams only.
 
 from . import quantize  # noqa: F401
 from .adapter import KernelAdapter, KernelParam  # noqa: F401
-from .kernels import dequantize_gemv, dequantize_w4  # noqa: F401
+from .kernels import dequantize_gemv, dequantize_w4, matmul_bf16_mxfp4  # noqa: F401
 from .profiler import Profiler, TensorSupplyType, do_bench  # noqa: F401
 
 __version__ = "0.1.0"

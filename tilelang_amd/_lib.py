@@ -28,6 +28,7 @@ SIGNATURES = {
     "init": [],
     "call_dequantize_gemv_w4a16": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequantize_w4": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "call_dequant_gemm_bf16_mxfp4": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
 }
 
 

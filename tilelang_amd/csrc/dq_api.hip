@@ -20,6 +20,9 @@ int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int 
 int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                     int mode, int layout, int rows_hint, hipStream_t stream);
 
+int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
+               int scale_bias, hipStream_t stream);
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static int check_w4_args(const char* fn, const void* B, const void* S, const void* Z, int N, int K, int group, int mode,
@@ -89,4 +92,22 @@ extern "C" int call_dequantize_w4(const void* B, const void* Scale, const void* 
   if (K % 8 != 0) DQ_FAIL("%s: K=%d must be a multiple of 8", fn, K);
   if (!aligned16(W)) DQ_FAIL("%s: W must be 16-byte aligned", fn);
   return w4_dequant(B, Scale, Zeros, W, N, K, group, mode, layout, (hipStream_t)stream);
+}
+
+extern "C" int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale, const void* Bias, void* C,
+                                            int M, int N, int K, int scale_size, int fp4_format, int scale_bias,
+                                            dq_stream_t stream) {
+  const char* fn = "call_dequant_gemm_bf16_mxfp4";
+  if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
+  if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
+  if (!Scale) DQ_FAIL("%s: Scale is expected to have non-NULL data pointer", fn);
+  if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
+  if (M <= 0 || N <= 0 || K <= 0) DQ_FAIL("%s: M, N, K must be positive (got %d %d %d)", fn, M, N, K);
+  if (scale_size != 32) DQ_FAIL("%s: scale_size must be 32 (got %d)", fn, scale_size);
+  if (K % 64 != 0) DQ_FAIL("%s: K=%d must be a multiple of 64", fn, K);
+  if (fp4_format < FP4_E2M1 || fp4_format > FP4_TWIDDLING) DQ_FAIL("%s: unknown fp4 format %d", fn, fp4_format);
+  if (scale_bias < 0 || scale_bias > 255) DQ_FAIL("%s: scale_bias must be in 0..255 (got %d)", fn, scale_bias);
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C) || (Bias && !aligned16(Bias)))
+    DQ_FAIL("%s: A, B, Bias and C must be 16-byte aligned", fn);
+  return mxfp4_gemm(A, B, Scale, Bias, C, M, N, K, fp4_format, scale_bias, (hipStream_t)stream);
 }

@@ -171,3 +171,65 @@ def dequantize_w4(
         return lib.call_dequantize_w4(ptrs[0], s, z, ptrs[-1], N, K, group_size, mode, layout, stream)
 
     return KernelAdapter("dequantize_w4", params, [-1], launch, _lib.last_error)
+
+
+FP4_E2M1, FP4_SIMPLE, FP4_TWIDDLING = 0, 1, 2
+_FP4_FORMATS = {"e2m1": FP4_E2M1, "simple": FP4_SIMPLE, "twiddling": FP4_TWIDDLING}
+
+
+def matmul_bf16_mxfp4(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="bfloat16",
+    out_dtype="bfloat16",
+    accum_dtype="float32",
+    source_format="uint32",
+    num_bits: int = 4,
+    scale_size: int = 32,
+    fast_dequant: bool = True,
+    with_bias: bool = False,
+    block_M: int = 256,
+    block_N: int = 256,
+    block_K: int = 64,
+    num_stages: int = 2,
+    threads: int = 256,
+    split: int = 1,
+    weight_format: str | None = None,
+    scale_bias: int = 0,
+) -> KernelAdapter:
+    """MXFP4-weight GEMM: ``C[M,N] = A[M,K] @ (fp4(B[N,K/2]) * 2**(Scale[N,K/32] - scale_bias)).T (+ Bias)``.
+
+    Same arguments as ``matmul`` of
+    examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:61-79 (tile sizes, stages,
+    threads and split are accepted and ignored).  ``C = kernel(A, B, Scale, Bias)`` as with the
+    example's ``out_idx=[-1]``; ``Bias`` is read only when ``with_bias``.
+
+    ``weight_format``: ``"twiddling"`` (the example's ``fast_dequant=True`` layout), ``"simple"``
+    (``fast_dequant=False``) or ``"e2m1"`` (plain OCP nibbles); by default it follows
+    ``fast_dequant`` like the example.  ``scale_bias=0`` multiplies by ``2**Scale`` like the
+    example's reference program; ``scale_bias=127`` treats Scale as E8M0.
+    """
+    if num_bits != 4 or scale_size != 32:
+        raise ValueError("matmul_bf16_mxfp4: num_bits must be 4 and scale_size 32")
+    if _dtype(in_dtype) != torch.bfloat16 or _dtype(out_dtype) != torch.bfloat16:
+        raise ValueError("matmul_bf16_mxfp4: in_dtype and out_dtype must be bfloat16")
+    if K % 64 != 0:
+        raise ValueError(f"matmul_bf16_mxfp4: K={K} must be a multiple of 64")
+    if weight_format is None:
+        weight_format = "twiddling" if fast_dequant else "simple"
+    fmt = _FP4_FORMATS[weight_format]
+    params = [
+        KernelParam("A", torch.bfloat16, (M, K)),
+        KernelParam("B", torch.uint8, (N, K // 2), packed=True),
+        KernelParam("Scale", torch.uint8, (N, K // scale_size), packed=True),
+        KernelParam("Bias", torch.bfloat16, (M, N)),
+        KernelParam("C", torch.bfloat16, (M, N)),
+    ]
+
+    def launch(ptrs, stream):
+        lib = _lib.get_library()
+        bias = ptrs[3] if with_bias else None
+        return lib.call_dequant_gemm_bf16_mxfp4(ptrs[0], ptrs[1], ptrs[2], bias, ptrs[4], M, N, K, scale_size, fmt, scale_bias, stream)
+
+    return KernelAdapter("matmul_bf16_mxfp4", params, [-1], launch, _lib.last_error)
