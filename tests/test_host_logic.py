@@ -1,0 +1,206 @@
+"""Host-side logic that needs no GPU: the C-ABI library loads and exports what include/dqgemm.h declares,
+the adapter validates arguments like the reference's wrapper, the packing helpers agree with the oracle."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from tilelang_amd import _lib, quantize, workloads
+from tilelang_amd.adapter import KernelAdapter, KernelParam
+from oracle import dq_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "dqgemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"^\s*(?:int|const char\*)\s+(\w+)\s*\(", text, flags=re.M)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load_library()
+    names = _declared_symbols()
+    assert "init" in names and "get_last_error" in names and len(names) >= 4
+    for n in names:
+        assert getattr(lib, n) is not None
+    # every declared entry point has a bound signature, and nothing undeclared is bound
+    assert sorted(set(_lib.SIGNATURES) | {"get_last_error"}) == names
+    assert lib.get_last_error().decode() == "" or isinstance(lib.get_last_error(), bytes)
+
+
+def test_entry_points_reject_bad_arguments_before_any_launch():
+    """NULL pointers and impossible sizes return -1 with a message; no GPU is touched."""
+    lib = _lib.load_library()
+    vp = ctypes.c_void_p
+    assert lib.call_dequantize_gemv_w4a16(vp(0), vp(0), vp(0), vp(0), vp(0), 1, 64, 256, 128, 3, 0, -1, vp(0)) == -1
+    assert "non-NULL data pointer" in lib.get_last_error().decode()
+    buf = ctypes.create_string_buffer(4096 + 64)
+    a = vp((ctypes.addressof(buf) + 63) & ~63)
+    assert lib.call_dequantize_gemv_w4a16(a, a, a, vp(0), a, 1, 64, 200, 128, 3, 0, -1, vp(0)) == -1
+    assert "multiple" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_w4a16(a, a, a, vp(0), a, 1, 64, 384, 96, 3, 0, -1, vp(0)) == -1
+    assert "group" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_w4a16(a, a, vp(0), vp(0), a, 1, 64, 256, 128, 3, 0, -1, vp(0)) == -1
+    assert "Scale is expected to have non-NULL" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_w4a16(a, a, a, vp(0), a, 1, 64, 256, 128, 99, 0, -1, vp(0)) == -1
+    assert "unknown mode" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_w4a16(vp(a.value + 2), a, a, vp(0), a, 1, 64, 256, 128, 3, 0, -1, vp(0)) == -1
+    assert "aligned" in lib.get_last_error().decode()
+    assert lib.call_dequant_gemm_bf16_mxfp4(a, a, a, vp(0), a, 64, 64, 100, 32, 0, 127, vp(0)) == -1
+    assert "multiple of 64" in lib.get_last_error().decode()
+    assert lib.call_dequant_gemm_bf16_mxfp4(a, a, a, vp(0), a, 64, 64, 128, 16, 0, 127, vp(0)) == -1
+    assert "scale_size" in lib.get_last_error().decode()
+
+
+# ---- adapter ----------------------------------------------------------------------------------------
+
+def _cpu_adapter(result_idx=()):
+    calls = []
+
+    def launch(ptrs, stream):
+        calls.append(([p.value for p in ptrs], stream))
+        return 0
+
+    params = [KernelParam("A", torch.float16, (2, 8)), KernelParam("B", torch.int8, (4, 4), packed=True),
+              KernelParam("C", torch.float16, (2, 4))]
+    return KernelAdapter("k", params, list(result_idx), launch, lambda: "boom", device_type="cpu"), calls
+
+
+def test_adapter_passes_pointers_and_stream():
+    k, calls = _cpu_adapter()
+    A, B, C = torch.zeros(2, 8, dtype=torch.float16), torch.zeros(4, 4, dtype=torch.uint8), torch.zeros(2, 4, dtype=torch.float16)
+    assert k(A, B, C) is None
+    assert calls[0][0] == [A.data_ptr(), B.data_ptr(), C.data_ptr()] and calls[0][1] == 0
+    k(A, B, C, stream=1234)
+    assert calls[1][1] == 1234
+    k(A, None, C)
+    assert calls[2][0][1] is None or calls[2][0][1] == 0
+
+
+def test_adapter_out_idx_allocates_outputs():
+    k, calls = _cpu_adapter(result_idx=[-1])
+    A, B = torch.zeros(2, 8, dtype=torch.float16), torch.zeros(4, 4, dtype=torch.int8)
+    C = k(A, B)
+    assert C.shape == (2, 4) and C.dtype == torch.float16 and calls[0][0][2] == C.data_ptr()
+
+
+@pytest.mark.parametrize("case,match", [
+    ("count", r"Expected 3 inputs, got 2 with 2 inputs and 0 outputs"),
+    ("dtype", r"Buffer dtype mismatch for parameter A: expected torch.float16, got torch.float32"),
+    ("ndim", r"Static shape mismatch for parameter A: expected 2 dimensions, got 1"),
+    ("shape", r"Static shape mismatch for parameter A: expected 8 at index 1, got 16"),
+    ("stride", r"Static stride mismatch for parameter C"),
+    ("device", r"Buffer device mismatch for parameter A"),
+])
+def test_adapter_validation_errors(case, match):
+    """Same classes as the reference wrapper (tilelang/jit/adapter/cython/cython_wrapper.pyx:78-156,172-175)."""
+    k, calls = _cpu_adapter()
+    A, B, C = torch.zeros(2, 8, dtype=torch.float16), torch.zeros(4, 4, dtype=torch.int8), torch.zeros(2, 4, dtype=torch.float16)
+    with pytest.raises(ValueError, match=match):
+        if case == "count":
+            k(A, B)
+        elif case == "dtype":
+            k(A.float(), B, C)
+        elif case == "ndim":
+            k(A.reshape(-1), B, C)
+        elif case == "shape":
+            k(torch.zeros(2, 16, dtype=torch.float16), B, C)
+        elif case == "stride":
+            k(A, B, torch.zeros(4, 2, dtype=torch.float16).t())
+        elif case == "device":
+            k(A.to("meta"), B, C)
+    assert not calls
+    if case != "count":
+        # validation can be skipped like in the reference
+        args = {"dtype": (A.float(), B, C), "ndim": (A.reshape(-1), B, C)}.get(case)
+        if args:
+            k(*args, skip_tensor_validation=True)
+            assert len(calls) == 1
+
+
+def test_adapter_error_code_raises_runtime_error():
+    params = [KernelParam("A", torch.float16, (1, 8))]
+    k = KernelAdapter("k", params, [], lambda ptrs, s: -1, lambda: "boom", device_type="cpu")
+    with pytest.raises(RuntimeError, match="Kernel call failed: boom"):
+        k(torch.zeros(1, 8, dtype=torch.float16))
+
+
+def test_kernels_refuse_cpu_tensors_and_bad_factory_arguments():
+    kern = tl.dequantize_gemv(1, 64, 256, group_size=128, source_format="int", with_scaling=True)
+    A, B = torch.zeros(1, 256, dtype=torch.float16), torch.zeros(64, 128, dtype=torch.int8)
+    S, C = torch.zeros(64, 2, dtype=torch.float16), torch.zeros(1, 64, dtype=torch.float16)
+    with pytest.raises(ValueError, match="Buffer device mismatch for parameter A: expected cuda"):
+        kern(A, B, S, C)
+    with pytest.raises(ValueError, match="multiple of 128"):
+        tl.dequantize_gemv(1, 64, 200)
+    with pytest.raises(ValueError, match="group_size"):
+        tl.dequantize_gemv(1, 64, 256, group_size=48, with_scaling=True)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        tl.matmul_bf16_mxfp4(64, 64, 96)
+    with pytest.raises(AssertionError):
+        tl.dequantize_gemv(1, 64, 256, trans_A=True)
+
+
+# ---- packing helpers against the oracle ---------------------------------------------------------------
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_general_compress_matches_oracle(bits):
+    rng = np.random.default_rng(bits)
+    x = rng.integers(0, 1 << bits, size=(6, 64)).astype(np.int8)
+    got = quantize.general_compress(torch.from_numpy(x), bits).numpy()
+    np.testing.assert_array_equal(got, orc.general_compress(x, bits))
+    assert got.dtype == np.int8
+
+
+@pytest.mark.parametrize("nbits,target", [(4, "float16"), (2, "int8"), (2, "float16"), (1, "int8"), (1, "float16"), (4, "int8")])
+def test_interleave_weight_matches_oracle(nbits, target):
+    rng = np.random.default_rng(nbits)
+    raw = rng.integers(-128, 128, size=(8, 32)).astype(np.int8)
+    got = quantize.interleave_weight(torch.from_numpy(raw), nbits, target).numpy()
+    np.testing.assert_array_equal(got, orc.interleave_weight(raw, nbits, target))
+    assert got.dtype == np.int8 and got.shape == raw.shape
+
+
+def test_pack_and_fp4_helpers_match_oracle():
+    rng = np.random.default_rng(0)
+    x = rng.integers(-8, 8, size=(4, 32)).astype(np.int8)
+    np.testing.assert_array_equal(quantize.pack_int4(torch.from_numpy(x)).numpy(), orc.pack_int4(x))
+    with pytest.raises(TypeError):
+        quantize.pack_int4(torch.zeros(2, 4, dtype=torch.int32))
+    with pytest.raises(ValueError):
+        quantize.pack_int4(torch.zeros(2, 3, dtype=torch.int8))
+    v = (rng.standard_normal((3, 64)) * 3).astype(np.float32)
+    v[0, :8] = [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.25]  # the rounding thresholds
+    codes = quantize.encode_fp4_e2m1_values(torch.from_numpy(v))
+    np.testing.assert_array_equal(codes.numpy(), orc.encode_fp4_e2m1_values(v))
+    packed = quantize.pack_fp4_e2m1_codes(codes)
+    np.testing.assert_array_equal(packed.numpy().view(np.uint8), orc.pack_fp4_e2m1_codes(codes.numpy()))
+    np.testing.assert_array_equal(quantize.decode_packed_fp4_e2m1(packed).numpy(), orc.decode_fp4_e2m1(packed.numpy()))
+    values = torch.tensor([[0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.5, -1.0]])
+    assert quantize.encode_fp4_e2m1_values(values).tolist() == [[0, 1, 2, 3, 4, 5, 6, 7, 9, 10]]
+
+
+def test_workload_generators_are_seeded_and_shaped():
+    a, b = workloads.w4a16(1, 64, 256, 128, seed=3), workloads.w4a16(1, 64, 256, 128, seed=3)
+    for k in a:
+        np.testing.assert_array_equal(a[k], b[k])
+    assert a["B"].shape == (64, 128) and a["Scale"].shape == (64, 2) and a["Scale"].dtype == np.float16
+    assert 0.005 <= a["Scale"].min() and a["Scale"].max() <= 0.02
+    z = workloads.w4a16(4, 32, 256, 128, seed=1, zeros_range=(6, 10))["Zeros"]
+    assert set(np.unique(z)).issubset({6, 7, 8, 9, 10})
+    m = workloads.mxfp4(8, 16, 128, seed=0)
+    assert m["Scale"].min() >= 119 and m["Scale"].max() <= 127 and m["A"].dtype == np.uint16
+    bn = workloads.bitnet(2, 8, 64, seed=0)
+    np.testing.assert_array_equal(orc.decode_i2(bn["B"], "offset"), bn["W"])
+    # algorithmic byte counts of the benchmark configurations
+    assert workloads.w4a16_bytes(1, 28672, 8192) == 121184256
+    assert workloads.w4a16_bytes(64, 28672, 8192, zeros=True) == 129499136
+    assert workloads.mxfp4_bytes(4096, 8192, 8192) == 169869312
+    assert workloads.bitnet_bytes(2048, 8192, 8192) == 67117060
+    assert workloads.flops(4096, 8192, 8192) == 549755813888

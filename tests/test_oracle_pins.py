@@ -1,0 +1,297 @@
+"""Pins of the CPU oracle (no GPU): golden vectors the reference's own tests hold, closed forms,
+brute force over finite domains, round trips, and reduction to integer / float64 arithmetic."""
+
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import dq_oracle as orc
+
+E2M1 = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0]
+
+
+# ---- golden vectors from the reference's tests ---------------------------------------------------
+
+@pytest.mark.parametrize("nbit,values", [(2, [-2, -1, 0, 1]), (4, list(range(-8, 8))), (8, [-128, -17, -1, 0, 1, 42, 127])])
+def test_sign_extend_known_answers(nbit, values):
+    """testing/python/issue/test_tilelang_u32_signed_decode.py:26-30: pack (value & mask) << (pos * nbit), decode."""
+    mask = (1 << nbit) - 1
+    lanes = 32 // nbit
+    words = []
+    for start in range(0, len(values), lanes):
+        w = 0
+        for pos, v in enumerate(values[start:start + lanes]):
+            w |= (v & mask) << (pos * nbit)
+        words.append(w)
+    out = []
+    for i in range(len(values)):
+        field = (words[i // lanes] >> ((i % lanes) * nbit)) & mask
+        out.append(int(orc.sign_extend(np.array([field]), nbit)[0]))
+    assert out == values
+
+
+def test_e2m1_encode_pack_known_answer():
+    """testing/python/quantize/test_tilelang_quantize_nvfp4_scale_layout.py:881-887."""
+    values = np.array([[0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.5, -1.0]], dtype=np.float32)
+    codes = orc.encode_fp4_e2m1_values(values)
+    assert codes.tolist() == [[0x0, 0x1, 0x2, 0x3, 0x4, 0x5, 0x6, 0x7, 0x9, 0xA]]
+    packed = orc.pack_fp4_e2m1_codes(codes)
+    assert packed.tolist() == [[0x10, 0x32, 0x54, 0x76, 0xA9]]
+    np.testing.assert_array_equal(orc.decode_fp4_e2m1(packed), values)
+
+
+def test_e2m1_table_all_bytes():
+    """Value table of nvfp4.py:17-34 / test_tilelang_mxfp4_gfx950.py:32,49, for all 256 bytes, low nibble first."""
+    b = np.arange(256, dtype=np.uint8).reshape(1, 256)
+    got = orc.decode_fp4_e2m1(b).reshape(256, 2)
+    for byte in range(256):
+        assert got[byte, 0] == E2M1[byte & 15] and got[byte, 1] == E2M1[byte >> 4]
+        assert np.signbit(got[byte, 0]) == (byte & 8 != 0) and np.signbit(got[byte, 1]) == (byte & 0x80 != 0)
+
+
+# ---- closed forms over finite domains ------------------------------------------------------------
+
+def test_simple_fp4_closed_form():
+    """bits (s<<15)|((E+126)<<7)|(m<<6) is the bf16 (-1)^s 2^(E-1) (1 + m/2) for every E; fp16 twin likewise."""
+    b = np.arange(256, dtype=np.uint8).reshape(1, 256)
+    bf = orc.bf16_bits_to_f32(orc.decode_fp4_simple_bf16_bits(b)).reshape(256, 2)
+    h = orc.decode_fp4_simple_f16(b).astype(np.float32).reshape(256, 2)
+    for byte in range(256):
+        for half, nib in enumerate((byte & 15, byte >> 4)):
+            s, E, m = nib >> 3, (nib >> 1) & 3, nib & 1
+            want = (-1.0) ** s * 2.0 ** (E - 1) * (1 + m / 2)
+            assert bf[byte, half] == want and h[byte, half] == want
+    # agrees with true e2m1 except for E == 0 (0.5, 0.75 instead of 0, 0.5)
+    for nib in range(16):
+        if (nib >> 1) & 3:
+            assert bf[nib, 0] == E2M1[nib]
+
+
+def test_simple_fp4_scaled_exponent_clamp():
+    """quantization.py:30-73: the scale byte adds to the exponent, clamped at 255."""
+    b = np.array([[0x31, 0xF7]], dtype=np.uint8)  # 4 nibbles
+    sc = np.array([[3]], dtype=np.uint8)
+    got = orc.bf16_bits_to_f32(orc.decode_fp4_simple_bf16_bits(b, sc, scale_size=4))
+    base = orc.bf16_bits_to_f32(orc.decode_fp4_simple_bf16_bits(b))
+    np.testing.assert_array_equal(got, base * 8)
+    big = orc.decode_fp4_simple_bf16_bits(b, np.array([[250]], dtype=np.uint8), scale_size=4)
+    assert ((big >> 7) & 0xFF).max() == 255
+
+
+def test_twiddling_all_65536_units():
+    """dequantize_utils.py:4-54 over every 16-bit unit: each of the 4 outputs is the e2m1 value of the code
+    gathered from the documented bit positions."""
+    w = np.arange(65536, dtype=np.uint32)
+    packed = np.stack((w >> 8, w & 0xFF), axis=-1).astype(np.uint8).reshape(1, -1)
+    got = orc.decode_fp4_twiddling(packed).reshape(65536, 4)
+    pos = [(15, 8, 7, 6), (12, 5, 4, 3), (9, 2, 1, 0), (14, 11, 10, 13)]
+    lut = np.array(E2M1, dtype=np.float32)
+    for p, (s, e1, e0, m) in enumerate(pos):
+        code = (((w >> s) & 1) << 3) | (((w >> e1) & 1) << 2) | (((w >> e0) & 1) << 1) | ((w >> m) & 1)
+        want = lut[code]
+        np.testing.assert_array_equal(got[:, p], want)
+        np.testing.assert_array_equal(np.signbit(got[:, p]), np.signbit(want))
+
+
+def test_twiddle_pack_round_trip():
+    rng = np.random.default_rng(0)
+    codes = rng.integers(0, 16, size=(7, 64), dtype=np.uint8)
+    np.testing.assert_array_equal(orc.decode_fp4_twiddling(orc.twiddle_pack_fp4(codes)), orc.E2M1_VALUES[codes])
+
+
+def test_magic_number_int_to_fp16():
+    """(0x6400 | q) is the fp16 1024 + q; minus 1032 / 1024 gives q - 8 / q exactly (lop3.py:12-24)."""
+    for q in range(16):
+        assert np.array([0x6400 | q], dtype=np.uint16).view(np.float16)[0] == 1024 + q
+    w = np.array([0x76543210, 0xFEDCBA98], dtype=np.uint32)
+    # fast decode emits nibble pairs (i, i+4)
+    got_u = orc.fast_decode_i4_to_f16(w, signed=False)
+    assert got_u[0].tolist() == [0, 4, 1, 5, 2, 6, 3, 7]
+    assert orc.fast_decode_i4_to_f16(w, signed=True)[1].tolist() == [0, 4, 1, 5, 2, 6, 3, 7]
+
+
+def test_w4_scale_single_rounding():
+    """(q - 8) * s in fp16 with one rounding equals the correctly rounded exact product for all q and many s."""
+    rng = np.random.default_rng(1)
+    s = rng.uniform(1e-4, 2.0, size=(1, 512)).astype(np.float16)
+    for q in range(16):
+        packed = np.full((1, 256), q | (q << 4), dtype=np.uint8)
+        got = orc.dequant_u4_scale(packed, s, group=1)
+        want = np.array([np.float16(float(q - 8) * float(x)) for x in s[0]], dtype=np.float16)  # exact in float64, one rounding
+        np.testing.assert_array_equal(got[0].view(np.uint16), want.view(np.uint16))
+
+
+def test_w4_zeros_modes_rounding_order():
+    packed = np.array([[0xF0, 0x7A]], dtype=np.uint8)  # q = 0, 15, 10, 7
+    s = np.array([[0.0123]], dtype=np.float16)
+    z = np.array([[7.5]], dtype=np.float16)
+    q = np.array([0, 15, 10, 7], dtype=np.float64)
+    orig = orc.dequant_u4_scale_zeros(packed, s, z, 4, "original")[0]
+    want = [np.float16(float(np.float16(x - 7.5)) * float(s[0, 0])) for x in q]
+    assert orig.tolist() == [float(v) for v in want]
+    resc = orc.dequant_u4_scale_zeros(packed, s, z, 4, "rescale")[0]
+    want = [np.float16(x * float(s[0, 0]) - 7.5) for x in q]
+    assert resc.tolist() == [float(v) for v in want]
+    quant = orc.dequant_u4_scale_zeros(packed, s, np.array([[7]]), 4, "quantized")[0]
+    want = [np.float16((x - 7) * float(s[0, 0])) for x in q]
+    assert quant.tolist() == [float(v) for v in want]
+
+
+def test_i2_conventions():
+    packed = np.array([[0b11100100]], dtype=np.uint8)  # codes 0,1,2,3 low first
+    assert orc.unpack_u2(packed).tolist() == [[0, 1, 2, 3]]
+    assert orc.decode_i2(packed, "unsigned").tolist() == [[0, 1, 2, 3]]
+    assert orc.decode_i2(packed, "offset").tolist() == [[-2, -1, 0, 1]]
+    assert orc.decode_i2(packed, "twos").tolist() == [[0, 1, -2, -1]]
+
+
+def test_bf16_rounding_helper():
+    x = np.array([1.0, 1.00390625, 1.01171875, 3.0e38, -2.5, 1e-40], dtype=np.float32)
+    import torch
+
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    np.testing.assert_array_equal(orc.f32_to_bf16_bits(x), want)
+
+
+# ---- packing invariants ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_general_compress_round_trip(bits):
+    rng = np.random.default_rng(bits)
+    x = rng.integers(0, 1 << bits, size=(5, 64), dtype=np.int8)
+    p = orc.general_compress(x, bits)
+    assert p.dtype == np.int8 and p.shape == (5, 64 * bits // 8)
+    np.testing.assert_array_equal(orc.general_decompress(p, bits), x.astype(np.uint8))
+    # element j*epb + k sits at bit bits*k of byte j
+    epb = 8 // bits
+    assert (int(p.view(np.uint8)[0, 0]) >> (bits * 1)) & ((1 << bits) - 1) == x[0, 1]
+    assert epb * p.shape[1] == x.shape[1]
+
+
+def test_interleave_fast_decode_equals_plain_decode():
+    """fast_decode(interleave_weight(p)) == plain_decode(p) for random words (4 bit -> fp16, 2 bit -> int8)."""
+    rng = np.random.default_rng(0)
+    raw = rng.integers(0, 256, size=(16, 64), dtype=np.uint8)
+    il = orc.interleave_weight(raw.view(np.int8), 4, "float16")
+    fast = orc.fast_decode_i4_to_f16(il.view(np.uint32).reshape(16, -1), signed=False).reshape(16, -1)
+    np.testing.assert_array_equal(fast, orc.unpack_u4(raw).astype(np.float16))
+    il2 = orc.interleave_weight(raw.view(np.int8), 2, "int8")
+    fast2 = orc.fast_decode_i2_to_i8(il2.view(np.uint32).reshape(16, -1), signed=True).reshape(16, -1)
+    np.testing.assert_array_equal(fast2, orc.decode_i2(raw, "offset"))
+    # a bit permutation: population count preserved, and nibble order 0,2,4,6,1,3,5,7
+    assert np.unpackbits(il.view(np.uint8)).sum() == np.unpackbits(raw).sum()
+    one = orc.interleave_weight(np.array([0x76543210], dtype=np.uint32).view(np.int8), 4, "float16").view(np.uint32)[0]
+    assert one == 0x75316420
+
+
+@pytest.mark.parametrize("nbits,target", [(1, "int8"), (2, "float16"), (1, "float16"), (2, "int8"), (4, "int8")])
+def test_interleave_is_bit_permutation(nbits, target):
+    for bit in range(32):
+        w = np.array([1 << bit], dtype=np.uint32)
+        out = orc.interleave_weight(w.view(np.int8), nbits, target).view(np.uint32)[0]
+        assert bin(int(out)).count("1") == 1
+    outs = {int(orc.interleave_weight(np.array([1 << b], dtype=np.uint32).view(np.int8), nbits, target).view(np.uint32)[0]) for b in range(32)}
+    assert len(outs) == 32
+
+
+def test_pack_int4():
+    x = np.array([[-8, 7, -1, 0, 3, -4]], dtype=np.int8)
+    p = orc.pack_int4(x)
+    assert p.view(np.uint8).tolist() == [[0x78, 0x0F, 0xC3]]
+    np.testing.assert_array_equal(orc.decode_i4_signed(p), x)
+    with pytest.raises(TypeError):
+        orc.pack_int4(x.astype(np.int32))
+    with pytest.raises(ValueError):
+        orc.pack_int4(x[:, :5])
+
+
+# ---- matmuls against brute force ------------------------------------------------------------------
+
+def test_ref_w4a16_brute_force():
+    rng = np.random.default_rng(2)
+    M, N, K, g = 2, 5, 64, 32
+    A = rng.standard_normal((M, K)).astype(np.float16)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    S = rng.uniform(0.005, 0.02, size=(N, K // g)).astype(np.float16)
+    got = orc.ref_w4a16(A, B, S, group=g, mode="scale")
+    for m, n in itertools.product(range(M), range(N)):
+        acc = 0.0
+        for k in range(K):
+            q = (B[n, k // 2] >> (4 * (k % 2))) & 15
+            w = np.float16(np.float64(q - 8.0) * np.float64(S[n, k // g]))
+            acc += float(A[m, k]) * float(w)
+        assert abs(float(got[m, n]) - acc) <= 2e-3 * max(1.0, abs(acc))
+
+
+def test_ref_int_paths_brute_force():
+    rng = np.random.default_rng(3)
+    M, N, K = 3, 4, 32
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    B4 = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    B2 = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    w4 = np.zeros((N, K), dtype=np.int64)
+    w2 = np.zeros((N, K), dtype=np.int64)
+    for n, k in itertools.product(range(N), range(K)):
+        q = (int(B4[n, k // 2]) >> (4 * (k % 2))) & 15
+        w4[n, k] = q - 16 if q >= 8 else q
+        w2[n, k] = ((int(B2[n, k // 4]) >> (2 * (k % 4))) & 3) - 2
+    a = A.astype(np.int64)
+    np.testing.assert_array_equal(orc.ref_w4a8(A, B4), (a @ w4.T).T)
+    np.testing.assert_array_equal(orc.ref_bitnet_int(A, B2, "offset"), a @ w2.T)
+    Ap = rng.integers(0, 256, size=(M, K // 2), dtype=np.uint8)
+    a4 = orc.decode_i4_signed(Ap).astype(np.int64)
+    np.testing.assert_array_equal(orc.ref_int4xint4(Ap, B4), a4 @ w4.T)
+    assert orc.ref_w4a8(A, B4).dtype == np.int32 and orc.ref_w4a8(A, B4).shape == (N, M)
+
+
+def test_ref_mxfp4_exact_scaling_and_identity():
+    rng = np.random.default_rng(4)
+    N, K = 8, 64
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    S = rng.integers(119, 128, size=(N, K // 32), dtype=np.uint8)
+    W = orc.mxfp4_dequant(B, S, "e2m1", 32, 127)
+    # exact: every value is an e2m1 value times a power of two, hence a bf16
+    np.testing.assert_array_equal(orc.round_to_bf16(W), W)
+    eye = orc.f32_to_bf16_bits(np.eye(K, dtype=np.float32))
+    C = orc.bf16_bits_to_f32(orc.ref_mxfp4(eye, B, S, fmt="e2m1", scale_bias=127))
+    np.testing.assert_array_equal(C, W.T)
+    # reference mode: raw exponent, 2**Scale
+    W0 = orc.mxfp4_dequant(B, np.full((N, 2), 2, np.uint8), "e2m1", 32, 0)
+    np.testing.assert_array_equal(W0, orc.decode_fp4_e2m1(B) * 4)
+
+
+def test_bitlinear_quantisers_and_epilogue():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, 16)).astype(np.float32) * 3
+    xq, s = orc.activation_quant(x)
+    assert xq.dtype == np.int8 and np.abs(xq).max() == 127 and s.shape == (3, 1)
+    np.testing.assert_allclose(s[:, 0], 127.0 / np.abs(x).max(axis=1), rtol=1e-6)
+    w = rng.standard_normal((4, 16)).astype(np.float32)
+    wq, sw = orc.weight_quant(w)
+    assert set(np.unique(wq)).issubset({-1, 0, 1}) and abs(sw - 1 / np.abs(w).mean()) < 1e-5
+    acc = np.array([[100, -7]], dtype=np.int32)
+    out = orc.post_quant_process(acc, np.array([[4.0]], np.float32), np.float32(2.0))
+    assert out.dtype == np.float16 and out.tolist() == [[12.5, -0.875]]
+
+
+def test_torch_restatement_matches_numpy_oracle():
+    import torch
+
+    from oracle import ref_torch
+    from tilelang_amd import workloads
+
+    d = workloads.w4a16(2, 64, 256, 128, seed=1, zeros_range=(6, 10))
+    a, b, s, z = (torch.from_numpy(d[k]) for k in ("A", "B", "Scale", "Zeros"))
+    np.testing.assert_allclose(ref_torch.ref_w4a16(a, b, s).numpy().astype(np.float32),
+                               orc.ref_w4a16(d["A"], d["B"], d["Scale"], group=128, mode="scale").astype(np.float32), rtol=2e-3, atol=2e-3)
+    np.testing.assert_allclose(ref_torch.ref_w4a16(a, b, s, z).numpy().astype(np.float32),
+                               orc.ref_w4a16(d["A"], d["B"], d["Scale"], d["Zeros"], 128, "original").astype(np.float32), rtol=2e-3, atol=2e-3)
+    m = workloads.mxfp4(8, 32, 128, seed=2, scale_bias=127)
+    got = ref_torch.ref_mxfp4_e2m1(torch.from_numpy(m["A"]).view(torch.bfloat16), torch.from_numpy(m["B"]), torch.from_numpy(m["Scale"]))
+    want = orc.bf16_bits_to_f32(orc.ref_mxfp4(m["A"], m["B"], m["Scale"], fmt="e2m1", scale_bias=127))
+    np.testing.assert_allclose(got.float().numpy(), want, rtol=1e-2, atol=1e-2)
+    bn = workloads.bitnet(4, 16, 64, seed=3)
+    got = ref_torch.ref_bitnet(torch.from_numpy(bn["A"]), torch.from_numpy(bn["B"]), torch.from_numpy(bn["s_a"]), float(bn["s_w"]))
+    want = orc.ref_bitnet(bn["A"], bn["B"], bn["s_a"], bn["s_w"], "offset")
+    np.testing.assert_allclose(got.numpy().astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=2e-3)

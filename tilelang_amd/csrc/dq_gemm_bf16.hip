@@ -322,8 +322,12 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
 #define DQ_MX(FMT_, BIAS_)                                                                                          \
   do {                                                                                                              \
     auto kern = mxfp4_gemm_kernel<FMT_, BIAS_>;                                                                     \
-    DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                     kLdsBytes));                                                                   \
+    static bool lds_limit_raised = false;                                                                           \
+    if (!lds_limit_raised) {                                                                                        \
+      DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                         \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));                     \
+      lds_limit_raised = true;                                                                                      \
+    }                                                                                                               \
     hipLaunchKernelGGL(kern, grid, block, kLdsBytes, stream, (const bf16_t*)A, (const uint8_t*)B, (const uint8_t*)S, \
                        (const bf16_t*)Bias, (bf16_t*)C, M, N, K, scale_off, tiles_m, tiles_n);                      \
   } while (0)

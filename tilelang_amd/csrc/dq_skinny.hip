@@ -262,9 +262,12 @@ int launch_skinny(const void* A, const void* B, const void* S, const void* Z, vo
 #define DQ_LAUNCH2(MODE_, APERM_, G128_)                                                                             \
   do {                                                                                                               \
     auto kern = w4a16_skinny_kernel<MB, RB, WAVES, U, MODE_, APERM_, G128_>;                                         \
-    if (lds_bytes > 48 * 1024)                                                                                       \
+    static bool lds_limit_raised = false; /* once per kernel: legal under stream capture afterwards */            \
+    if (!lds_limit_raised) {                                                                                         \
       DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                          \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));                 \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));                      \
+      lds_limit_raised = true;                                                                                       \
+    }                                                                                                                \
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,  \
                        (const half_t*)Z, (half_t*)C, M, N, K, group, KT);                                            \
   } while (0)
@@ -324,7 +327,8 @@ int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, voi
                  int mode, int layout, int variant, hipStream_t stream) {
   // variant < 0: heuristic.  Otherwise an explicit (benchmarking) choice, see switch below.
   if (variant < 0) {
-    if (M <= 16) variant = 0;
+    if (M <= 4) variant = 0;
+    else if (M <= 16) variant = 10;
     else if (M <= 32) variant = 4;
     else variant = 5;
   }
@@ -345,7 +349,7 @@ int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, voi
     DQ_V(7, 1, 1, 8, 8, false);
     DQ_V(8, 1, 1, 8, 4, false);
     DQ_V(9, 1, 2, 8, 4, false);
-    DQ_V(10, 1, 4, 4, 2, false);
+    DQ_V(10, 1, 4, 4, 2, true);
     DQ_V(11, 1, 1, 16, 4, false);
     DQ_V(12, 1, 1, 8, 2, false);
 #undef DQ_V
