@@ -87,6 +87,44 @@ enum dq_fp4_format {
 int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale, const void* Bias, void* C, int M,
                                  int N, int K, int scale_size, int fp4_format, int scale_bias, dq_stream_t stream);
 
+/* ---- further dequantize GEMMs (same 256x256 MFMA kernel, different decoders) ------------------ */
+
+/* fp16 x "simple" fp4: C[M,N] (transposed = 0) or Ct[N,M] (transposed = 1) fp16 =
+ * A[M,K] fp16 . fp16bits((s<<15)|((E+14)<<10)|(m<<9))(B[N,K/2])^T, fp32 accumulation.  Replaces
+ * `call(A, B, Ct, stream)` of examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:179-215.
+ * Requires K % 64 == 0. */
+int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int N, int K, int transposed,
+                               dq_stream_t stream);
+
+/* fp16 x uint4 with the integer decoders: C[M,N] fp16 = A[M,K] fp16 . dequant(B, Scale, Zeros)^T with
+ * the dequantised tile rounded to fp16 exactly as call_dequantize_w4 does.  Replaces `call(A, B, C)` of
+ * examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:45-88 (mode DQ_W4_UNSIGNED) and serves
+ * W4A16 at M > 64.  Requires K % 64 == 0; group rules as for call_dequantize_gemv_w4a16. */
+int call_dequant_gemm_w4_fp16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M,
+                              int N, int K, int group, int mode, int layout, dq_stream_t stream);
+
+enum dq_i2_convention {
+  DQ_I2_UNSIGNED = 0, /* w = c       decode_i2u_to_i8s, examples/dequantize_gemm/quantize/lop3.py:975-997 */
+  DQ_I2_OFFSET = 1,   /* w = c - 2   decode_i2s_to_i8s, lop3.py:950-973                                   */
+  DQ_I2_TWOS = 2      /* w = sext2(c) quantization.py:333-343                                             */
+};
+
+/* int8 x 2-bit: C[M,N] = A[M,K] int8 . decode(B[N,K/4])^T, exact int32 accumulation.  out_kind 0: C is
+ * int32.  out_kind 1: C is fp16 = (float(acc) / s_a[m]) / s_w, the BitLinear epilogue
+ * (examples/bitnet-1.58b/utils_quant.py:165-170), s_a fp32 [M].  B is the plain layout: byte j holds
+ * codes 4j..4j+3 at bits 0,2,4,6.  Replaces `call(A, B, C, stream)` of examples/bitnet-1.58b/
+ * kernel_benchmark/tilelang_bitnet_158_int8xint2_prefill.py:188-296.  Requires K % 128 == 0. */
+int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a,
+                        float s_w, int out_kind, dq_stream_t stream);
+
+/* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T.
+ * is_signed 1: two's-complement nibbles (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:10-21,
+ * `call(A, B, Ct)` :109-147); 0: unsigned nibbles (example_dequant_gemm_fine_grained.py int8 path).
+ * a_packed 1: A is packed int4 too, A[M,K/2] (examples/gemm_int4/example_tilelang_gemm_int4.py:17-38).
+ * Requires K % 128 == 0. */
+int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed,
+                        int transposed, dq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

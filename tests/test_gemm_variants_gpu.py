@@ -1,0 +1,171 @@
+"""GPU parity of the remaining dequantize GEMMs (through the C-ABI) against the CPU oracle: integer
+accumulations bit-exact, fp16 outputs within rtol=atol=1e-2."""
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from tilelang_amd import quantize, workloads
+from oracle import dq_oracle as orc
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def _dev(x, cuda):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(cuda)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (512, 512, 512), (100, 130, 384), (1, 8, 128)])
+def test_w4a8_exact(cuda, M, N, K):
+    """examples/dequantize_gemm/example_dequant_gemm_w4a8.py: Ct[N,M] int32, all byte values."""
+    d = workloads.int8_int4(M, N, K, seed=M)
+    Ct = tl.matmul_int8xint4(M, N, K)(_dev(d["A"], cuda), _dev(d["B"], cuda))
+    torch.cuda.synchronize()
+    assert Ct.shape == (N, M) and Ct.dtype == torch.int32
+    np.testing.assert_array_equal(Ct.cpu().numpy(), orc.ref_w4a8(d["A"], d["B"]))
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (16, 16, 128), (300, 200, 256)])
+def test_int4xint4_exact(cuda, M, N, K):
+    """examples/gemm_int4/example_tilelang_gemm_int4.py:70-103: rtol=0, atol=0."""
+    d = workloads.int4_int4(M, N, K, seed=K)
+    Ap = quantize.pack_int4(torch.from_numpy(d["A_logical"])).to(cuda)
+    Bp = quantize.pack_int4(torch.from_numpy(d["B_logical"])).to(cuda)
+    C = tl.matmul_nt_int4(M, N, K)(Ap, Bp)
+    torch.cuda.synchronize()
+    ref = d["A_logical"].astype(np.int64) @ d["B_logical"].astype(np.int64).T
+    np.testing.assert_array_equal(C.cpu().numpy(), ref.astype(np.int32))
+    np.testing.assert_array_equal(orc.ref_int4xint4(Ap.cpu().numpy(), Bp.cpu().numpy()), ref.astype(np.int32))
+
+
+@pytest.mark.parametrize("in_dtype", ["float16", "int8"])
+def test_fine_grained(cuda, in_dtype):
+    """examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:425-428 shapes (256^3), random nibbles."""
+    M = N = K = 256
+    rng = np.random.default_rng(0)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    kern = tl.matmul_w4_fine_grained(M, N, K, in_dtype=in_dtype)
+    if in_dtype == "int8":
+        A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+        C = kern(_dev(A, cuda), _dev(B, cuda).view(torch.int8))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_u4_int8(A, B))
+    else:
+        A = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+        C = kern(_dev(A, cuda), _dev(B, cuda).view(torch.int8))
+        torch.cuda.synchronize()
+        ref = orc.ref_w4a16(A, B, mode="unsigned")
+        np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL * 10)
+
+
+@pytest.mark.parametrize("transposed", [True, False])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (72, 200, 128)])
+def test_fp16_fp4(cuda, transposed, M, N, K):
+    """examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py: Ct[N,M] fp16, all byte values."""
+    rng = np.random.default_rng(1)
+    A = (rng.standard_normal((M, K), dtype=np.float32) * 0.5).astype(np.float16)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    out = tl.matmul_fp16_fp4(M, N, K, transposed_output=transposed)(_dev(A, cuda), _dev(B, cuda))
+    torch.cuda.synchronize()
+    ref = orc.ref_fp16xfp4(A, B)
+    if not transposed:
+        ref = ref.T
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+
+
+def test_fp16_fp4_weights_exact(cuda):
+    K, N = 128, 256
+    B = np.tile(np.arange(256, dtype=np.uint8), (N, 1))[:, : K // 2].copy()
+    B[1] = B[0][::-1] + 64
+    eye = np.eye(K, dtype=np.float16)
+    out = tl.matmul_fp16_fp4(K, N, K)(_dev(eye, cuda), _dev(B, cuda))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy().astype(np.float32), orc.decode_fp4_simple_f16(B).astype(np.float32))
+
+
+@pytest.mark.parametrize("mode", ["scale", "original", "rescale", "signed"])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_w4a16_large_m(cuda, mode, interleaved):
+    """W4A16 through the MFMA GEMM (M > 64): same tile-exact decoders as the decode kernel."""
+    M, N, K, group = 200, 320, 512, 128
+    d = workloads.w4a16(M, N, K, group, seed=2, scale_range=(0.002, 0.01), zeros_range=(6, 10))
+    kw = {"scale": dict(source_format="int"), "original": dict(source_format="uint", with_zeros=True),
+          "rescale": dict(source_format="uint", with_zeros=True, zeros_mode="rescale"),
+          "signed": dict(with_scaling=False)}[mode]
+    Bdev = _dev(d["B"], cuda).view(torch.int8)
+    if interleaved:
+        if mode == "signed":
+            pytest.skip("the sign-extending decoder is the plain-layout slow path")
+        Bdev = quantize.interleave_weight(Bdev, 4, "float16")
+    kern = tl.matmul_w4a16(M, N, K, group_size=group, fast_decoding=interleaved, **kw)
+    args = [_dev(d["A"], cuda), Bdev]
+    if kw.get("with_scaling", True):
+        args.append(_dev(d["Scale"], cuda))
+    if kw.get("with_zeros"):
+        args.append(_dev(d["Zeros"], cuda))
+    C = torch.empty((M, N), dtype=torch.float16, device=cuda)
+    kern(*args, C)
+    torch.cuda.synchronize()
+    ref = orc.ref_w4a16(d["A"], d["B"], d["Scale"], d["Zeros"], group, mode)
+    np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384)])
+def test_bitnet_gemm_int32_exact(cuda, convention, M, N, K):
+    """tilelang_bitnet_158_int8xint2_prefill.py:360-381 (256^3, B in {0,1}) generalised to all codes, exact."""
+    rng = np.random.default_rng(M + K)
+    A = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+    B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    C = torch.zeros((M, N), dtype=torch.int32, device=cuda)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, convention=convention)(_dev(A, cuda), _dev(B, cuda).view(torch.int8), C)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
+
+
+def test_bitnet_reference_example_inputs(cuda):
+    """The reference's own check: A in [0,4), B in {0,1} compressed with general_compress (no interleave here)."""
+    M = N = K = 256
+    torch.manual_seed(42)
+    A = torch.randint(0, 4, (M, K), dtype=torch.int8)
+    W = torch.randint(0, 2, (N, K), dtype=torch.int8)
+    qw = quantize.general_compress(W, source_bits=2)
+    C = torch.zeros((M, N), dtype=torch.int32, device=cuda)
+    tl.bitnet_158_int8xint2_prefill(M, N, K)(A.to(cuda), qw.to(cuda), C)
+    torch.cuda.synchronize()
+    ref = torch.matmul(A.float(), W.float().T).to(torch.int32)
+    assert torch.equal(C.cpu(), ref)
+
+
+@pytest.mark.parametrize("M", [1, 256, 2048])
+def test_bitlinear_config5(cuda, M):
+    """Benchmark configuration 5 at N=K=1024 (oracle-sized): ternary weights stored as w+2, per-row activation
+    scale, per-tensor weight scale, fp16 out = (acc / s_a) / s_w."""
+    N = K = 1024
+    d = workloads.bitnet(M, N, K, seed=M)
+    out = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]))(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["s_a"], cuda))
+    torch.cuda.synchronize()
+    ref = orc.ref_bitnet(d["A"], d["B"], d["s_a"], d["s_w"], "offset")
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+    acc = torch.zeros((M, N), dtype=torch.int32, device=cuda)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), acc)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(acc.cpu().numpy(), d["A"].astype(np.int64) @ d["W"].astype(np.int64).T)
+
+
+def test_bitnet_full_size_checksum(cuda):
+    """Configuration 5 at full size (M=2048, N=K=8192): exact int32 checked through column sums,
+    sum_n C[m, n] = A[m, :] . sum_n W[n, :], and a sample of entries."""
+    M, N, K = 2048, 8192, 8192
+    d = workloads.bitnet(M, N, K, seed=0)
+    acc = torch.zeros((M, N), dtype=torch.int32, device=cuda)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), acc)
+    torch.cuda.synchronize()
+    got = acc.cpu().numpy().astype(np.int64)
+    wsum = d["W"].astype(np.int64).sum(axis=0)
+    np.testing.assert_array_equal(got.sum(axis=1), d["A"].astype(np.int64) @ wsum)
+    rows, cols = np.arange(0, M, 97), np.arange(0, N, 211)
+    ref = d["A"][rows].astype(np.int64) @ d["W"][cols].astype(np.int64).T
+    np.testing.assert_array_equal(got[np.ix_(rows, cols)], ref)

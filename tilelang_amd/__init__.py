@@ -7,7 +7,18 @@ examples' kernels.  PyTorch is used for tensors and streams only.
 
 from . import quantize  # noqa: F401
 from .adapter import KernelAdapter, KernelParam  # noqa: F401
-from .kernels import dequantize_gemv, dequantize_w4, matmul_bf16_mxfp4  # noqa: F401
+from .kernels import (  # noqa: F401
+    bitlinear_int8xint2,
+    bitnet_158_int8xint2_prefill,
+    dequantize_gemv,
+    dequantize_w4,
+    matmul_bf16_mxfp4,
+    matmul_fp16_fp4,
+    matmul_int8xint4,
+    matmul_nt_int4,
+    matmul_w4_fine_grained,
+    matmul_w4a16,
+)
 from .profiler import Profiler, TensorSupplyType, do_bench  # noqa: F401
 
 __version__ = "0.1.0"

@@ -23,6 +23,14 @@ int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, 
 int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
                int scale_bias, hipStream_t stream);
 
+int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream);
+int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                int mode, int layout, hipStream_t stream);
+int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
+            int bitnet_epilogue, hipStream_t stream);
+int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
+            hipStream_t stream);
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static int check_w4_args(const char* fn, const void* B, const void* S, const void* Z, int N, int K, int group, int mode,
@@ -110,4 +118,45 @@ extern "C" int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const 
   if (!aligned16(A) || !aligned16(B) || !aligned16(C) || (Bias && !aligned16(Bias)))
     DQ_FAIL("%s: A, B, Bias and C must be 16-byte aligned", fn);
   return mxfp4_gemm(A, B, Scale, Bias, C, M, N, K, fp4_format, scale_bias, (hipStream_t)stream);
+}
+
+static int check_gemm_args(const char* fn, const void* A, const void* B, const void* C, int M, int N, int K, int kmult) {
+  if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
+  if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
+  if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
+  if (M <= 0 || N <= 0 || K <= 0) DQ_FAIL("%s: M, N, K must be positive (got %d %d %d)", fn, M, N, K);
+  if (K % kmult != 0) DQ_FAIL("%s: K=%d must be a multiple of %d", fn, K, kmult);
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C)) DQ_FAIL("%s: A, B and C must be 16-byte aligned", fn);
+  return 0;
+}
+
+extern "C" int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int N, int K, int transposed,
+                                          dq_stream_t stream) {
+  if (check_gemm_args("call_dequant_gemm_fp16_fp4", A, B, C, M, N, K, 64)) return -1;
+  return fp16_fp4_gemm(A, B, C, M, N, K, transposed, (hipStream_t)stream);
+}
+
+extern "C" int call_dequant_gemm_w4_fp16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
+                                         int M, int N, int K, int group, int mode, int layout, dq_stream_t stream) {
+  const char* fn = "call_dequant_gemm_w4_fp16";
+  if (check_gemm_args(fn, A, B, C, M, N, K, 64)) return -1;
+  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
+  return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
+}
+
+extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention,
+                                   const void* s_a, float s_w, int out_kind, dq_stream_t stream) {
+  const char* fn = "call_gemm_int8xint2";
+  if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
+  if (convention < I2_UNSIGNED || convention > I2_TWOS) DQ_FAIL("%s: unknown code convention %d", fn, convention);
+  if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
+  if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);
+  if (out_kind == 1 && !(s_w != 0.f)) DQ_FAIL("%s: s_w must be non-zero", fn);
+  return i2_gemm(A, B, C, M, N, K, convention, s_a, s_w, out_kind, (hipStream_t)stream);
+}
+
+extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed,
+                                   int a_packed, int transposed, dq_stream_t stream) {
+  if (check_gemm_args("call_gemm_int8xint4", A, B, C, M, N, K, 128)) return -1;
+  return i4_gemm(A, B, C, M, N, K, is_signed, a_packed, transposed, (hipStream_t)stream);
 }

@@ -252,7 +252,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int row = 8 * (i >> 2) + 4 * g + (i & 3);
-        slab[row * kSlabStride + nb * 32 + r] = __builtin_bit_cast(uint32_t, acc[mb][nb][i]);
+        // copy the element out first: bit-casting the vector-element expression itself is unreliable
+        const decltype(acc[0][0][0] + 0) elem = acc[mb][nb][i];
+        uint32_t bits;
+        __builtin_memcpy(&bits, &elem, 4);
+        slab[row * kSlabStride + nb * 32 + r] = bits;
       }
     __builtin_amdgcn_wave_barrier();
     if constexpr (!P::kTransposed) {

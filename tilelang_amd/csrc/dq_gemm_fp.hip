@@ -1,0 +1,210 @@
+// 16-bit operand policies of the LDS-staged dequantize GEMM (dq_gemm_core.h): MXFP4 x bf16,
+// "simple" fp4 x fp16 and uint4 x fp16.
+#include "dq_gemm_core.h"
+
+namespace dq {
+
+namespace {
+
+using gemm::Params;
+
+// exponent byte -> fp32 power of two 2^(e + off - 127); only the exponent field matters to the
+// conversion instruction.  Clamped to [2^-127, 2^127].
+__device__ __forceinline__ float scale_to_f32(int e, int off) {
+  int ex = e + off;
+  ex = ex < 0 ? 0 : (ex > 254 ? 254 : ex);
+  uint32_t bits = (uint32_t)ex << 23;
+  bits = bits < 0x00400000u ? 0x00400000u : bits;  // exponent 0 means 2^-127 (a subnormal)
+  return __builtin_bit_cast(float, bits);
+}
+
+// eight e2m1 nibbles (natural k order) times a power of two -> bf16, exact
+__device__ __forceinline__ bf16x8_t cvt_e2m1x8(uint32_t w, float scale) {
+  const bf16x2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 0);
+  const bf16x2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 1);
+  const bf16x2_t p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 2);
+  const bf16x2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 3);
+  bf16x8_t o;
+  o[0] = p0[0]; o[1] = p0[1]; o[2] = p1[0]; o[3] = p1[1];
+  o[4] = p2[0]; o[5] = p2[1]; o[6] = p3[0]; o[7] = p3[1];
+  return o;
+}
+
+// "twiddled" 16-bit units -> plain e2m1 nibbles (natural order), both units of the dword at once.
+// unit = (byte[2j] << 8) | byte[2j+1]; code p of a unit is (s, E1, E0, m) =
+// p0 (15, 8, 7, 6), p1 (12, 5, 4, 3), p2 (9, 2, 1, 0), p3 (14, 11, 10, 13)
+// (examples/dequantize_gemm/dequantize_utils.py:33-45).
+__device__ __forceinline__ uint32_t twiddled_to_plain(uint32_t w) {
+  const uint32_t x = __builtin_amdgcn_perm(w, w, 0x02030001u);  // swap the bytes of each half
+  const uint32_t c0 = ((x >> 12) & 0x00080008u) | ((x >> 6) & 0x00070007u);
+  const uint32_t c1 = ((x >> 9) & 0x00080008u) | ((x >> 3) & 0x00070007u);
+  const uint32_t c2 = ((x >> 6) & 0x00080008u) | (x & 0x00070007u);
+  const uint32_t c3 = ((x >> 11) & 0x00080008u) | ((x >> 9) & 0x00060006u) | ((x >> 13) & 0x00010001u);
+  return c0 | (c1 << 4) | (c2 << 8) | (c3 << 12);
+}
+
+// "simple" fp4: 16-bit pattern (s << 15) | ((E + bias) << MB) | (m << (MB - 1)) for every E, two
+// nibbles of one byte per dword (natural k order).  `expadd` carries the bias (and the block
+// exponent) already shifted into both halves.
+template <int MANT_BITS>
+__device__ __forceinline__ uint4_t simple_fp4x8(uint32_t w, uint32_t expadd) {
+  uint4_t r;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const uint32_t lo = (w >> (8 * b)) & 0xFu;
+    const uint32_t hi = (w >> (8 * b + 4)) & 0xFu;
+    const uint32_t p = lo | (hi << 16);
+    r[b] = (((p & 0x00080008u) << 12) | ((p & 0x00070007u) << (MANT_BITS - 1))) + expadd;
+  }
+  return r;
+}
+
+struct Bf16Mfma {
+  static constexpr int kKPerBlock = 64;
+  using frag_t = bf16x8_t;
+  using acc_t = float16_t;
+  __device__ static __forceinline__ acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct F16Mfma {
+  static constexpr int kKPerBlock = 64;
+  using frag_t = half8_t;
+  using acc_t = float16_t;
+  __device__ static __forceinline__ acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// ---- MXFP4 x bf16 -------------------------------------------------------------------------------
+// Scale[N, K/32] uint8, p.p0 = 127 - scale_bias.  Lane group g owns one 32-k scale block per tile.
+template <int FMT, bool HAS_BIAS>
+struct MxPolicy : Bf16Mfma, gemm::PlainA {
+  static constexpr int kBRowBytes = 32;
+  static constexpr bool kTransposed = false;
+  using out_t = bf16_t;
+  using ScaleRaw = int;
+  struct Scale { float f; uint32_t add; };
+  __device__ static __forceinline__ ScaleRaw fetch_scale(const Params& p, int row, int kb, int g) {
+    return ((const uint8_t*)p.S)[(size_t)row * (p.K >> 5) + kb * 2 + g];
+  }
+  __device__ static __forceinline__ Scale prep_scale(ScaleRaw e, const Params& p) {
+    Scale s;
+    if constexpr (FMT == FP4_SIMPLE) {
+      int ex = 126 + e + p.p0 - 127;
+      ex = ex < 0 ? 0 : (ex > 252 ? 252 : ex);  // E adds up to 3
+      s.add = ((uint32_t)ex << 7) * 0x00010001u;
+      s.f = 0.f;
+    } else {
+      s.f = scale_to_f32(e, p.p0);
+      s.add = 0;
+    }
+    return s;
+  }
+  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale& s) {
+    if constexpr (FMT == FP4_E2M1) return cvt_e2m1x8(w[j], s.f);
+    else if constexpr (FMT == FP4_TWIDDLING) return cvt_e2m1x8(twiddled_to_plain(w[j]), s.f);
+    else return __builtin_bit_cast(frag_t, simple_fp4x8<7>(w[j], s.add));
+  }
+  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params& p, int m, int n) {
+    float v = __builtin_bit_cast(float, raw);
+    // reference: C = bf16(float(acc) + float(Bias))
+    if constexpr (HAS_BIAS) v += (float)((const bf16_t*)p.Bias)[(size_t)m * p.N + n];
+    return (bf16_t)v;
+  }
+};
+
+// ---- "simple" fp4 x fp16 (examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py) ------------
+template <bool TRANSPOSED>
+struct Fp16Fp4Policy : F16Mfma, gemm::PlainA, gemm::NoScale {
+  static constexpr int kBRowBytes = 32;
+  static constexpr bool kTransposed = TRANSPOSED;
+  using out_t = half_t;
+  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
+    return __builtin_bit_cast(frag_t, simple_fp4x8<10>(w[j], 0x38003800u));  // (E + 14) << 10
+  }
+  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params&, int, int) {
+    return (half_t)__builtin_bit_cast(float, raw);
+  }
+};
+
+// ---- uint4 x fp16 with the integer decoders (fine-grained example, W4A16 at large M) ---------------
+// Scale / Zeros fp16 [N, K/group], p.p0 = log2(group) (31 when group == K), p.p1 = K / group.
+template <int MODE, bool INTERLEAVED>
+struct W4F16Policy : F16Mfma {
+  static constexpr int kBRowBytes = 32;
+  static constexpr bool kTransposed = false;
+  static constexpr bool kAPacked = false;
+  using out_t = half_t;
+  struct ScaleRaw { half_t s, z; };
+  using Scale = ScaleRaw;
+  // the plain-layout decoder emits nibble pairs (e, e+4): activations get the same order
+  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : permute_k8_16bit(v); }
+  __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
+  __device__ static __forceinline__ ScaleRaw fetch_scale(const Params& p, int row, int kb, int g) {
+    ScaleRaw r{(half_t)1.f, (half_t)0.f};
+    const size_t idx = (size_t)row * p.p1 + ((kb * 64 + g * 32) >> p.p0);
+    if constexpr (MODE >= W4_SCALE) r.s = ((const half_t*)p.S)[idx];
+    if constexpr (MODE >= W4_ZEROS_ORIGINAL) r.z = ((const half_t*)p.Z)[idx];
+    return r;
+  }
+  __device__ static __forceinline__ Scale prep_scale(ScaleRaw r, const Params&) { return r; }
+  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale& s) {
+    return decode_w4<MODE>(w[j], s.s, s.z);
+  }
+  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params&, int, int) {
+    return (half_t)__builtin_bit_cast(float, raw);
+  }
+};
+
+}  // namespace
+
+int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
+               int scale_bias, hipStream_t stream) {
+  Params p = gemm::make_params(A, B, S, nullptr, Bias, C, M, N, K);
+  p.p0 = 127 - scale_bias;
+#define DQ_MX(FMT_)                                                        \
+  do {                                                                     \
+    if (Bias) return gemm::launch<MxPolicy<FMT_, true>>(p, stream);        \
+    return gemm::launch<MxPolicy<FMT_, false>>(p, stream);                 \
+  } while (0)
+  switch (fmt) {
+    case FP4_E2M1: DQ_MX(FP4_E2M1);
+    case FP4_SIMPLE: DQ_MX(FP4_SIMPLE);
+    case FP4_TWIDDLING: DQ_MX(FP4_TWIDDLING);
+    default: DQ_FAIL("mxfp4 gemm: unknown weight format %d", fmt);
+  }
+#undef DQ_MX
+}
+
+int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream) {
+  Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
+  if (transposed) return gemm::launch<Fp16Fp4Policy<true>>(p, stream);
+  return gemm::launch<Fp16Fp4Policy<false>>(p, stream);
+}
+
+int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                int mode, int layout, hipStream_t stream) {
+  Params p = gemm::make_params(A, B, S, Z, nullptr, C, M, N, K);
+  p.p0 = (group == K) ? 31 : (31 - __builtin_clz(group));
+  p.p1 = K / group;
+#define DQ_W4(MODE_)                                                                        \
+  do {                                                                                      \
+    if (layout == LAYOUT_PLAIN) return gemm::launch<W4F16Policy<MODE_, false>>(p, stream);  \
+    return gemm::launch<W4F16Policy<MODE_, true>>(p, stream);                               \
+  } while (0)
+  switch (mode) {
+    case W4_UNSIGNED: DQ_W4(W4_UNSIGNED);
+    case W4_SIGNED: DQ_W4(W4_SIGNED);
+    case W4_OFFSET8: DQ_W4(W4_OFFSET8);
+    case W4_SCALE: DQ_W4(W4_SCALE);
+    case W4_USCALE: DQ_W4(W4_USCALE);
+    case W4_ZEROS_ORIGINAL: DQ_W4(W4_ZEROS_ORIGINAL);
+    case W4_ZEROS_RESCALE: DQ_W4(W4_ZEROS_RESCALE);
+    default: DQ_FAIL("w4 fp16 gemm: unknown mode %d", mode);
+  }
+#undef DQ_W4
+}
+
+}  // namespace dq

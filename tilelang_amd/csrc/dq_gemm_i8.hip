@@ -1,0 +1,158 @@
+// int8-MFMA policies of the LDS-staged dequantize GEMM (dq_gemm_core.h): BitNet W2A8
+// (int8 x 2-bit), W4A8 (int8 x int4), int4 x int4 and int8 x uint4.  Accumulation is int32 and
+// exact; the epilogue is either the raw int32 (optionally transposed) or BitLinear's
+// out = (float(acc) / s_a[m]) / s_w -> fp16.
+#include "dq_gemm_core.h"
+
+namespace dq {
+
+namespace {
+
+using gemm::Params;
+
+struct I8Mfma {
+  static constexpr int kKPerBlock = 128;
+  using frag_t = int4_t;
+  using acc_t = int16_t_;
+  __device__ static __forceinline__ acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+
+// 16 consecutive int8 (a0..a15) -> dword i = (a[i], a[4+i], a[8+i], a[12+i]): the element order
+// of the 2-bit decoder, whose dword i holds the codes at bit 2i of each packed byte.
+__device__ __forceinline__ uint4_t transpose4x4_bytes(uint4_t d) {
+  const uint32_t t01_lo = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u);  // d0.b0 d1.b0 d0.b1 d1.b1
+  const uint32_t t01_hi = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);  // d0.b2 d1.b2 d0.b3 d1.b3
+  const uint32_t t23_lo = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+  const uint32_t t23_hi = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+  uint4_t o;
+  o[0] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x05040100u);
+  o[1] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x07060302u);
+  o[2] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x05040100u);
+  o[3] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x07060302u);
+  return o;
+}
+
+// 16 consecutive int8 -> (a0 a2 a4 a6) (a1 a3 a5 a7) (a8 a10 a12 a14) (a9 a11 a13 a15): the element
+// order of the nibble decoder, whose dwords hold the even / odd nibbles of one packed word.
+__device__ __forceinline__ uint4_t split_even_odd_bytes(uint4_t d) {
+  uint4_t o;
+  o[0] = __builtin_amdgcn_perm(d[1], d[0], 0x06040200u);
+  o[1] = __builtin_amdgcn_perm(d[1], d[0], 0x07050301u);
+  o[2] = __builtin_amdgcn_perm(d[3], d[2], 0x06040200u);
+  o[3] = __builtin_amdgcn_perm(d[3], d[2], 0x07050301u);
+  return o;
+}
+
+// ---- epilogues --------------------------------------------------------------------------------------
+template <int SHIFT, bool TRANSPOSED>
+struct Int32Out {
+  static constexpr bool kTransposed = TRANSPOSED;
+  using out_t = int32_t;
+  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params&, int, int) {
+    return (int32_t)raw >> SHIFT;  // operands were decoded as 16 x value: exact
+  }
+};
+
+// BitLinear: out = (float(acc) / s_a[m]) / s_w -> fp16, two fp32 divides in that order
+// (examples/bitnet-1.58b/utils_quant.py:165-170).  p.S = s_a (float[M]), p.f0 = s_w.
+struct BitnetOut {
+  static constexpr bool kTransposed = false;
+  using out_t = half_t;
+  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params& p, int m, int) {
+    float v = (float)(int32_t)raw;
+    v = v / ((const float*)p.S)[m];
+    v = v / p.f0;
+    return (half_t)v;
+  }
+};
+
+// ---- int8 x 2-bit ---------------------------------------------------------------------------------
+// packed byte j of a row holds codes 4j..4j+3 at bits 0, 2, 4, 6.
+template <int CONV, class EPI>
+struct I2Policy : I8Mfma, gemm::NoScale, EPI {
+  static constexpr int kBRowBytes = 32;
+  static constexpr bool kAPacked = false;
+  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return transpose4x4_bytes(v); }
+  __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
+  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
+    frag_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint32_t d = (w[j] >> (2 * i)) & 0x03030303u;
+      if constexpr (CONV == I2_OFFSET) {
+        // per byte c - 2 without a borrow between bytes: ((c | 0x80) - 2) ^ 0x80
+        d = ((d | 0x80808080u) - 0x02020202u) ^ 0x80808080u;
+      } else if constexpr (CONV == I2_TWOS) {
+        // sext2(c) = (c ^ 2) - 2
+        d = (((d ^ 0x02020202u) | 0x80808080u) - 0x02020202u) ^ 0x80808080u;
+      }
+      o[i] = (int)d;
+    }
+    return o;
+  }
+};
+
+// ---- int8 x 4-bit ---------------------------------------------------------------------------------
+// SIGNED: nibbles are two's complement; they are decoded as 16 x value (nibble in the top of the
+// byte) and the accumulator is shifted back in the epilogue.  A_PACKED: A is packed int4 too and
+// is expanded the same way while it is staged, so both operands carry the factor 16.
+template <bool SIGNED, bool A_PACKED, class EPI>
+struct I4Policy : I8Mfma, gemm::NoScale, EPI {
+  static constexpr int kBRowBytes = 64;
+  static constexpr bool kAPacked = A_PACKED;
+  __device__ static __forceinline__ uint32_t even(uint32_t w) {
+    return SIGNED ? ((w << 4) & 0xF0F0F0F0u) : (w & 0x0F0F0F0Fu);
+  }
+  __device__ static __forceinline__ uint32_t odd(uint32_t w) {
+    return SIGNED ? (w & 0xF0F0F0F0u) : ((w >> 4) & 0x0F0F0F0Fu);
+  }
+  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return split_even_odd_bytes(v); }
+  __device__ static __forceinline__ void expand_a(uint4_t v, uint4_t& lo, uint4_t& hi) {
+    lo = uint4_t{even(v[0]), odd(v[0]), even(v[1]), odd(v[1])};
+    hi = uint4_t{even(v[2]), odd(v[2]), even(v[3]), odd(v[3])};
+  }
+  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
+    const uint32_t w0 = w[2 * j], w1 = w[2 * j + 1];
+    return frag_t{(int)even(w0), (int)odd(w0), (int)even(w1), (int)odd(w1)};
+  }
+};
+
+}  // namespace
+
+int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
+            int bitnet_epilogue, hipStream_t stream) {
+  Params p = gemm::make_params(A, B, s_a, nullptr, nullptr, C, M, N, K);
+  p.f0 = s_w;
+#define DQ_I2(CONV_)                                                                       \
+  do {                                                                                     \
+    if (bitnet_epilogue) return gemm::launch<I2Policy<CONV_, BitnetOut>>(p, stream);       \
+    return gemm::launch<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);                   \
+  } while (0)
+  switch (convention) {
+    case I2_UNSIGNED: DQ_I2(I2_UNSIGNED);
+    case I2_OFFSET: DQ_I2(I2_OFFSET);
+    case I2_TWOS: DQ_I2(I2_TWOS);
+    default: DQ_FAIL("int2 gemm: unknown code convention %d", convention);
+  }
+#undef DQ_I2
+}
+
+int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
+            hipStream_t stream) {
+  Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
+  if (a_packed) {
+    if (!is_signed) DQ_FAIL("int4 gemm: packed A is built for signed int4 only");
+    if (transposed) return gemm::launch<I4Policy<true, true, Int32Out<8, true>>>(p, stream);
+    return gemm::launch<I4Policy<true, true, Int32Out<8, false>>>(p, stream);
+  }
+  if (is_signed) {
+    if (transposed) return gemm::launch<I4Policy<true, false, Int32Out<4, true>>>(p, stream);
+    return gemm::launch<I4Policy<true, false, Int32Out<4, false>>>(p, stream);
+  }
+  if (transposed) return gemm::launch<I4Policy<false, false, Int32Out<0, true>>>(p, stream);
+  return gemm::launch<I4Policy<false, false, Int32Out<0, false>>>(p, stream);
+}
+
+}  // namespace dq

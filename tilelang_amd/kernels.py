@@ -233,3 +233,224 @@ def matmul_bf16_mxfp4(
         return lib.call_dequant_gemm_bf16_mxfp4(ptrs[0], ptrs[1], ptrs[2], bias, ptrs[4], M, N, K, scale_size, fmt, scale_bias, stream)
 
     return KernelAdapter("matmul_bf16_mxfp4", params, [-1], launch, _lib.last_error)
+
+
+def matmul_fp16_fp4(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="float16",
+    out_dtype="float16",
+    accum_dtype="float32",
+    num_bits: int = 4,
+    block_M: int = 128,
+    block_N: int = 128,
+    block_K: int = 128,
+    num_stages: int = 2,
+    threads: int = 256,
+    split: int = 1,
+    transposed_output: bool = True,
+) -> KernelAdapter:
+    """fp16 x "simple" fp4 GEMM: ``Ct[N,M] = (A[M,K] @ fp4_to_f16(B[N,K/2]).T).T``.
+
+    Same arguments as ``matmul`` of examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:110-125;
+    ``Ct = kernel(A, B)`` (``out_idx=[2]``).  ``split`` is accepted: the K reduction stays inside one
+    workgroup in fp32 (the example's split variant sums ``split`` partial tiles in a second kernel), so the
+    result does not depend on it.  ``transposed_output=False`` gives ``C[M,N]``.
+    """
+    if num_bits != 4:
+        raise ValueError("matmul_fp16_fp4: num_bits must be 4")
+    if _dtype(in_dtype) != torch.float16 or _dtype(out_dtype) != torch.float16:
+        raise ValueError("matmul_fp16_fp4: in_dtype and out_dtype must be float16")
+    if K % 64 != 0:
+        raise ValueError(f"matmul_fp16_fp4: K={K} must be a multiple of 64")
+    out_shape = (N, M) if transposed_output else (M, N)
+    params = [
+        KernelParam("A", torch.float16, (M, K)),
+        KernelParam("B", torch.uint8, (N, K // 2), packed=True),
+        KernelParam("Ct" if transposed_output else "C", torch.float16, out_shape),
+    ]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_dequant_gemm_fp16_fp4(ptrs[0], ptrs[1], ptrs[2], M, N, K, int(transposed_output), stream)
+
+    return KernelAdapter("matmul_fp16_fp4", params, [2], launch, _lib.last_error)
+
+
+def matmul_w4_fine_grained(
+    M: int,
+    N: int,
+    K: int,
+    block_M: int = 128,
+    block_N: int = 128,
+    block_K: int = 32,
+    in_dtype="float16",
+    out_dtype="float16",
+    accum_dtype="float32",
+    num_stages: int = 3,
+    threads: int = 128,
+    num_bits: int = 4,
+) -> KernelAdapter:
+    """Weight-only uint4 GEMM ``C[M,N] = A[M,K] @ q(B[N,K/2]).T`` with unsigned nibbles.
+
+    Same arguments as ``matmul`` of examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:16-29;
+    ``C = kernel(A, B)``.  ``in_dtype="float16"`` gives fp16 out (fp32 accumulation);
+    ``in_dtype="int8"`` gives exact int32 out.
+    """
+    if num_bits != 4:
+        raise ValueError("matmul_w4_fine_grained: num_bits must be 4")
+    it = _dtype(in_dtype)
+    if it == torch.float16:
+        if K % 64 != 0:
+            raise ValueError(f"matmul_w4_fine_grained: K={K} must be a multiple of 64")
+        params = [KernelParam("A", torch.float16, (M, K)), KernelParam("B", torch.int8, (N, K // 2), packed=True),
+                  KernelParam("C", torch.float16, (M, N))]
+
+        def launch(ptrs, stream):
+            return _lib.get_library().call_dequant_gemm_w4_fp16(ptrs[0], ptrs[1], None, None, ptrs[2], M, N, K, K, W4_UNSIGNED,
+                                                                LAYOUT_PLAIN, stream)
+    elif it == torch.int8:
+        if K % 128 != 0:
+            raise ValueError(f"matmul_w4_fine_grained: K={K} must be a multiple of 128 for int8")
+        params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 2), packed=True),
+                  KernelParam("C", torch.int32, (M, N))]
+
+        def launch(ptrs, stream):
+            return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, 0, 0, 0, stream)
+    else:
+        raise ValueError("matmul_w4_fine_grained: in_dtype must be float16 or int8")
+    return KernelAdapter("matmul_w4_fine_grained", params, [2], launch, _lib.last_error)
+
+
+def matmul_w4a16(M: int, N: int, K: int, group_size: int = -1, source_format: str = "int", fast_decoding: bool = False,
+                 with_scaling: bool = True, with_zeros: bool = False, zeros_mode: str = "original",
+                 storage_dtype="int8") -> KernelAdapter:
+    """W4A16 GEMM for any M through the 256x256 MFMA kernel (tile-exact fp16 dequantisation):
+    ``kernel(A, B[, Scale[, Zeros]], C)``, same decode options as :func:`dequantize_gemv`."""
+    if group_size == -1:
+        group_size = K
+    if K % 64 != 0:
+        raise ValueError(f"matmul_w4a16: K={K} must be a multiple of 64")
+    mode = _w4_mode(source_format, fast_decoding, with_scaling, with_zeros, zeros_mode)
+    layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
+    groups = K // group_size
+    params = [KernelParam("A", torch.float16, (M, K)), KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True)]
+    if with_scaling:
+        params.append(KernelParam("Scale", torch.float16, (N, groups)))
+    if with_zeros:
+        params.append(KernelParam("Zeros", torch.float16, (N, groups)))
+    params.append(KernelParam("C", torch.float16, (M, N)))
+
+    def launch(ptrs, stream):
+        s = ptrs[2] if with_scaling else None
+        z = ptrs[3] if with_zeros else None
+        return _lib.get_library().call_dequant_gemm_w4_fp16(ptrs[0], ptrs[1], s, z, ptrs[-1], M, N, K, group_size, mode, layout, stream)
+
+    return KernelAdapter("matmul_w4a16", params, [], launch, _lib.last_error)
+
+
+def matmul_int8xint4(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="int8",
+    out_dtype="int32",
+    accum_dtype="int32",
+    num_bits: int = 4,
+    block_M: int = 32,
+    block_N: int = 32,
+    block_K: int = 128,
+    num_stages: int = 1,
+    threads: int = 128,
+) -> KernelAdapter:
+    """W4A8: ``Ct[N,M] int32 = (A[M,K] int8 @ sext4(B[N,K/2]).T).T``, exact.
+
+    Same arguments as ``matmul_int8xint4`` of examples/dequantize_gemm/example_dequant_gemm_w4a8.py:87-100;
+    ``Ct = kernel(A, B)`` (``out_idx=[2]``).
+    """
+    if num_bits != 4 or _dtype(in_dtype) != torch.int8 or _dtype(out_dtype) != torch.int32:
+        raise ValueError("matmul_int8xint4: int8 activations, 4-bit weights and int32 output only")
+    if K % 128 != 0:
+        raise ValueError(f"matmul_int8xint4: K={K} must be a multiple of 128")
+    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.uint8, (N, K // 2), packed=True),
+              KernelParam("Ct", torch.int32, (N, M))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, 1, 0, 1, stream)
+
+    return KernelAdapter("matmul_int8xint4", params, [2], launch, _lib.last_error)
+
+
+def matmul_nt_int4(M: int, N: int, K: int, block_M: int = 128, block_N: int = 128, block_K: int = 64, threads: int = 128) -> KernelAdapter:
+    """int4 x int4: ``C[M,N] int32 = sext4(A[M,K/2]) @ sext4(B[N,K/2]).T``, both operands packed two per byte.
+
+    Same arguments as ``matmul_nt_int4`` of examples/gemm_int4/example_tilelang_gemm_int4.py:17-38;
+    ``C = kernel(A_packed, B_packed)`` (``out_idx=-1``).
+    """
+    if K % 128 != 0:
+        raise ValueError(f"matmul_nt_int4: K={K} must be a multiple of 128")
+    params = [KernelParam("A", torch.int8, (M, K // 2), packed=True), KernelParam("B", torch.int8, (N, K // 2), packed=True),
+              KernelParam("C", torch.int32, (M, N))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, 1, 1, 0, stream)
+
+    return KernelAdapter("matmul_nt_int4", params, [-1], launch, _lib.last_error)
+
+
+I2_UNSIGNED, I2_OFFSET, I2_TWOS = 0, 1, 2
+_I2_CONVENTIONS = {"unsigned": I2_UNSIGNED, "offset": I2_OFFSET, "twos": I2_TWOS}
+
+
+def bitnet_158_int8xint2_prefill(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="int8",
+    out_dtype="int32",
+    accum_dtype="int32",
+    fast_decoding: bool = True,
+    block_row_warps: int = 2,
+    block_col_warps: int = 2,
+    warp_row_tiles: int = 32,
+    warp_col_tiles: int = 32,
+    chunk: int = 64,
+    convention: str = "unsigned",
+) -> KernelAdapter:
+    """BitNet W2A8 GEMM: ``C[M,N] int32 = A[M,K] int8 @ decode(B[N,K/4]).T``, exact; ``kernel(A, B, C)``.
+
+    Same arguments as ``bitnet_158_int8xint2_prefill`` of examples/bitnet-1.58b/kernel_benchmark/
+    tilelang_bitnet_158_int8xint2_prefill.py:72-85.  B is the plain packing (``general_compress(W, 2)``,
+    no ``interleave_weight``).  ``convention``: ``"unsigned"`` (what the example's kernel decodes),
+    ``"offset"`` (``w = c - 2``, ternary weights stored as ``w + 2``) or ``"twos"``.
+    """
+    if _dtype(in_dtype) != torch.int8 or _dtype(out_dtype) != torch.int32:
+        raise ValueError("bitnet_158_int8xint2_prefill: int8 in, int32 out")
+    if K % 128 != 0:
+        raise ValueError(f"bitnet_158_int8xint2_prefill: K={K} must be a multiple of 128")
+    conv = _I2_CONVENTIONS[convention]
+    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 4), packed=True),
+              KernelParam("C", torch.int32, (M, N))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, None, 1.0, 0, stream)
+
+    return KernelAdapter("bitnet_158_int8xint2_prefill", params, [], launch, _lib.last_error)
+
+
+def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "offset") -> KernelAdapter:
+    """BitLinear forward after activation quantisation: ``out[M,N] fp16 = ((A int8 @ W.T) / s_a[m]) / s_w``.
+
+    The matmul plus ``post_quant_process`` of examples/bitnet-1.58b/utils_quant.py:165-170,199-209 in one
+    kernel.  ``out = kernel(A, B, s_a)`` with ``s_a`` fp32 ``[M]`` (the per-row activation scale).
+    """
+    if K % 128 != 0:
+        raise ValueError(f"bitlinear_int8xint2: K={K} must be a multiple of 128")
+    conv = _I2_CONVENTIONS[convention]
+    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 4), packed=True),
+              KernelParam("s_a", torch.float32, (M,)), KernelParam("out", torch.float16, (M, N))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv, ptrs[2], float(s_w), 1, stream)
+
+    return KernelAdapter("bitlinear_int8xint2", params, [-1], launch, _lib.last_error)
