@@ -169,3 +169,30 @@ def test_bitnet_full_size_checksum(cuda):
     rows, cols = np.arange(0, M, 97), np.arange(0, N, 211)
     ref = d["A"][rows].astype(np.int64) @ d["W"][cols].astype(np.int64).T
     np.testing.assert_array_equal(got[np.ix_(rows, cols)], ref)
+
+
+@pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 256), (1, 1000, 8192), (2, 130, 4096), (3, 64, 2048), (4, 4096, 8192), (1, 96, 16384), (2, 40, 16384)])
+def test_bitnet_decode_gemv_exact(cuda, convention, M, N, K):
+    """tilelang_bitnet_158_int8xint2_decode.py:237-258 (1x256x256) generalised: all codes, int8 range, exact."""
+    rng = np.random.default_rng(M * 7 + K)
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    tl.bitnet_158_int8xint2_decode(M, N, K, convention=convention)(_dev(A, cuda), _dev(B, cuda).view(torch.int8), C)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
+
+
+def test_bitnet_decode_full_size(cuda):
+    """Configuration 5, M=1, N=K=8192: exact against the integer oracle, plus the fp16 BitLinear epilogue."""
+    M, N, K = 1, 8192, 8192
+    d = workloads.bitnet(M, N, K, seed=1)
+    C = torch.zeros((M, N), dtype=torch.int32, device=cuda)
+    tl.bitnet_158_int8xint2_decode(M, N, K, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), C)
+    out = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]))(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["s_a"], cuda))
+    torch.cuda.synchronize()
+    ref = d["A"].astype(np.int64) @ d["W"].astype(np.int64).T
+    np.testing.assert_array_equal(C.cpu().numpy(), ref)
+    np.testing.assert_allclose(out.float().cpu().numpy(), orc.post_quant_process(ref, d["s_a"].reshape(-1, 1), d["s_w"]).astype(np.float32),
+                               rtol=RTOL, atol=ATOL)

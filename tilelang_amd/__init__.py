@@ -9,6 +9,7 @@ from . import quantize  # noqa: F401
 from .adapter import KernelAdapter, KernelParam  # noqa: F401
 from .kernels import (  # noqa: F401
     bitlinear_int8xint2,
+    bitnet_158_int8xint2_decode,
     bitnet_158_int8xint2_prefill,
     dequantize_gemv,
     dequantize_w4,

@@ -28,6 +28,8 @@ int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void
                 int mode, int layout, hipStream_t stream);
 int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
             int bitnet_epilogue, hipStream_t stream);
+int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
+            int out_kind, hipStream_t stream);
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
             hipStream_t stream);
 
@@ -81,6 +83,8 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
   if (K % 128 != 0) DQ_FAIL("%s: K=%d must be a multiple of 128", fn, K);
   if (!aligned16(A) || !aligned16(C)) DQ_FAIL("%s: A and C must be 16-byte aligned", fn);
+  // prefill-sized M: the 256 x 256 MFMA GEMM (same tile-exact decoders)
+  if (variant < 0 && M > 64) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread
   // (r = 0: its own choice).  0..99: a configuration of the MFMA kernel.
   if (variant < 0 || variant >= 100) {
@@ -152,6 +156,10 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
   if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);
   if (out_kind == 1 && !(s_w != 0.f)) DQ_FAIL("%s: s_w must be non-zero", fn);
+  if (M <= 4) {  // decode: the streaming dot4 kernel
+    const int rc = i2_gemv(A, B, C, M, N, K, convention, s_a, s_w, out_kind, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
   return i2_gemm(A, B, C, M, N, K, convention, s_a, s_w, out_kind, (hipStream_t)stream);
 }
 

@@ -19,32 +19,6 @@ struct I8Mfma {
   }
 };
 
-// 16 consecutive int8 (a0..a15) -> dword i = (a[i], a[4+i], a[8+i], a[12+i]): the element order
-// of the 2-bit decoder, whose dword i holds the codes at bit 2i of each packed byte.
-__device__ __forceinline__ uint4_t transpose4x4_bytes(uint4_t d) {
-  const uint32_t t01_lo = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u);  // d0.b0 d1.b0 d0.b1 d1.b1
-  const uint32_t t01_hi = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);  // d0.b2 d1.b2 d0.b3 d1.b3
-  const uint32_t t23_lo = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
-  const uint32_t t23_hi = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
-  uint4_t o;
-  o[0] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x05040100u);
-  o[1] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x07060302u);
-  o[2] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x05040100u);
-  o[3] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x07060302u);
-  return o;
-}
-
-// 16 consecutive int8 -> (a0 a2 a4 a6) (a1 a3 a5 a7) (a8 a10 a12 a14) (a9 a11 a13 a15): the element
-// order of the nibble decoder, whose dwords hold the even / odd nibbles of one packed word.
-__device__ __forceinline__ uint4_t split_even_odd_bytes(uint4_t d) {
-  uint4_t o;
-  o[0] = __builtin_amdgcn_perm(d[1], d[0], 0x06040200u);
-  o[1] = __builtin_amdgcn_perm(d[1], d[0], 0x07050301u);
-  o[2] = __builtin_amdgcn_perm(d[3], d[2], 0x06040200u);
-  o[3] = __builtin_amdgcn_perm(d[3], d[2], 0x07050301u);
-  return o;
-}
-
 // ---- epilogues --------------------------------------------------------------------------------------
 template <int SHIFT, bool TRANSPOSED>
 struct Int32Out {

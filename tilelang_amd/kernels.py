@@ -454,3 +454,27 @@ def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "o
         return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv, ptrs[2], float(s_w), 1, stream)
 
     return KernelAdapter("bitlinear_int8xint2", params, [-1], launch, _lib.last_error)
+
+
+def bitnet_158_int8xint2_decode(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="int8",
+    out_dtype="int32",
+    accum_dtype="int32",
+    fast_decoding: bool = True,
+    n_partition: int = 4,
+    reduce_thread: int = 32,
+    convention: str = "unsigned",
+) -> KernelAdapter:
+    """BitNet W2A8 decode GEMV: ``C[M,N] int32 = A[M,K] int8 @ decode(B[N,K/4]).T``, exact; ``kernel(A, B, C)``.
+
+    Same arguments as ``bitnet_158_int8xint2_decode`` of examples/bitnet-1.58b/kernel_benchmark/
+    tilelang_bitnet_158_int8xint2_decode.py:66-76.  M <= 4 runs the streaming dot4 kernel, larger M the
+    MFMA GEMM.  B is the plain packing (no ``interleave_weight``); ``convention`` as in
+    :func:`bitnet_158_int8xint2_prefill`.
+    """
+    k = bitnet_158_int8xint2_prefill(M, N, K, in_dtype, out_dtype, accum_dtype, fast_decoding, convention=convention)
+    k.name = "bitnet_158_int8xint2_decode"
+    return k
