@@ -10,8 +10,9 @@
 //   * block tile 256 x 256 x BK (BK = 128 bytes of A per row: 64 x 16-bit or 128 x int8), 4 waves
 //     as 2 x 2, 128 x 128 per wave = 4 x 4 MFMA 32x32 accumulators (256 registers per lane);
 //   * A (transformed by the policy, 16 bytes at a time, on its way through registers) and the
-//     PACKED B tile are double-buffered in LDS; the next tile travels global -> registers while
-//     the current one is multiplied;
+//     PACKED B tile live in three LDS stages; tile kb+3 travels global -> registers and tile kb+2
+//     registers -> LDS while tile kb is multiplied, and the operands of every MFMA step are
+//     fetched (and decoded) one step ahead, across tile boundaries too;
 //   * B is never materialised in memory at the compute type: lane (g, c) of a wave reads the
 //     packed bytes of the half-tile k in [g*BK/2, (g+1)*BK/2) of its weight row and decodes them
 //     in registers straight into MFMA operands.  The contraction index of MFMA step j is labelled
@@ -63,6 +64,91 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tm = first_m + in_band % gm;
   tn = in_band / gm;
 }
+
+// Epilogue shared by both kernel variants (a macro: it uses the kernel's locals).
+// acc[mb][nb][i] = C[m0 + wm*128 + mb*32 + 8*(i/4) + 4*g + i%4][n0 + wn*128 + nb*32 + r].  Staged through
+// LDS (every tile is consumed: the loop ended with a barrier) so that each lane stores 16 contiguous
+// bytes.  Each wave owns a 32 x (128 + 4) slab of 32-bit values; LDS operations of one wave execute
+// in order, so no workgroup barrier is needed between the phases.
+#define DQ_GEMM_EPILOGUE \
+  using out_t = typename P::out_t; \
+  constexpr int kSlabStride = 132; \
+  constexpr int kOutPerPiece = 16 / sizeof(out_t); \
+  uint32_t* slab = reinterpret_cast<uint32_t*>(smem) + wave * (32 * kSlabStride); \
+  _Pragma("unroll") \
+  for (int mb = 0; mb < 4; ++mb) { \
+  _Pragma("unroll") \
+    for (int nb = 0; nb < 4; ++nb) \
+  _Pragma("unroll") \
+      for (int i = 0; i < 16; ++i) { \
+        const int row = 8 * (i >> 2) + 4 * g + (i & 3); \
+        const decltype(acc[0][0][0] + 0) elem = acc[mb][nb][i]; \
+        uint32_t bits; \
+        __builtin_memcpy(&bits, &elem, 4); \
+        slab[row * kSlabStride + nb * 32 + r] = bits; \
+      } \
+    __builtin_amdgcn_wave_barrier(); \
+    if constexpr (!P::kTransposed) { \
+      constexpr int kPiecesPerRow = 128 / kOutPerPiece; \
+      constexpr int kIters = 32 * kPiecesPerRow / 64; \
+  _Pragma("unroll") \
+      for (int it = 0; it < kIters; ++it) { \
+        const int q = lane + 64 * it; \
+        const int row = q / kPiecesPerRow, piece = q % kPiecesPerRow; \
+        const int m = m0 + wm * 128 + mb * 32 + row; \
+        const int n = n0 + wn * 128 + piece * kOutPerPiece; \
+        uint32_t raw[kOutPerPiece]; \
+  _Pragma("unroll") \
+        for (int e = 0; e < kOutPerPiece; e += 4) { \
+          const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * kSlabStride + piece * kOutPerPiece + e); \
+          raw[e] = v[0]; raw[e + 1] = v[1]; raw[e + 2] = v[2]; raw[e + 3] = v[3]; \
+        } \
+        if (m < M && n < N) { \
+          out_t o[kOutPerPiece]; \
+  _Pragma("unroll") \
+          for (int e = 0; e < kOutPerPiece; ++e) o[e] = P::finish(raw[e], p, m, min(n + e, N - 1)); \
+          out_t* dst = (out_t*)p.C + (size_t)m * N + n; \
+          if ((n + kOutPerPiece <= N) && ((N % kOutPerPiece) == 0)) { \
+            uint4_t pk; \
+            __builtin_memcpy(&pk, o, 16); \
+            *reinterpret_cast<uint4_t*>(dst) = pk; \
+          } else { \
+  _Pragma("unroll") \
+            for (int e = 0; e < kOutPerPiece; ++e) \
+              if (n + e < N) dst[e] = o[e]; \
+          } \
+        } \
+      } \
+    } else { \
+      constexpr int kPiecesPerCol = 32 / kOutPerPiece; \
+      constexpr int kIters = 128 * kPiecesPerCol / 64; \
+  _Pragma("unroll") \
+      for (int it = 0; it < kIters; ++it) { \
+        const int q = lane + 64 * it; \
+        const int col = q / kPiecesPerCol, piece = q % kPiecesPerCol; \
+        const int n = n0 + wn * 128 + col; \
+        const int m = m0 + wm * 128 + mb * 32 + piece * kOutPerPiece; \
+        if (n < N && m < M) { \
+          out_t o[kOutPerPiece]; \
+  _Pragma("unroll") \
+          for (int e = 0; e < kOutPerPiece; ++e) \
+            o[e] = P::finish(slab[(piece * kOutPerPiece + e) * kSlabStride + col], p, min(m + e, M - 1), n); \
+          out_t* dst = (out_t*)p.C + (size_t)n * M + m; \
+          if ((m + kOutPerPiece <= M) && ((M % kOutPerPiece) == 0)) { \
+            uint4_t pk; \
+            __builtin_memcpy(&pk, o, 16); \
+            *reinterpret_cast<uint4_t*>(dst) = pk; \
+          } else { \
+  _Pragma("unroll") \
+            for (int e = 0; e < kOutPerPiece; ++e) \
+              if (m + e < M) dst[e] = o[e]; \
+          } \
+        } \
+      } \
+    } \
+    __builtin_amdgcn_wave_barrier(); \
+  } \
+  /* end of epilogue */
 
 // Policy interface (all static):
 //   kBRowBytes        packed B bytes per weight row per k-block: 32 or 64
@@ -189,145 +275,317 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
-  // ---- prologue --------------------------------------------------------------------------------
-  load_tile(0);
-  typename P::ScaleRaw sc_cur[4], sc_next[4];
+  // ---- fragment readers ---------------------------------------------------------------------
+  using frag_t = typename P::frag_t;
+  auto read_a = [&](const unsigned char* base, int j, frag_t (&af)[4]) {
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) sc_cur[nb] = P::fetch_scale(p, w_row[nb], 0, g);
-  store_tile(0);
-  if (KB > 1) load_tile(1);
-  __syncthreads();
-
-  for (int kb = 0; kb < KB; ++kb) {
-    const int stage = kb & 1;
-    const unsigned char* base = smem + stage * kStage;
-    if (kb + 1 < KB) {
-      store_tile(stage ^ 1);  // tile kb+1 (loaded during the previous iteration) -> other stage
+    for (int mb = 0; mb < 4; ++mb)
+      af[mb] = *reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
+  };
+  auto read_b = [&](const unsigned char* base, uint32_t (&bw)[4][kBWords]) {
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) sc_next[nb] = P::fetch_scale(p, w_row[nb], kb + 1, g);
-    }
-    if (kb + 2 < KB) load_tile(kb + 2);
-
-    uint32_t bw[4][kBWords];
-    typename P::Scale sc[4];
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+    for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
       for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
         const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb][h]);
         bw[nb][4 * h + 0] = v[0]; bw[nb][4 * h + 1] = v[1]; bw[nb][4 * h + 2] = v[2]; bw[nb][4 * h + 3] = v[3];
       }
-      sc[nb] = P::prep_scale(sc_cur[nb], p);
+  };
+
+  // ---- prologue: tiles 0 and 1 in LDS, tile 2 in registers, fragments of (tile 0, step 0) ready --
+  // Three LDS stages.  During iteration kb: tile kb+2 goes registers -> stage (kb+2)%3 (last read in
+  // iteration kb-1, protected by the barrier that ended it), tile kb+3 goes global -> registers, tile
+  // kb is multiplied out of stage kb%3, and during its last step the first fragments of tile kb+1 are
+  // already fetched from stage (kb+1)%3 (written in iteration kb-1): one barrier per iteration and the
+  // LDS -> register -> MFMA pipeline never drains.
+  typename P::ScaleRaw sc_raw1[4], sc_raw2[4];  // raw scales of tiles kb+1 and kb+2
+  typename P::Scale sc_c[4], sc_n[4];
+  load_tile(0);
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    sc_c[nb] = P::prep_scale(P::fetch_scale(p, w_row[nb], 0, g), p);
+    sc_raw1[nb] = P::fetch_scale(p, w_row[nb], KB > 1 ? 1 : 0, g);
+  }
+  store_tile(0);
+  if (KB > 1) {
+    load_tile(1);
+    store_tile(1);
+  }
+  if (KB > 2) load_tile(2);
+  __syncthreads();
+
+  uint32_t bw_c[4][kBWords], bw_n[4][kBWords];
+  frag_t af_c[4], bf_c[4], af_n[4], bf_n[4];
+  read_b(smem, bw_c);
+  read_a(smem, 0, af_c);
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) bf_c[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
+
+  int stage = 0;
+  for (int kb = 0; kb < KB; ++kb) {
+    const int stage1 = stage == 2 ? 0 : stage + 1;
+    const int stage2 = stage1 == 2 ? 0 : stage1 + 1;
+    const unsigned char* base = smem + stage * kStage;
+    const unsigned char* base_n = smem + stage1 * kStage;
+    if (kb + 2 < KB) {
+      store_tile(stage2);
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) sc_raw2[nb] = P::fetch_scale(p, w_row[nb], kb + 2, g);
     }
+    if (kb + 3 < KB) load_tile(kb + 3);
+    const bool has_next = kb + 1 < KB;
+
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      typename P::frag_t af[4], bf[4];
+      // fetch and decode the operands of the next step while this step's MFMAs run
+      if (j < 3) {
+        read_a(base, j + 1, af_n);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
+        if (j == 2 && has_next) read_b(base_n, bw_n);
+      } else if (has_next) {
+        read_a(base_n, 0, af_n);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+          sc_n[nb] = P::prep_scale(sc_raw1[nb], p);
+          bf_n[nb] = P::decode(bw_n[nb], 0, sc_n[nb]);
+        }
+      }
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb)
-        af[mb] = *reinterpret_cast<const typename P::frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) bf[nb] = P::decode(bw[nb], j, sc[nb]);
+        for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = P::mfma(af_c[mb], bf_c[nb], acc[mb][nb]);
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = P::mfma(af[mb], bf[nb], acc[mb][nb]);
+      for (int q = 0; q < 4; ++q) {
+        af_c[q] = af_n[q];
+        bf_c[q] = bf_n[q];
+      }
     }
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) sc_cur[nb] = sc_next[nb];
+    for (int nb = 0; nb < 4; ++nb) {
+      sc_c[nb] = sc_n[nb];
+      sc_raw1[nb] = sc_raw2[nb];
+#pragma unroll
+      for (int w = 0; w < kBWords; ++w) bw_c[nb][w] = bw_n[nb][w];
+    }
+    stage = stage1;
     __syncthreads();
   }
 
-  // ---- epilogue: acc[mb][nb][i] = C[m0 + wm*128 + mb*32 + 8*(i/4) + 4*g + i%4][n0 + wn*128 + nb*32 + r]
-  // Staged through LDS (every tile is consumed: the loop ended with a barrier).  Each wave owns
-  // a 32 x (128 + 4) slab of 32-bit values; LDS operations of one wave execute in order, so no
-  // workgroup barrier is needed between the phases.
-  using out_t = typename P::out_t;
-  constexpr int kSlabStride = 132;
-  constexpr int kOutPerPiece = 16 / sizeof(out_t);  // values per 16-byte store: 8 (16-bit) or 4 (int32)
-  uint32_t* slab = reinterpret_cast<uint32_t*>(smem) + wave * (32 * kSlabStride);
+  DQ_GEMM_EPILOGUE
+}
+
+// ---- direct-to-LDS variant ---------------------------------------------------------------------
+// For policies whose A needs no transform (P::kPlainA) and whose scales are either absent or one
+// byte per 32 k (P::kScaleBytes): the A and packed-B tiles, and the scale bytes, travel
+// global -> LDS with global_load_lds_dwordx4 / _dword, two tiles ahead of the MFMAs, without
+// passing through registers.  A lane's 16 bytes land at LDS base + lane * 16 whatever its source
+// address, so the XOR swizzle of the A rows is applied by permuting the SOURCE addresses.  These
+// loads are issued from inline assembly and tracked by hand (one s_waitcnt vmcnt per tile): the
+// kernel issues no other vector-memory load inside the main loop, so the counter only ever
+// holds these.  Requires K % 128 == 0 and A, B smaller than 4 GiB (32-bit lane offsets).
+__device__ __forceinline__ void dma16(unsigned lds_addr, unsigned voff, const void* sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const void* sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+
+template <class P>
+__global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  static_assert(P::kBRowBytes == 32, "direct-to-LDS variant: 32 packed bytes per weight row per tile");
+  constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
+  constexpr int kStage = kAStage + kBStage;    // 40 KiB
+  constexpr int kStages = 3;
+  constexpr int kRing = kStages * kStage;      // scale ring: 4 slots x 1 KiB (256 rows x 4 scale bytes = 2 tiles)
+  constexpr int kBWords = 4;
+  constexpr int kTileLoads = 10;               // DMA instructions per thread per tile: 8 (A) + 2 (B)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int g = lane >> 5, r = lane & 31;
+  const int M = p.M, N = p.N, K = p.K;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int KB = K / P::kKPerBlock;
+  const unsigned lds0 = (unsigned)(size_t)smem;  // LDS byte address of the dynamic segment
+
+  // ---- per-lane source offsets: LDS chunk c (16 bytes) of a tile <- which global 16 bytes --------
+  unsigned a_voff[8], b_voff[2];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = (wave * 8 + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
+    const int row = c >> 3, pp = c & 7;
+    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * 2) + (unsigned)((pp ^ (row & 7)) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int c = (wave * 2 + i) * 64 + lane;  // B chunk: row c / 2, physical piece c % 2
+    const int row = c >> 1, pp = c & 1;
+    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K >> 1) + (unsigned)(((pp + (row >> 2)) & 1) << 4);
+  }
+  const unsigned s_voff = (unsigned)min(n0 + tid, N - 1) * (unsigned)(K >> 5);
+
+  auto issue_tile = [&](int kb, int stage) {
+    const unsigned sbase = lds0 + stage * kStage;
+    const unsigned char* ga = (const unsigned char*)p.A + (size_t)kb * 128;
+    const unsigned char* gb = (const unsigned char*)p.B + (size_t)kb * 32;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma16(sbase + (wave * 8 + i) * 1024, a_voff[i], ga);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dma16(sbase + kAStage + (wave * 2 + i) * 1024, b_voff[i], gb);
+  };
+  auto issue_scales = [&](int pair) {  // scale bytes of tiles 2 pair and 2 pair + 1
+    if constexpr (P::kScaleBytes)
+      dma4(lds0 + kRing + (pair & 3) * 1024 + wave * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
+  };
+
+  // ---- fragment read offsets (same LDS geometry as the register-staged kernel) --------------------
+  int a_row_off[4], a_row_sw[4], b_off[4], s_off[4];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
+    const int row = wm * 128 + mb * 32 + r;
+    a_row_off[mb] = row * 128;
+    a_row_sw[mb] = row & 7;
+  }
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    const int row = wn * 128 + nb * 32 + r;
+    b_off[nb] = kAStage + row * 32 + (((g + (row >> 2)) & 1) << 4);
+    s_off[nb] = kRing + row * 4 + g;
+  }
+  using frag_t = typename P::frag_t;
+  auto read_a = [&](const unsigned char* base, int j, frag_t (&af)[4]) {
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+      af[mb] = *reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
+  };
+  auto read_b = [&](const unsigned char* base, uint32_t (&bw)[4][kBWords]) {
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb]);
+      bw[nb][0] = v[0]; bw[nb][1] = v[1]; bw[nb][2] = v[2]; bw[nb][3] = v[3];
+    }
+  };
+  auto read_scales = [&](int kb, typename P::Scale (&sc)[4]) {
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      int e = 0;
+      if constexpr (P::kScaleBytes) e = smem[s_off[nb] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2];
+      sc[nb] = P::prep_scale(e, p);
+    }
+  };
+
+  typename P::acc_t acc[4][4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int row = 8 * (i >> 2) + 4 * g + (i & 3);
-        // copy the element out first: bit-casting the vector-element expression itself is unreliable
-        const decltype(acc[0][0][0] + 0) elem = acc[mb][nb][i];
-        uint32_t bits;
-        __builtin_memcpy(&bits, &elem, 4);
-        slab[row * kSlabStride + nb * 32 + r] = bits;
+      for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
+
+  // ---- prologue: tiles 0 and 1 (and their scales) in flight, wait, first fragments ------------------
+  issue_scales(0);
+  issue_tile(0, 0);
+  if (KB > 1) issue_tile(1, 1);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  typename P::Scale sc_c[4], sc_n[4];
+  uint32_t bw_c[4][kBWords], bw_n[4][kBWords];
+  frag_t af_c[4], bf_c[4], af_n[4], bf_n[4];
+  read_scales(0, sc_c);
+  read_b(smem, bw_c);
+  read_a(smem, 0, af_c);
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) bf_c[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
+
+  int stage = 0;
+  for (int kb = 0; kb < KB; ++kb) {
+    const int stage1 = stage == 2 ? 0 : stage + 1;
+    const int stage2 = stage1 == 2 ? 0 : stage1 + 1;
+    const unsigned char* base = smem + stage * kStage;
+    const unsigned char* base_n = smem + stage1 * kStage;
+    const bool has_next = kb + 1 < KB;
+    const bool has_next2 = kb + 2 < KB;
+    // stage2 was read during iteration kb-1; the barrier that ended it makes it free
+    if (has_next2) {
+      if ((kb & 1) == 0) issue_scales((kb + 2) >> 1);
+      issue_tile(kb + 2, stage2);
+    }
+
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (j < 3) {
+        read_a(base, j + 1, af_n);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
+        if (j == 2 && has_next) {
+          read_b(base_n, bw_n);
+          read_scales(kb + 1, sc_n);
+        }
+      } else if (has_next) {
+        read_a(base_n, 0, af_n);
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_n[nb], 0, sc_n[nb]);
       }
-    __builtin_amdgcn_wave_barrier();
-    if constexpr (!P::kTransposed) {
-      // C[M, N]: 32 rows x 128 columns, 16 bytes per lane per store
-      constexpr int kPiecesPerRow = 128 / kOutPerPiece;  // 16 or 32
-      constexpr int kIters = 32 * kPiecesPerRow / 64;    // 8 or 16
 #pragma unroll
-      for (int it = 0; it < kIters; ++it) {
-        const int q = lane + 64 * it;
-        const int row = q / kPiecesPerRow, piece = q % kPiecesPerRow;
-        const int m = m0 + wm * 128 + mb * 32 + row;
-        const int n = n0 + wn * 128 + piece * kOutPerPiece;
-        uint32_t raw[kOutPerPiece];
+      for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-        for (int e = 0; e < kOutPerPiece; e += 4) {
-          const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * kSlabStride + piece * kOutPerPiece + e);
-          raw[e] = v[0]; raw[e + 1] = v[1]; raw[e + 2] = v[2]; raw[e + 3] = v[3];
-        }
-        if (m < M && n < N) {
-          out_t o[kOutPerPiece];
+        for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = P::mfma(af_c[mb], bf_c[nb], acc[mb][nb]);
 #pragma unroll
-          for (int e = 0; e < kOutPerPiece; ++e) o[e] = P::finish(raw[e], p, m, min(n + e, N - 1));
-          out_t* dst = (out_t*)p.C + (size_t)m * N + n;
-          if ((n + kOutPerPiece <= N) && ((N % kOutPerPiece) == 0)) {
-            uint4_t pk;
-            __builtin_memcpy(&pk, o, 16);
-            *reinterpret_cast<uint4_t*>(dst) = pk;
-          } else {
-#pragma unroll
-            for (int e = 0; e < kOutPerPiece; ++e)
-              if (n + e < N) dst[e] = o[e];
-          }
-        }
-      }
-    } else {
-      // Ct[N, M]: the slab holds 32 (m) x 128 (n); a lane gathers kOutPerPiece consecutive m of one n
-      constexpr int kPiecesPerCol = 32 / kOutPerPiece;    // 4 or 8
-      constexpr int kIters = 128 * kPiecesPerCol / 64;    // 8 or 16
-#pragma unroll
-      for (int it = 0; it < kIters; ++it) {
-        const int q = lane + 64 * it;
-        const int col = q / kPiecesPerCol, piece = q % kPiecesPerCol;
-        const int n = n0 + wn * 128 + col;
-        const int m = m0 + wm * 128 + mb * 32 + piece * kOutPerPiece;
-        if (n < N && m < M) {
-          out_t o[kOutPerPiece];
-#pragma unroll
-          for (int e = 0; e < kOutPerPiece; ++e)
-            o[e] = P::finish(slab[(piece * kOutPerPiece + e) * kSlabStride + col], p, min(m + e, M - 1), n);
-          out_t* dst = (out_t*)p.C + (size_t)n * M + m;
-          if ((m + kOutPerPiece <= M) && ((M % kOutPerPiece) == 0)) {
-            uint4_t pk;
-            __builtin_memcpy(&pk, o, 16);
-            *reinterpret_cast<uint4_t*>(dst) = pk;
-          } else {
-#pragma unroll
-            for (int e = 0; e < kOutPerPiece; ++e)
-              if (m + e < M) dst[e] = o[e];
-          }
-        }
+      for (int q = 0; q < 4; ++q) {
+        af_c[q] = af_n[q];
+        bf_c[q] = bf_n[q];
       }
     }
-    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      sc_c[nb] = sc_n[nb];
+#pragma unroll
+      for (int w = 0; w < kBWords; ++w) bw_c[nb][w] = bw_n[nb][w];
+    }
+    stage = stage1;
+    // tile kb+2 must have landed before the next iteration prefetches from it: everything but the
+    // kTileLoads loads of tile kb+3 (issued at the top of the next iteration) - i.e. at this point
+    // only this iteration's own tile may still be in flight
+    if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kTileLoads) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
   }
+
+  DQ_GEMM_EPILOGUE
 }
 
 template <class P>
 int launch(const Params& p, hipStream_t stream) {
-  constexpr int kLds = 2 * (kAStage + BN * P::kBRowBytes);
+  constexpr int kLds = 3 * (kAStage + BN * P::kBRowBytes);
   auto kern = gemm_kernel<P>;
   static bool lds_limit_raised = false;  // once per kernel: legal under stream capture afterwards
+  if (!lds_limit_raised) {
+    DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+    lds_limit_raised = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(kThreads), kLds, stream, p);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <class P>
+bool dma_eligible(const Params& p) {
+  return (p.K % 128 == 0) && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
+}
+
+template <class P>
+int launch_dma(const Params& p, hipStream_t stream) {
+  constexpr int kLds = 3 * (kAStage + BN * P::kBRowBytes) + 4 * 1024;
+  auto kern = gemm_kernel_dma<P>;
+  static bool lds_limit_raised = false;
   if (!lds_limit_raised) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
     lds_limit_raised = true;
@@ -358,6 +616,7 @@ struct NoScale {
 
 struct PlainA {
   static constexpr bool kAPacked = false;
+  static constexpr bool kPlainA = true;  // stage_a is the identity: A may go global -> LDS directly
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return v; }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
 };

@@ -85,6 +85,7 @@ struct MxPolicy : Bf16Mfma, gemm::PlainA {
   static constexpr bool kTransposed = false;
   using out_t = bf16_t;
   using ScaleRaw = int;
+  static constexpr bool kScaleBytes = true;  // one scale byte per 32 k: eligible for the direct-to-LDS kernel
   struct Scale { float f; uint32_t add; };
   __device__ static __forceinline__ ScaleRaw fetch_scale(const Params& p, int row, int kb, int g) {
     return ((const uint8_t*)p.S)[(size_t)row * (p.K >> 5) + kb * 2 + g];
@@ -119,6 +120,9 @@ struct MxPolicy : Bf16Mfma, gemm::PlainA {
 template <bool TRANSPOSED>
 struct Fp16Fp4Policy : F16Mfma, gemm::PlainA, gemm::NoScale {
   static constexpr int kBRowBytes = 32;
+  static constexpr bool kScaleBytes = false;
+  __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
+  using gemm::NoScale::prep_scale;
   static constexpr bool kTransposed = TRANSPOSED;
   using out_t = half_t;
   __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
@@ -164,10 +168,14 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
                int scale_bias, hipStream_t stream) {
   Params p = gemm::make_params(A, B, S, nullptr, Bias, C, M, N, K);
   p.p0 = 127 - scale_bias;
-#define DQ_MX(FMT_)                                                        \
-  do {                                                                     \
-    if (Bias) return gemm::launch<MxPolicy<FMT_, true>>(p, stream);        \
-    return gemm::launch<MxPolicy<FMT_, false>>(p, stream);                 \
+#define DQ_MX(FMT_)                                                                          \
+  do {                                                                                       \
+    if (gemm::dma_eligible<MxPolicy<FMT_, false>>(p)) {                                      \
+      if (Bias) return gemm::launch_dma<MxPolicy<FMT_, true>>(p, stream);                    \
+      return gemm::launch_dma<MxPolicy<FMT_, false>>(p, stream);                             \
+    }                                                                                        \
+    if (Bias) return gemm::launch<MxPolicy<FMT_, true>>(p, stream);                          \
+    return gemm::launch<MxPolicy<FMT_, false>>(p, stream);                                   \
   } while (0)
   switch (fmt) {
     case FP4_E2M1: DQ_MX(FP4_E2M1);
@@ -180,6 +188,10 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
 
 int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream) {
   Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
+  if (gemm::dma_eligible<Fp16Fp4Policy<true>>(p)) {
+    if (transposed) return gemm::launch_dma<Fp16Fp4Policy<true>>(p, stream);
+    return gemm::launch_dma<Fp16Fp4Policy<false>>(p, stream);
+  }
   if (transposed) return gemm::launch<Fp16Fp4Policy<true>>(p, stream);
   return gemm::launch<Fp16Fp4Policy<false>>(p, stream);
 }
