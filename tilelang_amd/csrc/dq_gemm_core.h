@@ -28,6 +28,8 @@
 
 #include "dq_common.h"
 
+#include <type_traits>
+
 namespace dq {
 namespace gemm {
 
@@ -400,7 +402,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   constexpr int kStages = 3;
   constexpr int kRing = kStages * kStage;      // scale ring: 4 slots x 1 KiB (256 rows x 4 scale bytes = 2 tiles)
   constexpr int kBWords = 4;
-  constexpr int kTileLoads = 10;               // DMA instructions per thread per tile: 8 (A) + 2 (B)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -431,19 +432,26 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   }
   const unsigned s_voff = (unsigned)min(n0 + tid, N - 1) * (unsigned)(K >> 5);
 
-  auto issue_tile = [&](int kb, int stage) {
+  // One tile = 11 DMA instructions per thread: op 0 the scale dword (rows tid, tiles 2p and 2p+1; issued
+  // with every tile, i.e. twice per pair, which keeps the loop branch-free), ops 1..8 the A chunks, ops
+  // 9..10 the packed-B chunks.
+  constexpr int kTileOps = 11;
+  auto issue_op = [&](int op, int kb, int stage) {
     const unsigned sbase = lds0 + stage * kStage;
-    const unsigned char* ga = (const unsigned char*)p.A + (size_t)kb * 128;
-    const unsigned char* gb = (const unsigned char*)p.B + (size_t)kb * 32;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) dma16(sbase + (wave * 8 + i) * 1024, a_voff[i], ga);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) dma16(sbase + kAStage + (wave * 2 + i) * 1024, b_voff[i], gb);
+    if (op == 0) {
+      if constexpr (P::kScaleBytes) {
+        const int pair = kb >> 1;
+        dma4(lds0 + kRing + (pair & 3) * 1024 + wave * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
+      }
+    } else if (op <= 8) {
+      const int i = op - 1;
+      dma16(sbase + (wave * 8 + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
+    } else {
+      const int i = op - 9;
+      dma16(sbase + kAStage + (wave * 2 + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * 32);
+    }
   };
-  auto issue_scales = [&](int pair) {  // scale bytes of tiles 2 pair and 2 pair + 1
-    if constexpr (P::kScaleBytes)
-      dma4(lds0 + kRing + (pair & 3) * 1024 + wave * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
-  };
+  constexpr int kWaitOps = P::kScaleBytes ? kTileOps : kTileOps - 1;  // outstanding DMA instructions of one tile
 
   // ---- fragment read offsets (same LDS geometry as the register-staged kernel) --------------------
   int a_row_off[4], a_row_sw[4], b_off[4], s_off[4];
@@ -460,25 +468,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
     s_off[nb] = kRing + row * 4 + g;
   }
   using frag_t = typename P::frag_t;
-  auto read_a = [&](const unsigned char* base, int j, frag_t (&af)[4]) {
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-      af[mb] = *reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
+  auto read_a1 = [&](const unsigned char* base, int j, int mb) -> frag_t {
+    return *reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
   };
-  auto read_b = [&](const unsigned char* base, uint32_t (&bw)[4][kBWords]) {
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-      const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb]);
-      bw[nb][0] = v[0]; bw[nb][1] = v[1]; bw[nb][2] = v[2]; bw[nb][3] = v[3];
-    }
+  auto read_b1 = [&](const unsigned char* base, int nb, uint32_t (&bw)[kBWords]) {
+    const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb]);
+    bw[0] = v[0]; bw[1] = v[1]; bw[2] = v[2]; bw[3] = v[3];
   };
-  auto read_scales = [&](int kb, typename P::Scale (&sc)[4]) {
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-      int e = 0;
-      if constexpr (P::kScaleBytes) e = smem[s_off[nb] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2];
-      sc[nb] = P::prep_scale(e, p);
-    }
+  auto read_scale1 = [&](int kb, int nb) -> typename P::Scale {
+    int e = 0;
+    if constexpr (P::kScaleBytes) e = smem[s_off[nb] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2];
+    return P::prep_scale(e, p);
   };
 
   typename P::acc_t acc[4][4];
@@ -489,55 +489,59 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
-  // ---- prologue: tiles 0 and 1 (and their scales) in flight, wait, first fragments ------------------
-  issue_scales(0);
-  issue_tile(0, 0);
-  if (KB > 1) issue_tile(1, 1);
+  // ---- prologue: tiles 0 and 1 (and their scales) in flight, wait, first operands -------------------
+#pragma unroll
+  for (int op = 0; op < kTileOps; ++op) issue_op(op, 0, 0);
+#pragma unroll
+  for (int op = 0; op < kTileOps; ++op) issue_op(op, 1, 1);  // KB >= 2 because K % 128 == 0
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   typename P::Scale sc_c[4], sc_n[4];
   uint32_t bw_c[4][kBWords], bw_n[4][kBWords];
   frag_t af_c[4], bf_c[4], af_n[4], bf_n[4];
-  read_scales(0, sc_c);
-  read_b(smem, bw_c);
-  read_a(smem, 0, af_c);
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) bf_c[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
+  for (int q = 0; q < 4; ++q) {
+    sc_c[q] = read_scale1(0, q);
+    read_b1(smem, q, bw_c[q]);
+    af_c[q] = read_a1(smem, 0, q);
+    bf_c[q] = P::decode(bw_c[q], 0, sc_c[q]);
+  }
 
-  int stage = 0;
-  for (int kb = 0; kb < KB; ++kb) {
+  // One iteration = tile kb out of `stage`.  The 64 MFMAs are laid out as 16 chunks of 4 (one A
+  // fragment against the four B fragments); every chunk carries its share of the side work - one
+  // A-fragment read and one B-fragment decode for the NEXT step (next tile in the last step), one DMA
+  // instruction of tile kb+2 - and a scheduling barrier keeps the chunks in this order, so that work
+  // issues in the shadow of the chunk's MFMAs.  Stage (kb+2) % 3 was last read in iteration kb-1 and is
+  // free since the barrier that ended it.
+  auto iteration = [&](int kb, int stage, auto next_tag, auto next2_tag) {
+    constexpr bool has_next = decltype(next_tag)::value;
+    constexpr bool has_next2 = decltype(next2_tag)::value;
     const int stage1 = stage == 2 ? 0 : stage + 1;
     const int stage2 = stage1 == 2 ? 0 : stage1 + 1;
     const unsigned char* base = smem + stage * kStage;
     const unsigned char* base_n = smem + stage1 * kStage;
-    const bool has_next = kb + 1 < KB;
-    const bool has_next2 = kb + 2 < KB;
-    // stage2 was read during iteration kb-1; the barrier that ended it makes it free
-    if (has_next2) {
-      if ((kb & 1) == 0) issue_scales((kb + 2) >> 1);
-      issue_tile(kb + 2, stage2);
-    }
-
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      if (j < 3) {
-        read_a(base, j + 1, af_n);
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
-        if (j == 2 && has_next) {
-          read_b(base_n, bw_n);
-          read_scales(kb + 1, sc_n);
+      for (int q = 0; q < 4; ++q) {
+        const int chunk = j * 4 + q;
+        if (j < 3) {
+          af_n[q] = read_a1(base, j + 1, q);
+          bf_n[q] = P::decode(bw_c[q], j + 1, sc_c[q]);
+          if (j == 2 && has_next) {
+            read_b1(base_n, q, bw_n[q]);
+            sc_n[q] = read_scale1(kb + 1, q);
+          }
+        } else if (has_next) {
+          af_n[q] = read_a1(base_n, 0, q);
+          bf_n[q] = P::decode(bw_n[q], 0, sc_n[q]);
         }
-      } else if (has_next) {
-        read_a(base_n, 0, af_n);
+        if (has_next2 && chunk < kTileOps) issue_op(chunk, kb + 2, stage2);
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_n[nb], 0, sc_n[nb]);
+        for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
+        __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = P::mfma(af_c[mb], bf_c[nb], acc[mb][nb]);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         af_c[q] = af_n[q];
@@ -550,14 +554,22 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
 #pragma unroll
       for (int w = 0; w < kBWords; ++w) bw_c[nb][w] = bw_n[nb][w];
     }
-    stage = stage1;
-    // tile kb+2 must have landed before the next iteration prefetches from it: everything but the
-    // kTileLoads loads of tile kb+3 (issued at the top of the next iteration) - i.e. at this point
-    // only this iteration's own tile may still be in flight
-    if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kTileLoads) : "memory");
+    // tile kb+1 must have landed before the next iteration reads it: at this point only tile kb+2
+    // (issued during this iteration) may still be in flight
+    if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+  };
+
+  int stage = 0;
+  int kb = 0;
+  for (; kb + 2 < KB; ++kb) {
+    iteration(kb, stage, std::true_type{}, std::true_type{});
+    stage = stage == 2 ? 0 : stage + 1;
   }
+  iteration(kb, stage, std::true_type{}, std::false_type{});
+  stage = stage == 2 ? 0 : stage + 1;
+  iteration(kb + 1, stage, std::false_type{}, std::false_type{});
 
   DQ_GEMM_EPILOGUE
 }
