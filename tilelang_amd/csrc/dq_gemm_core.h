@@ -30,6 +30,10 @@
 
 #include <type_traits>
 
+#ifndef DQ_SWZ_SHIFT
+#define DQ_SWZ_SHIFT 1
+#endif
+
 namespace dq {
 namespace gemm {
 
@@ -37,6 +41,9 @@ constexpr int BM = 256, BN = 256;
 constexpr int kThreads = 256;
 constexpr int kARowBytes = 128;            // bytes of one A row per k-block in LDS
 constexpr int kAStage = BM * kARowBytes;   // 32 KiB
+
+// XOR key of the 16-byte pieces of A row `row` in LDS (rows are 128 B).
+__host__ __device__ constexpr int a_swz(int row) { return (row >> DQ_SWZ_SHIFT) & 7; }
 
 struct Params {
   const void* A;
@@ -200,12 +207,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
     if constexpr (P::kAPacked) {
       const int row = q >> 2, piece = q & 3;
       a_src[i] = (const unsigned char*)p.A + (size_t)min(m0 + row, M - 1) * a_row_bytes + piece * 16;
-      a_dst[i] = row * 128 + (((2 * piece) ^ (row & 7)) << 4);
-      a_dst2[i] = row * 128 + (((2 * piece + 1) ^ (row & 7)) << 4);
+      a_dst[i] = row * 128 + (((2 * piece) ^ a_swz(row)) << 4);
+      a_dst2[i] = row * 128 + (((2 * piece + 1) ^ a_swz(row)) << 4);
     } else {
       const int row = q >> 3, piece = q & 7;
       a_src[i] = (const unsigned char*)p.A + (size_t)min(m0 + row, M - 1) * a_row_bytes + piece * 16;
-      a_dst[i] = row * 128 + ((piece ^ (row & 7)) << 4);
+      a_dst[i] = row * 128 + ((piece ^ a_swz(row)) << 4);
       a_dst2[i] = 0;
     }
   }
@@ -216,8 +223,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
     const int q = tid + kThreads * i;
     const int row = q / kBPiecesPerRow, piece = q % kBPiecesPerRow;
     b_src[i] = (const unsigned char*)p.B + (size_t)min(n0 + row, N - 1) * b_row_bytes + piece * 16;
-    // rotate the pieces of a row by (row / 4) so that 8 consecutive rows cover all bank groups
-    b_dst[i] = kAStage + row * P::kBRowBytes + (((piece + (row >> (kBPiecesPerRow == 2 ? 2 : 1))) % kBPiecesPerRow) << 4);
+    // rotate the pieces of a row so that the 16 rows of one ds_read_b128 phase cover all 64 banks
+    b_dst[i] = kAStage + row * P::kBRowBytes + (((piece + (row >> (kBPiecesPerRow == 2 ? 3 : 2))) % kBPiecesPerRow) << 4);
   }
 
   uint4_t a_reg[kALoads], b_reg[kBLoads];
@@ -253,7 +260,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
   for (int mb = 0; mb < 4; ++mb) {
     const int row = wm * 128 + mb * 32 + r;
     a_row_off[mb] = row * 128;
-    a_row_sw[mb] = row & 7;
+    a_row_sw[mb] = a_swz(row);
   }
   // packed B of n-block nb: row wn*128 + nb*32 + r, the half of the row that belongs to group g
   int b_off[4][kBPiecesPerRow / 2];
@@ -265,7 +272,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
 #pragma unroll
     for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
       const int piece = g * (kBPiecesPerRow / 2) + h;
-      b_off[nb][h] = kAStage + row * P::kBRowBytes + (((piece + (row >> (kBPiecesPerRow == 2 ? 2 : 1))) % kBPiecesPerRow) << 4);
+      b_off[nb][h] = kAStage + row * P::kBRowBytes + (((piece + (row >> (kBPiecesPerRow == 2 ? 3 : 2))) % kBPiecesPerRow) << 4);
     }
   }
 
@@ -422,13 +429,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   for (int i = 0; i < 8; ++i) {
     const int c = (wave * 8 + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
     const int row = c >> 3, pp = c & 7;
-    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * 2) + (unsigned)((pp ^ (row & 7)) << 4);
+    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * 2) + (unsigned)((pp ^ a_swz(row)) << 4);
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int c = (wave * 2 + i) * 64 + lane;  // B chunk: row c / 2, physical piece c % 2
     const int row = c >> 1, pp = c & 1;
-    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K >> 1) + (unsigned)(((pp + (row >> 2)) & 1) << 4);
+    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K >> 1) + (unsigned)(((pp + (row >> 3)) & 1) << 4);
   }
   const unsigned s_voff = (unsigned)min(n0 + tid, N - 1) * (unsigned)(K >> 5);
 
@@ -459,12 +466,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   for (int mb = 0; mb < 4; ++mb) {
     const int row = wm * 128 + mb * 32 + r;
     a_row_off[mb] = row * 128;
-    a_row_sw[mb] = row & 7;
+    a_row_sw[mb] = a_swz(row);
   }
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
     const int row = wn * 128 + nb * 32 + r;
-    b_off[nb] = kAStage + row * 32 + (((g + (row >> 2)) & 1) << 4);
+    b_off[nb] = kAStage + row * 32 + (((g + (row >> 3)) & 1) << 4);
     s_off[nb] = kRing + row * 4 + g;
   }
   using frag_t = typename P::frag_t;
@@ -489,54 +496,73 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
-  // ---- prologue: tiles 0 and 1 (and their scales) in flight, wait, first operands -------------------
+  // ---- prologue: tiles 0 and 1 (and their scales) in flight; only tile 0 has to have landed -------
 #pragma unroll
   for (int op = 0; op < kTileOps; ++op) issue_op(op, 0, 0);
 #pragma unroll
   for (int op = 0; op < kTileOps; ++op) issue_op(op, 1, 1);  // KB >= 2 because K % 128 == 0
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
   __syncthreads();
 
-  typename P::Scale sc_c[4], sc_n[4];
-  uint32_t bw_c[4][kBWords], bw_n[4][kBWords];
+  typename P::Scale sc_c[4];
+  uint32_t bw_c[4][kBWords];
   frag_t af_c[4], bf_c[4], af_n[4], bf_n[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    sc_c[q] = read_scale1(0, q);
-    read_b1(smem, q, bw_c[q]);
-    af_c[q] = read_a1(smem, 0, q);
-    bf_c[q] = P::decode(bw_c[q], 0, sc_c[q]);
-  }
 
-  // One iteration = tile kb out of `stage`.  The 64 MFMAs are laid out as 16 chunks of 4 (one A
-  // fragment against the four B fragments); every chunk carries its share of the side work - one
-  // A-fragment read and one B-fragment decode for the NEXT step (next tile in the last step), one DMA
-  // instruction of tile kb+2 - and a scheduling barrier keeps the chunks in this order, so that work
-  // issues in the shadow of the chunk's MFMAs.  Stage (kb+2) % 3 was last read in iteration kb-1 and is
-  // free since the barrier that ended it.
-  auto iteration = [&](int kb, int stage, auto next_tag, auto next2_tag) {
-    constexpr bool has_next = decltype(next_tag)::value;
+  // One iteration = tile kb out of `stage`, as 16 chunks of 4 MFMAs (one A fragment against the four
+  // B fragments) kept in order by scheduling barriers; every chunk carries side work that issues in
+  // the shadow of its MFMAs.  The loop is skewed by one MFMA step so that nothing waits on LDS right
+  // after the barrier:
+  //   chunks  0..3   MFMAs of step 3 of tile kb-1 (operands already in registers); side work: read
+  //                  the packed B words, the scales and the step-0 A fragments of tile kb, decode step 0
+  //   chunks  4..15  MFMAs of steps 0..2 of tile kb; side work: read / decode the operands of the next
+  //                  step (the step-3 operands stay in registers for the next iteration)
+  //   chunks  0..10  also issue one DMA instruction each of tile kb+2 into stage (kb+2) % 3, which
+  //                  was last read in iteration kb-1 and is free since the barrier that ended it.
+  // Tile kb+2 is not read before iteration kb+2: its loads have almost two iterations to land.
+  auto iteration = [&](int kb, int stage, auto first_tag, auto next2_tag) {
+    constexpr bool first = decltype(first_tag)::value;
     constexpr bool has_next2 = decltype(next2_tag)::value;
-    const int stage1 = stage == 2 ? 0 : stage + 1;
-    const int stage2 = stage1 == 2 ? 0 : stage1 + 1;
+    const int stage2 = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3
     const unsigned char* base = smem + stage * kStage;
-    const unsigned char* base_n = smem + stage1 * kStage;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int q = 0; q < 4; ++q) {
+      if (q == 0) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+          read_b1(base, nb, bw_c[nb]);
+          sc_c[nb] = read_scale1(kb, nb);
+        }
+      } else if (q == 1) {
+        af_n[0] = read_a1(base, 0, 0);
+        af_n[1] = read_a1(base, 0, 1);
+      } else if (q == 2) {
+        af_n[2] = read_a1(base, 0, 2);
+        af_n[3] = read_a1(base, 0, 3);
+        bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]);
+        bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]);
+      } else {
+        bf_n[2] = P::decode(bw_c[2], 0, sc_c[2]);
+        bf_n[3] = P::decode(bw_c[3], 0, sc_c[3]);
+      }
+      if (has_next2) issue_op(q, kb + 2, stage2);
+      if (!first) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      af_c[q] = af_n[q];
+      bf_c[q] = bf_n[q];
+    }
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int chunk = j * 4 + q;
-        if (j < 3) {
-          af_n[q] = read_a1(base, j + 1, q);
-          bf_n[q] = P::decode(bw_c[q], j + 1, sc_c[q]);
-          if (j == 2 && has_next) {
-            read_b1(base_n, q, bw_n[q]);
-            sc_n[q] = read_scale1(kb + 1, q);
-          }
-        } else if (has_next) {
-          af_n[q] = read_a1(base_n, 0, q);
-          bf_n[q] = P::decode(bw_n[q], 0, sc_n[q]);
-        }
+        const int chunk = 4 + j * 4 + q;
+        af_n[q] = read_a1(base, j + 1, q);
+        bf_n[q] = P::decode(bw_c[q], j + 1, sc_c[q]);
         if (has_next2 && chunk < kTileOps) issue_op(chunk, kb + 2, stage2);
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
@@ -548,14 +574,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
         bf_c[q] = bf_n[q];
       }
     }
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-      sc_c[nb] = sc_n[nb];
-#pragma unroll
-      for (int w = 0; w < kBWords; ++w) bw_c[nb][w] = bw_n[nb][w];
-    }
-    // tile kb+1 must have landed before the next iteration reads it: at this point only tile kb+2
-    // (issued during this iteration) may still be in flight
+    // tile kb+1 must have landed before the next iteration reads it; tile kb+2 (issued during this
+    // iteration) may still be in flight
     if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -563,13 +583,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
 
   int stage = 0;
   int kb = 0;
-  for (; kb + 2 < KB; ++kb) {
-    iteration(kb, stage, std::true_type{}, std::true_type{});
+  if (KB > 2) {
+    iteration(0, 0, std::true_type{}, std::true_type{});
+    stage = 1;
+    for (kb = 1; kb + 2 < KB; ++kb) {
+      iteration(kb, stage, std::false_type{}, std::true_type{});
+      stage = stage == 2 ? 0 : stage + 1;
+    }
+    iteration(kb, stage, std::false_type{}, std::false_type{});
     stage = stage == 2 ? 0 : stage + 1;
+    iteration(kb + 1, stage, std::false_type{}, std::false_type{});
+  } else {  // KB == 2
+    iteration(0, 0, std::true_type{}, std::false_type{});
+    iteration(1, 1, std::false_type{}, std::false_type{});
   }
-  iteration(kb, stage, std::true_type{}, std::false_type{});
-  stage = stage == 2 ? 0 : stage + 1;
-  iteration(kb + 1, stage, std::false_type{}, std::false_type{});
+  // step 3 of the last tile
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
 
   DQ_GEMM_EPILOGUE
 }
