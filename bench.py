@@ -113,6 +113,58 @@ def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev):
     return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "graph": graphed}
 
 
+def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev):
+    """BitLinear forward on quantised operands: int8 x 2-bit (offset-binary ternary), fused acc/s_a/s_w epilogue."""
+    d = workloads.bitnet(M, N, K, seed=0)
+    nbytes = workloads.bitnet_bytes(M, N, K)
+    nc = _copies(nbytes, hi=40)
+    A = torch.from_numpy(d["A"]).to(dev)
+    Bs = [torch.from_numpy(d["B"]).to(dev).view(torch.int8).clone() for _ in range(nc)]
+    s_a = torch.from_numpy(np.asarray(d["s_a"], dtype=np.float32)).to(dev)
+    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset")
+    out = [None]
+
+    def mk(i):
+        def f():
+            out[0] = kern(A, Bs[i], s_a, skip_tensor_validation=True)
+        return f
+
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
+
+
+def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev):
+    """W4A8 (int8 x int4, Ct[N,M] int32) or int4 x int4 (C[M,N] int32), exact."""
+    if a_packed:
+        from tilelang_amd import quantize
+
+        d = workloads.int4_int4(M, N, K, seed=0)
+        kern = tl.matmul_nt_int4(M, N, K)
+        nbytes = M * K // 2 + N * K // 2 + 4 * M * N
+        A = quantize.pack_int4(torch.from_numpy(d["A_logical"])).to(dev)
+        B = quantize.pack_int4(torch.from_numpy(d["B_logical"])).to(dev)
+    else:
+        d = workloads.int8_int4(M, N, K, seed=0)
+        kern = tl.matmul_int8xint4(M, N, K)
+        nbytes = M * K + N * K // 2 + 4 * M * N
+        A = torch.from_numpy(d["A"]).to(dev)
+        B = torch.from_numpy(d["B"]).to(dev)
+    out = [None]
+
+    def f():
+        out[0] = kern(A, B, skip_tensor_validation=True)
+
+    ms, graphed = _time_launches(torch, [f], steps, warmup)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
+
+
+def _row(config, r, bound, peak):
+    sec = r["us"] * 1e-6
+    row = {"config": config, "us": r["us"], "GB/s": r["bytes"] / sec / 1e9, "TFLOP/s": r["flops"] / sec / 1e12, "bound": bound}
+    row["frac"] = (r["bytes"] / sec / HBM_PEAK) if bound == "hbm" else (r["flops"] / sec / peak)
+    return row
+
+
 def cpu_baseline_w4a16(N, K, rows, budget_s=20.0):
     """torch-CPU ref_program on the first `rows` weight rows of the headline shape, extrapolated to N rows."""
     import torch
@@ -182,9 +234,16 @@ def main():
             shapes.append({"config": f"w4a16_zeros M={m} N=28672 K=8192", "us": r["us"], "GB/s": r["bytes"] / r["us"] / 1e3,
                            "TFLOP/s": r["flops"] / r["us"] / 1e6, "bound": "hbm", "frac": r["bytes"] / (r["us"] * 1e-6) / HBM_PEAK,
                            "frac_mfma": r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK})
-        r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, max(6, args.steps // 10), 2, dev)
-        shapes.append({"config": "mxfp4_gemm M=4096 N=8192 K=8192", "us": r["us"], "GB/s": r["bytes"] / r["us"] / 1e3,
-                       "TFLOP/s": r["flops"] / r["us"] / 1e6, "bound": "mfma", "frac": r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK})
+        kg = max(6, args.steps // 10)
+        r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, kg, 2, dev)
+        shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
+        for m in (1, 256, 2048):
+            r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, k if m == 1 else kg, 2, dev)
+            shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, False, kg, 2, dev)
+        shapes.append(_row("w4a8_gemm M=4096 N=4096 K=4096 (Ct int32)", r, "mfma", MFMA_I8_PEAK))
+        r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, True, kg, 2, dev)
+        shapes.append(_row("int4xint4_gemm M=4096 N=4096 K=4096", r, "mfma", MFMA_I8_PEAK))
 
     cpu = None
     if not args.no_cpu:

@@ -26,73 +26,101 @@ namespace dq {
 
 namespace {
 
-// Sum over each 32-lane half of the wave; lane 31 and lane 63 receive the two totals.
-__device__ __forceinline__ float wave_half_reduce(float v) {
-  // quad_perm(1,0,3,2), quad_perm(2,3,0,1), row_half_mirror, row_mirror: all 16 lanes of a
-  // DPP row then hold the row total
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
-  // row_bcast:15 into rows 1 and 3: lanes 16..31 += lane 15, lanes 48..63 += lane 47
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));
-  return v;
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
 }
 
-constexpr int kMaxRowsPerWg = 128;
+// Sums N per-lane values over each DPP row of 16 lanes at once.  While more than one value is
+// left, a level lets a lane keep the value its lane bit selects and add the partner lane's copy
+// of it, which halves the number of values; afterwards a level is a plain add.  Levels: xor 1,
+// xor 2 (quad_perm), rotate by 4, rotate by 8 (row_ror).  On return lane l holds the row total
+// of value (l & (N - 1)).  N values cost about 3 (N - 1) + 4 instructions instead of 4 N.
+template <int N, int LEVEL>
+struct RowReduce {
+  static __device__ __forceinline__ float run(const float* v, int lane) {
+    if constexpr (LEVEL == 4) {
+      return v[0];
+    } else {
+      constexpr int kCtrl = LEVEL == 0 ? 0xB1 : (LEVEL == 1 ? 0x4E : (LEVEL == 2 ? 0x124 : 0x128));
+      if constexpr (N == 1) {
+        const float t[1] = {v[0] + dpp_move<kCtrl>(v[0])};
+        return RowReduce<1, LEVEL + 1>::run(t, lane);
+      } else {
+        const bool bit = (lane >> LEVEL) & 1;
+        float t[N / 2];
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+          const float keep = bit ? v[2 * i + 1] : v[2 * i];
+          const float give = bit ? v[2 * i] : v[2 * i + 1];
+          t[i] = keep + dpp_move<kCtrl>(give);
+        }
+        return RowReduce<N / 2, LEVEL + 1>::run(t, lane);
+      }
+    }
+  }
+};
 
-// R rows (per row slot) are in flight per thread; a workgroup walks NB batches of R rows and
-// re-issues the load of a row's successor as soon as that row's registers are consumed, so
-// the same R * NP loads stay in flight from the first instruction to the last batch.
-template <int MROWS, int NP, int R, bool HAS_SCALE, bool HAS_ZEROS, bool G128>
+constexpr int kMaxRowsPerWg = 128;  // also bounds nb * R (partial sums kept in LDS)
+
+// 256 threads.  A weight row is spread over tpr = 32..256 threads (16 bytes each per pass), so
+// a pass of the workgroup covers rpp = 256 / tpr rows; R row groups are in flight per thread
+// and a workgroup walks nb batches of R groups, re-issuing a group's loads for the next batch
+// as soon as its registers are consumed.  WIDE: tpr = 256 (one row per pass), which makes every
+// row address uniform (scalar base + per-thread offset).
+template <int MROWS, int NP, int R, bool HAS_SCALE, bool HAS_ZEROS, bool G128, bool FLIP, bool WIDE>
 __global__ __launch_bounds__(256) void w4a16_gemv_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                           const half_t* __restrict__ S, const half_t* __restrict__ Z,
                                                           half_t* __restrict__ C, int M, int N, int K, int group,
-                                                          int tpr_shift, int nb, uint32_t flip_mask, float zsub_const,
-                                                          int interleaved) {
-  __shared__ float red[kMaxRowsPerWg * 4 * MROWS];  // [row in workgroup][wave of the row][m]
+                                                          int tpr_shift_arg, int nb, float zsub_const, int interleaved) {
+  constexpr int NV = R * MROWS;  // values reduced together per batch
+  static_assert(NV <= 16, "at most 16 values per lane row");
+  // partial sums: [batch][16-lane row of the workgroup (16)][value]
+  __shared__ float red[kMaxRowsPerWg * 16 * MROWS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int tpr = 1 << tpr_shift;            // threads per row: 32, 64, 128 or 256
+  const int tpr_shift = WIDE ? 8 : tpr_shift_arg;
+  const int tpr = 1 << tpr_shift;            // threads per row
   const int rpp = 256 >> tpr_shift;          // rows per pass
-  const int slot = tid >> tpr_shift;         // which row of the pass
+  const int slot = WIDE ? 0 : (tid >> tpr_shift);
   const int ct = tid & (tpr - 1);            // chunk within the pass
-  const int wave_in_row = ct >> 6;
   const int c16 = K >> 5;                    // 16-byte chunks per row
   const int rows_per_batch = R * rpp;
   const int rows_per_wg = nb * rows_per_batch;
   const int row0 = blockIdx.x * rows_per_wg;
-  const size_t row_bytes = (size_t)(K >> 1);
+  const uint32_t row_bytes = (uint32_t)(K >> 1);
   const int groups_per_row = K / group;
   const int gshift = (group == K) ? 31 : (31 - __builtin_clz(group));
 
-  // per-pass byte offsets inside a row (chunk clamped: its activations are zeroed below)
-  int boff[NP], goff[NP];
+  // per-thread offsets from the (uniform) first row of a row group
+  uint32_t boff[NP], goff[NP];
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
-    const int chunk = min(p * tpr + ct, c16 - 1);
-    boff[p] = chunk * 16;
-    goff[p] = G128 ? (chunk >> 2) : ((chunk << 5) >> gshift);
+    const int chunk = min(p * tpr + ct, c16 - 1);  // clamped: its activations are zeroed below
+    boff[p] = (uint32_t)slot * row_bytes + (uint32_t)chunk * 16u;
+    goff[p] = (uint32_t)(slot * groups_per_row + (G128 ? (chunk >> 2) : ((chunk << 5) >> gshift))) * 2u;
   }
 
   uint4_t bq[R][NP];
   half_t sc[R][NP], zp[R][NP];
-  auto issue_row = [&](int u, int b) {
-    // rows past N are clamped to a valid row and masked at the store
-    const int row = min(row0 + b * rows_per_batch + u * rpp + slot, N - 1);
-    const uint8_t* bp = B + (size_t)row * row_bytes;
+  auto issue_group = [&](int u, int b) {
+    // groups past N (N is a multiple of rpp) are clamped to the last one and dropped at the store
+    const int rb = min(row0 + (b * R + u) * rpp, N - rpp);
+    const uint8_t* bp = B + (size_t)rb * row_bytes;
+    const uint8_t* sp = reinterpret_cast<const uint8_t*>(S) + (size_t)rb * groups_per_row * 2;
+    const uint8_t* zq = reinterpret_cast<const uint8_t*>(Z) + (size_t)rb * groups_per_row * 2;
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       bq[u][p] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(bp + boff[p]));
-      if constexpr (HAS_SCALE) sc[u][p] = S[(size_t)row * groups_per_row + goff[p]];
-      if constexpr (HAS_ZEROS) zp[u][p] = Z[(size_t)row * groups_per_row + goff[p]];
+      if constexpr (HAS_SCALE) sc[u][p] = *reinterpret_cast<const half_t*>(sp + goff[p]);
+      if constexpr (HAS_ZEROS) zp[u][p] = *reinterpret_cast<const half_t*>(zq + goff[p]);
     }
   };
 
   // ---- first batch of weight / scale / zero loads goes out before anything else ----------
 #pragma unroll
-  for (int u = 0; u < R; ++u) issue_row(u, 0);
+  for (int u = 0; u < R; ++u) issue_group(u, 0);
 
   // ---- this thread's activations, paired in decoder order ------------------------------
   uint32_t a[NP][MROWS][16];
@@ -118,92 +146,91 @@ __global__ __launch_bounds__(256) void w4a16_gemv_kernel(const half_t* __restric
           else s_even = __builtin_amdgcn_fdot2(as_half2(d[i]), one2, s_even, false);
         }
       }
-      abias[p][m] = 1024.f * s_even + 64.f * s_odd;
       asum[p][m] = s_even + s_odd;
+      // without per-group zeros the whole correction is one constant per thread
+      abias[p][m] = 1024.f * s_even + 64.f * s_odd + (HAS_ZEROS ? 0.f : zsub_const * asum[p][m]);
     }
   }
+
+  const bool writer = (lane & 15) < NV;
+  float* red_w = red + (tid >> 4) * NV + (lane & (NV - 1));
 
   // ---- stream the batches ----------------------------------------------------------------
   auto process_batch = [&](int b, auto refill_tag) {
     constexpr bool kRefill = decltype(refill_tag)::value;
-    float acc[R][MROWS];
+    float acc[NV];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
 #pragma unroll
-      for (int m = 0; m < MROWS; ++m) acc[u][m] = 0.f;
+      for (int m = 0; m < MROWS; ++m) acc[u * MROWS + m] = 0.f;
 #pragma unroll
       for (int p = 0; p < NP; ++p) {
-        float dot[MROWS];
+        float dot[MROWS][2];
 #pragma unroll
-        for (int m = 0; m < MROWS; ++m) dot[m] = 0.f;
+        for (int m = 0; m < MROWS; ++m) dot[m][0] = dot[m][1] = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           uint32_t t[4];
-          u4x8_to_biased_half(bq[u][p][j] ^ flip_mask, t);
+          u4x8_to_biased_half(FLIP ? (bq[u][p][j] ^ 0x88888888u) : bq[u][p][j], t);
 #pragma unroll
           for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int m = 0; m < MROWS; ++m)
-              dot[m] = __builtin_amdgcn_fdot2(as_half2(t[i]), as_half2(a[p][m][j * 4 + i]), dot[m], false);
+              dot[m][i & 1] = __builtin_amdgcn_fdot2(as_half2(t[i]), as_half2(a[p][m][j * 4 + i]), dot[m][i & 1], false);
         }
         const float s = HAS_SCALE ? (float)sc[u][p] : 1.f;
-        const float zsub = HAS_ZEROS ? (float)zp[u][p] : zsub_const;
 #pragma unroll
-        for (int m = 0; m < MROWS; ++m) acc[u][m] += s * (dot[m] - abias[p][m] - zsub * asum[p][m]);
-      }
-      // this row's registers are free again: refill them with the same row of the next batch.
-      // The scheduling barriers keep the refill behind this row's arithmetic (no second register
-      // set) and ahead of the next row's.
-      if constexpr (kRefill) {
-        __builtin_amdgcn_sched_barrier(0);
-        issue_row(u, b + 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-
-    // reduce over the threads of each row; the chains of the R rows are independent
-#pragma unroll
-    for (int u = 0; u < R; ++u) {
-      const int rl = b * rows_per_batch + u * rpp + slot;
-#pragma unroll
-      for (int m = 0; m < MROWS; ++m) {
-        float v = wave_half_reduce(acc[u][m]);
-        if (tpr >= 64) {
-          // lane 63 += lane 31 (row_bcast:31 into rows 2 and 3)
-          v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));
-          if (lane == 63) red[(rl * 4 + wave_in_row) * MROWS + m] = v;
-        } else {
-          // two rows per wave: lane 31 carries the even slot, lane 63 the odd one
-          if ((lane & 31) == 31) red[(rl * 4 + 0) * MROWS + m] = v;
+        for (int m = 0; m < MROWS; ++m) {
+          float d = (dot[m][0] + dot[m][1]) - abias[p][m];
+          if constexpr (HAS_ZEROS) d -= (float)zp[u][p] * asum[p][m];
+          acc[u * MROWS + m] += s * d;
         }
       }
+      // this group's registers are free again: refill them with the same group of the next
+      // batch.  The scheduling barriers keep the refill behind this group's arithmetic (no
+      // second register set) and ahead of the next group's.
+      if constexpr (kRefill) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_group(u, b + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
+    const float v = RowReduce<NV, 0>::run(acc, lane);
+    if (writer) red_w[b * 16 * NV] = v;
   };
   for (int b = 0; b + 1 < nb; ++b) process_batch(b, std::true_type{});
   process_batch(nb - 1, std::false_type{});
   __syncthreads();
-  const int waves_per_row = tpr >= 64 ? (tpr >> 6) : 1;
+
+  // ---- fixed-order sum of the 16-lane partials of each output ----------------------------
+  const int parts = tpr >> 4;  // 16-lane rows per weight row
   for (int o = tid; o < rows_per_wg * MROWS; o += 256) {
     const int rl = o / MROWS, m = o - rl * MROWS;
-    float v = red[(rl * 4 + 0) * MROWS + m];
-    for (int w = 1; w < waves_per_row; ++w) v += red[(rl * 4 + w) * MROWS + m];
+    const int b = rl / rows_per_batch, within = rl - b * rows_per_batch;
+    const int u = within >> (8 - tpr_shift), sl = within & (rpp - 1);
+    const float* src = red + (b * 16 + sl * parts) * NV + u * MROWS + m;
+    float v = src[0];
+    for (int j = 1; j < parts; ++j) v += src[j * NV];
     const int row = row0 + rl;
     if (row < N && m < M) C[(size_t)m * N + row] = (half_t)v;
   }
 }
 
-template <int MROWS, int NP, int R>
+template <int MROWS, int NP, int R, bool WIDE>
 int launch_gemv(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                 int mode, int layout, int tpr_shift, int nb, hipStream_t stream) {
-  const int rows_per_wg = nb * R * (256 >> tpr_shift);
-  if (rows_per_wg > kMaxRowsPerWg) DQ_FAIL("w4a16 gemv: %d rows per workgroup exceed %d", rows_per_wg, kMaxRowsPerWg);
+  const int rpp = 256 >> tpr_shift;
+  const int rows_per_wg = nb * R * rpp;
+  if (rows_per_wg > kMaxRowsPerWg || nb * R > kMaxRowsPerWg)
+    DQ_FAIL("w4a16 gemv: %d rows per workgroup exceed %d", rows_per_wg, kMaxRowsPerWg);
+  if (N % rpp != 0 || N < rpp) DQ_FAIL("w4a16 gemv: N=%d must be a multiple of %d for K=%d", N, rpp, K);
+  if (WIDE != (tpr_shift == 8)) DQ_FAIL("w4a16 gemv: internal dispatch error (tpr_shift %d)", tpr_shift);
   const dim3 grid((N + rows_per_wg - 1) / rows_per_wg), block(256);
-  uint32_t flip = 0;
   float zsub = 0.f;
-  bool has_scale = false, has_zeros = false;
+  bool has_scale = false, has_zeros = false, flip = false;
   switch (mode) {
     case W4_UNSIGNED: break;
-    case W4_SIGNED: flip = 0x88888888u; zsub = 8.f; break;
+    case W4_SIGNED: flip = true; zsub = 8.f; break;
     case W4_OFFSET8: zsub = 8.f; break;
     case W4_SCALE: zsub = 8.f; has_scale = true; break;
     case W4_USCALE: has_scale = true; break;
@@ -211,14 +238,14 @@ int launch_gemv(const void* A, const void* B, const void* S, const void* Z, void
     default: DQ_FAIL("w4a16 gemv: unknown mode %d", mode);
   }
   const int il = layout == LAYOUT_INTERLEAVED;
-#define DQ_GEMV(HS, HZ, G)                                                                                       \
-  hipLaunchKernelGGL((w4a16_gemv_kernel<MROWS, NP, R, HS, HZ, G>), grid, block, 0, stream, (const half_t*)A,      \
-                     (const uint8_t*)B, (const half_t*)S, (const half_t*)Z, (half_t*)C, M, N, K, group, tpr_shift, \
-                     nb, flip, zsub, il)
+#define DQ_GEMV(HS, HZ, G, FL)                                                                                   \
+  hipLaunchKernelGGL((w4a16_gemv_kernel<MROWS, NP, R, HS, HZ, G, FL, WIDE>), grid, block, 0, stream,              \
+                     (const half_t*)A, (const uint8_t*)B, (const half_t*)S, (const half_t*)Z, (half_t*)C, M, N, K, \
+                     group, tpr_shift, nb, zsub, il)
   const bool g128 = group == 128;
-  if (!has_scale) DQ_GEMV(false, false, false);
-  else if (!has_zeros) { if (g128) DQ_GEMV(true, false, true); else DQ_GEMV(true, false, false); }
-  else { if (g128) DQ_GEMV(true, true, true); else DQ_GEMV(true, true, false); }
+  if (!has_scale) { if (flip) DQ_GEMV(false, false, false, true); else DQ_GEMV(false, false, false, false); }
+  else if (!has_zeros) { if (g128) DQ_GEMV(true, false, true, false); else DQ_GEMV(true, false, false, false); }
+  else { if (g128) DQ_GEMV(true, true, true, false); else DQ_GEMV(true, true, false, false); }
 #undef DQ_GEMV
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
@@ -241,32 +268,38 @@ int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, 
   if (np_needed > 4) return 1;
   const int mrows = M == 1 ? 1 : (M == 2 ? 2 : 4);
   if (np * mrows > 4) return 1;
-  // rows_hint = r + 16 * nb (0 = choose here).  r rows in flight per thread (4 by default,
-  // fewer when the grid would be small); nb batches per workgroup so that the whole grid is
-  // resident at once (7 workgroups per CU) when the matrix is large enough.
   const int rpp = 256 >> tpr_shift;
+  if (N % rpp != 0 || N < rpp) return 1;
+  // rows_hint = r + 16 * nb (0 = choose here).  r row groups in flight per thread; nb batches
+  // per workgroup so that the grid is about one resident wave of workgroups on a large matrix.
   int r = rows_hint & 15, nb = rows_hint >> 4;
   if (r == 0) r = (((long)N / (4 * rpp)) >= 1024 ? 4 : 2);
-  if (np * r > 8) r = 8 / np;  // keep registers bounded
-  if (r != 2 && r != 4 && r != 8) r = 2;
+  if (r != 2 && r != 4) r = 2;
+  if (r * np * mrows > 8) r = 2;  // keep registers bounded
+  if (r * mrows > 16) return 1;
   if (nb == 0) {
     const long wgs1 = ((long)N + r * rpp - 1) / (r * rpp);
     nb = (int)((wgs1 + 1791) / 1792);
   }
-  while (nb > 1 && nb * r * rpp > 128) --nb;
+  while (nb > 1 && (nb * r * rpp > kMaxRowsPerWg || nb * r > kMaxRowsPerWg)) --nb;
   if (nb < 1) nb = 1;
-#define DQ_R(MR, NP_)                                                                                            \
-  do {                                                                                                           \
-    if (r == 8) return launch_gemv<MR, NP_, 8>(A, B, S, Z, C, M, N, K, group, mode, layout, tpr_shift, nb, stream); \
-    if (r == 4) return launch_gemv<MR, NP_, 4>(A, B, S, Z, C, M, N, K, group, mode, layout, tpr_shift, nb, stream); \
-    return launch_gemv<MR, NP_, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, tpr_shift, nb, stream);          \
+#define DQ_R(MR, NP_, W)                                                                                              \
+  do {                                                                                                                \
+    if (r == 4) return launch_gemv<MR, NP_, 4, W>(A, B, S, Z, C, M, N, K, group, mode, layout, tpr_shift, nb, stream); \
+    return launch_gemv<MR, NP_, 2, W>(A, B, S, Z, C, M, N, K, group, mode, layout, tpr_shift, nb, stream);            \
   } while (0)
-  if (mrows == 1 && np == 1) DQ_R(1, 1);
-  if (mrows == 1 && np == 2) DQ_R(1, 2);
-  if (mrows == 1 && np == 4) DQ_R(1, 4);
-  if (mrows == 2 && np == 1) DQ_R(2, 1);
-  if (mrows == 2 && np == 2) DQ_R(2, 2);
-  if (mrows == 4 && np == 1) DQ_R(4, 1);
+  if (tpr_shift == 8) {
+    if (mrows == 1 && np == 1) DQ_R(1, 1, true);
+    if (mrows == 1 && np == 2) DQ_R(1, 2, true);
+    if (mrows == 1 && np == 4) { r = 2; DQ_R(1, 4, true); }
+    if (mrows == 2 && np == 1) DQ_R(2, 1, true);
+    if (mrows == 2 && np == 2) { r = 2; DQ_R(2, 2, true); }
+    if (mrows == 4 && np == 1) DQ_R(4, 1, true);
+  } else {
+    if (mrows == 1) DQ_R(1, 1, false);
+    if (mrows == 2) DQ_R(2, 1, false);
+    if (mrows == 4) DQ_R(4, 1, false);
+  }
 #undef DQ_R
   return 1;
 }
