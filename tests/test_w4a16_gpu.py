@@ -147,6 +147,17 @@ def test_kernel_variants(cuda, variant):
     _run_gemv(cuda, 1, 1000, 2048 + 128, 128, "original", variant=variant)
 
 
+@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35])
+@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
+def test_streaming_small_batch_kernel(cuda, variant, mode):
+    """The direct-to-LDS kernel: ragged M and N, a single K step, fewer steps than ring stages, many steps,
+    both layouts."""
+    _run_gemv(cuda, 37, 16 * 13 + 3, 256 * 3, 128, mode, variant=variant)
+    _run_gemv(cuda, 64, 130, 256, 128, mode, variant=variant)
+    _run_gemv(cuda, 5, 64, 256 * 9, 128, mode, variant=variant, interleaved=True)
+    _run_gemv(cuda, 16, 256, 4096, 128, mode, variant=variant)
+
+
 def test_multi_tile_k(cuda):
     """K large enough that the activations are staged in several LDS tiles."""
     _run_gemv(cuda, 16, 256, 8192, 128, "scale")

@@ -13,6 +13,8 @@ static char g_error_buf[kErrorBufSize];
 char* error_buf() { return g_error_buf; }
 
 // kernels (defined in the .hip files next to this one)
+int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                 int mode, int layout, int config, hipStream_t stream);
 int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int variant, hipStream_t stream);
 int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
@@ -67,7 +69,7 @@ extern "C" int init(void) {
     DQ_FAIL("init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
   int max_lds = 0;
   DQ_CHECK_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
-  const int kLargestLdsRequest = 144 * 1024;
+  const int kLargestLdsRequest = 160 * 1024;
   if (kLargestLdsRequest > max_lds)
     DQ_FAIL("Requested dynamic shared memory %d exceeds device limit %d", kLargestLdsRequest, max_lds);
   return 0;
@@ -86,12 +88,25 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   // prefill-sized M: the 256 x 256 MFMA GEMM (same tile-exact decoders)
   if (variant < 0 && M > 64) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread
-  // (r = 0: its own choice).  0..99: a configuration of the MFMA kernel.
+  // (r = 0: its own choice).  30..35: a configuration of the direct-to-LDS small-batch kernel.  0..12: a
+  // configuration of the tiled MFMA kernel (covers every shape).
+  if (variant >= 30 && variant < 40) {
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant - 30, (hipStream_t)stream);
+    if (rc > 0) DQ_FAIL("%s: the streaming small-batch kernel does not cover N=%d K=%d group=%d", fn, N, K, group);
+    return rc;
+  }
   if (variant < 0 || variant >= 100) {
     const int rc = w4a16_gemv_dot2(A, B, Scale, Zeros, C, M, N, K, group, mode, layout,
                                    variant >= 100 ? variant - 100 : 0, (hipStream_t)stream);
     if (rc <= 0) return rc;
     if (variant >= 100) DQ_FAIL("%s: the dot2 GEMV kernel does not cover M=%d K=%d", fn, M, K);
+  }
+  if (variant < 0 && M > 4) {
+    // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
+    const bool wide = N >= 128 * 200;
+    const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : 2);
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, config, (hipStream_t)stream);
+    if (rc <= 0) return rc;
   }
   return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
 }
