@@ -53,7 +53,8 @@ def _time_launches(torch, fns, steps, warmup):
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         if graph is not None:
-            graph.replay()  # untimed replay: warms the instantiated graph
+            for _ in range(3):  # untimed replays: warm the instantiated graph and the clocks
+                graph.replay()
             stream.synchronize()
             e0.record(stream)
             graph.replay()

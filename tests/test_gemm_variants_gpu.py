@@ -17,7 +17,8 @@ def _dev(x, cuda):
     return torch.from_numpy(np.ascontiguousarray(x)).to(cuda)
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (512, 512, 512), (100, 130, 384), (1, 8, 128)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (512, 512, 512), (100, 130, 384), (1, 8, 128),
+                                   (1500, 2000, 256), (3581, 3589, 128)])  # the last two: 128x128 and 256x256 tiles
 def test_w4a8_exact(cuda, M, N, K):
     """examples/dequantize_gemm/example_dequant_gemm_w4a8.py: Ct[N,M] int32, all byte values."""
     d = workloads.int8_int4(M, N, K, seed=M)
@@ -27,7 +28,7 @@ def test_w4a8_exact(cuda, M, N, K):
     np.testing.assert_array_equal(Ct.cpu().numpy(), orc.ref_w4a8(d["A"], d["B"]))
 
 
-@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (16, 16, 128), (300, 200, 256)])
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (16, 16, 128), (300, 200, 256), (1500, 2000, 256), (3584, 3590, 128)])
 def test_int4xint4_exact(cuda, M, N, K):
     """examples/gemm_int4/example_tilelang_gemm_int4.py:70-103: rtol=0, atol=0."""
     d = workloads.int4_int4(M, N, K, seed=K)
@@ -61,7 +62,7 @@ def test_fine_grained(cuda, in_dtype):
 
 
 @pytest.mark.parametrize("transposed", [True, False])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (72, 200, 128)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (72, 200, 128), (1500, 2000, 128), (3581, 3589, 256)])  # last: direct-to-LDS kernel
 def test_fp16_fp4(cuda, transposed, M, N, K):
     """examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py: Ct[N,M] fp16, all byte values."""
     rng = np.random.default_rng(1)
@@ -87,9 +88,10 @@ def test_fp16_fp4_weights_exact(cuda):
 
 @pytest.mark.parametrize("mode", ["scale", "original", "rescale", "signed"])
 @pytest.mark.parametrize("interleaved", [False, True])
-def test_w4a16_large_m(cuda, mode, interleaved):
+@pytest.mark.parametrize("M,N,K", [(200, 320, 512), (1500, 2000, 256), (3581, 3589, 128)])  # 128x64, 128x128, 256x256 tiles
+def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
     """W4A16 through the MFMA GEMM (M > 64): same tile-exact decoders as the decode kernel."""
-    M, N, K, group = 200, 320, 512, 128
+    group = 128
     d = workloads.w4a16(M, N, K, group, seed=2, scale_range=(0.002, 0.01), zeros_range=(6, 10))
     kw = {"scale": dict(source_format="int"), "original": dict(source_format="uint", with_zeros=True),
           "rescale": dict(source_format="uint", with_zeros=True, zeros_mode="rescale"),
@@ -113,7 +115,7 @@ def test_w4a16_large_m(cuda, mode, interleaved):
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384), (1500, 2000, 256), (3590, 3580, 128)])
 def test_bitnet_gemm_int32_exact(cuda, convention, M, N, K):
     """tilelang_bitnet_158_int8xint2_prefill.py:360-381 (256^3, B in {0,1}) generalised to all codes, exact."""
     rng = np.random.default_rng(M + K)

@@ -58,6 +58,16 @@ def test_ragged_shapes(cuda, M, N, K):
     _check(cuda, M, N, K, "e2m1", scale_bias=127)
 
 
+@pytest.mark.parametrize("fmt", ["e2m1", "twiddling", "simple"])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_many_tiles(cuda, fmt, with_bias):
+    """Enough 256 x 256 tiles for the direct-to-LDS kernel (ragged edges, K of 2 and of 5 tiles), and the
+    128 x 128 tile choice below it."""
+    _check(cuda, 3581, 3589, 128, fmt, scale_bias=127, with_bias=with_bias)
+    _check(cuda, 3584, 3584, 320, fmt, scale_bias=0, with_bias=with_bias, exp_range=(0, 4))
+    _check(cuda, 1500, 2000, 192, fmt, scale_bias=127, with_bias=with_bias)
+
+
 @pytest.mark.parametrize("fmt", ["e2m1", "simple"])
 def test_bias(cuda, fmt):
     _check(cuda, 384, 512, 256, fmt, scale_bias=127, with_bias=True)

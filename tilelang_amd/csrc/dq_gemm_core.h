@@ -75,19 +75,20 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 }
 
 // Epilogue shared by both kernel variants (a macro: it uses the kernel's locals).
-// acc[mb][nb][i] = C[m0 + wm*128 + mb*32 + 8*(i/4) + 4*g + i%4][n0 + wn*128 + nb*32 + r].  Staged through
+// acc[mb][nb][i] = C[m0 + (wm*kMBW + mb)*32 + 8*(i/4) + 4*g + i%4][n0 + (wn*kNBW + nb)*32 + r], with kMBW x kNBW
+// blocks of 32 x 32 per wave (constants of the kernel that expands the macro).  Staged through
 // LDS (every tile is consumed: the loop ended with a barrier) so that each lane stores 16 contiguous
 // bytes.  Each wave owns a 32 x (128 + 4) slab of 32-bit values; LDS operations of one wave execute
-// in order, so no workgroup barrier is needed between the phases.
+// in order, so no workgroup barrier is needed between the phases.  Each wave owns a 32 x (32 kNBW + 4) slab.
 #define DQ_GEMM_EPILOGUE \
   using out_t = typename P::out_t; \
-  constexpr int kSlabStride = 132; \
+  constexpr int kSlabStride = 32 * kNBW + 4; \
   constexpr int kOutPerPiece = 16 / sizeof(out_t); \
   uint32_t* slab = reinterpret_cast<uint32_t*>(smem) + wave * (32 * kSlabStride); \
   _Pragma("unroll") \
-  for (int mb = 0; mb < 4; ++mb) { \
+  for (int mb = 0; mb < kMBW; ++mb) { \
   _Pragma("unroll") \
-    for (int nb = 0; nb < 4; ++nb) \
+    for (int nb = 0; nb < kNBW; ++nb) \
   _Pragma("unroll") \
       for (int i = 0; i < 16; ++i) { \
         const int row = 8 * (i >> 2) + 4 * g + (i & 3); \
@@ -98,14 +99,14 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
       } \
     __builtin_amdgcn_wave_barrier(); \
     if constexpr (!P::kTransposed) { \
-      constexpr int kPiecesPerRow = 128 / kOutPerPiece; \
+      constexpr int kPiecesPerRow = 32 * kNBW / kOutPerPiece; \
       constexpr int kIters = 32 * kPiecesPerRow / 64; \
   _Pragma("unroll") \
       for (int it = 0; it < kIters; ++it) { \
         const int q = lane + 64 * it; \
         const int row = q / kPiecesPerRow, piece = q % kPiecesPerRow; \
-        const int m = m0 + wm * 128 + mb * 32 + row; \
-        const int n = n0 + wn * 128 + piece * kOutPerPiece; \
+        const int m = m0 + wm * (32 * kMBW) + mb * 32 + row; \
+        const int n = n0 + wn * (32 * kNBW) + piece * kOutPerPiece; \
         uint32_t raw[kOutPerPiece]; \
   _Pragma("unroll") \
         for (int e = 0; e < kOutPerPiece; e += 4) { \
@@ -130,13 +131,13 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
       } \
     } else { \
       constexpr int kPiecesPerCol = 32 / kOutPerPiece; \
-      constexpr int kIters = 128 * kPiecesPerCol / 64; \
+      constexpr int kIters = 32 * kNBW * kPiecesPerCol / 64; \
   _Pragma("unroll") \
       for (int it = 0; it < kIters; ++it) { \
         const int q = lane + 64 * it; \
         const int col = q / kPiecesPerCol, piece = q % kPiecesPerCol; \
-        const int n = n0 + wn * 128 + col; \
-        const int m = m0 + wm * 128 + mb * 32 + piece * kOutPerPiece; \
+        const int n = n0 + wn * (32 * kNBW) + col; \
+        const int m = m0 + wm * (32 * kMBW) + mb * 32 + piece * kOutPerPiece; \
         if (n < N && m < M) { \
           out_t o[kOutPerPiece]; \
   _Pragma("unroll") \
@@ -171,20 +172,23 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 //   decode(const uint32_t* words, int j, const Scale&)  -> B operand of MFMA step j; `words` are
 //       the lane's kBRowBytes/2 packed bytes as dwords
 //   Epilogue: out_t, kTransposed, finish(acc value, p, m, n) -> value stored
-template <class P>
+template <class P, int kMBW, int kNBW>
 __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int BM = 64 * kMBW, BN = 64 * kNBW;  // 2 x 2 waves of kMBW x kNBW blocks of 32 x 32 (shadow the 256 x 256 default)
+  constexpr int kAStage = BM * kARowBytes;
   constexpr int kBStage = BN * P::kBRowBytes;
   constexpr int kStage = kAStage + kBStage;
   constexpr int kBPiecesPerRow = P::kBRowBytes / 16;           // 2 or 4
-  constexpr int kBLoads = BN * kBPiecesPerRow / kThreads;       // 2 or 4
+  constexpr int kBPieces = BN * kBPiecesPerRow;                 // 16-byte pieces of a packed B tile
+  constexpr int kBLoads = (kBPieces + kThreads - 1) / kThreads;
   constexpr int kBWords = P::kBRowBytes / 8;                    // dwords per lane: 4 or 8
-  constexpr int kALoads = P::kAPacked ? 4 : 8;                  // 16-byte global loads of A per thread
+  constexpr int kALoads = (P::kAPacked ? 4 : 8) * BM / 256;     // 16-byte global loads of A per thread
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves, 128 x 128 each
+  const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves
   const int g = lane >> 5, r = lane & 31;
   const int M = p.M, N = p.N, K = p.K;
 
@@ -218,9 +222,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
   }
   const unsigned char* b_src[kBLoads];
   int b_dst[kBLoads];
+  bool b_on[kBLoads];  // a tile narrower than the workgroup leaves some threads without a piece
 #pragma unroll
   for (int i = 0; i < kBLoads; ++i) {
-    const int q = tid + kThreads * i;
+    const int q0 = tid + kThreads * i;
+    b_on[i] = q0 < kBPieces;
+    const int q = b_on[i] ? q0 : 0;
     const int row = q / kBPiecesPerRow, piece = q % kBPiecesPerRow;
     b_src[i] = (const unsigned char*)p.B + (size_t)min(n0 + row, N - 1) * b_row_bytes + piece * 16;
     // rotate the pieces of a row so that the 16 rows of one ds_read_b128 phase cover all 64 banks
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
     for (int i = 0; i < kALoads; ++i) a_reg[i] = *reinterpret_cast<const uint4_t*>(a_src[i] + (size_t)kb * a_step);
 #pragma unroll
     for (int i = 0; i < kBLoads; ++i)
-      b_reg[i] = *reinterpret_cast<const uint4_t*>(b_src[i] + (size_t)kb * P::kBRowBytes);
+      if (b_on[i]) b_reg[i] = *reinterpret_cast<const uint4_t*>(b_src[i] + (size_t)kb * P::kBRowBytes);
   };
   auto store_tile = [&](int stage) {
     unsigned char* base = smem + stage * kStage;
@@ -250,24 +257,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
       }
     }
 #pragma unroll
-    for (int i = 0; i < kBLoads; ++i) *reinterpret_cast<uint4_t*>(base + b_dst[i]) = b_reg[i];
+    for (int i = 0; i < kBLoads; ++i)
+      if (b_on[i]) *reinterpret_cast<uint4_t*>(base + b_dst[i]) = b_reg[i];
   };
 
   // ---- fragment read offsets -----------------------------------------------------------------
   // A fragment of m-block mb, step j: row wm*128 + mb*32 + r, logical piece g*4 + j
-  int a_row_off[4], a_row_sw[4];
+  int a_row_off[kMBW], a_row_sw[kMBW];
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    const int row = wm * 128 + mb * 32 + r;
+  for (int mb = 0; mb < kMBW; ++mb) {
+    const int row = wm * (32 * kMBW) + mb * 32 + r;
     a_row_off[mb] = row * 128;
     a_row_sw[mb] = a_swz(row);
   }
   // packed B of n-block nb: row wn*128 + nb*32 + r, the half of the row that belongs to group g
-  int b_off[4][kBPiecesPerRow / 2];
-  int w_row[4];
+  int b_off[kNBW][kBPiecesPerRow / 2];
+  int w_row[kNBW];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    const int row = wn * 128 + nb * 32 + r;
+  for (int nb = 0; nb < kNBW; ++nb) {
+    const int row = wn * (32 * kNBW) + nb * 32 + r;
     w_row[nb] = min(n0 + row, N - 1);
 #pragma unroll
     for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
@@ -276,24 +284,24 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
     }
   }
 
-  typename P::acc_t acc[4][4];
+  typename P::acc_t acc[kMBW][kNBW];
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
+  for (int mb = 0; mb < kMBW; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < kNBW; ++nb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
   // ---- fragment readers ---------------------------------------------------------------------
   using frag_t = typename P::frag_t;
-  auto read_a = [&](const unsigned char* base, int j, frag_t (&af)[4]) {
+  auto read_a = [&](const unsigned char* base, int j, frag_t (&af)[kMBW]) {
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < kMBW; ++mb)
       af[mb] = *reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
   };
-  auto read_b = [&](const unsigned char* base, uint32_t (&bw)[4][kBWords]) {
+  auto read_b = [&](const unsigned char* base, uint32_t (&bw)[kNBW][kBWords]) {
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < kNBW; ++nb)
 #pragma unroll
       for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
         const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb][h]);
@@ -307,11 +315,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
   // kb is multiplied out of stage kb%3, and during its last step the first fragments of tile kb+1 are
   // already fetched from stage (kb+1)%3 (written in iteration kb-1): one barrier per iteration and the
   // LDS -> register -> MFMA pipeline never drains.
-  typename P::ScaleRaw sc_raw1[4], sc_raw2[4];  // raw scales of tiles kb+1 and kb+2
-  typename P::Scale sc_c[4], sc_n[4];
+  typename P::ScaleRaw sc_raw1[kNBW], sc_raw2[kNBW];  // raw scales of tiles kb+1 and kb+2
+  typename P::Scale sc_c[kNBW], sc_n[kNBW];
   load_tile(0);
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
+  for (int nb = 0; nb < kNBW; ++nb) {
     sc_c[nb] = P::prep_scale(P::fetch_scale(p, w_row[nb], 0, g), p);
     sc_raw1[nb] = P::fetch_scale(p, w_row[nb], KB > 1 ? 1 : 0, g);
   }
@@ -323,12 +331,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
   if (KB > 2) load_tile(2);
   __syncthreads();
 
-  uint32_t bw_c[4][kBWords], bw_n[4][kBWords];
-  frag_t af_c[4], bf_c[4], af_n[4], bf_n[4];
+  uint32_t bw_c[kNBW][kBWords], bw_n[kNBW][kBWords];
+  frag_t af_c[kMBW], bf_c[kNBW], af_n[kMBW], bf_n[kNBW];
   read_b(smem, bw_c);
   read_a(smem, 0, af_c);
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) bf_c[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
+  for (int nb = 0; nb < kNBW; ++nb) bf_c[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
 
   int stage = 0;
   for (int kb = 0; kb < KB; ++kb) {
@@ -339,7 +347,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
     if (kb + 2 < KB) {
       store_tile(stage2);
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) sc_raw2[nb] = P::fetch_scale(p, w_row[nb], kb + 2, g);
+      for (int nb = 0; nb < kNBW; ++nb) sc_raw2[nb] = P::fetch_scale(p, w_row[nb], kb + 2, g);
     }
     if (kb + 3 < KB) load_tile(kb + 3);
     const bool has_next = kb + 1 < KB;
@@ -350,28 +358,27 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
       if (j < 3) {
         read_a(base, j + 1, af_n);
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
+        for (int nb = 0; nb < kNBW; ++nb) bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
         if (j == 2 && has_next) read_b(base_n, bw_n);
       } else if (has_next) {
         read_a(base_n, 0, af_n);
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
+        for (int nb = 0; nb < kNBW; ++nb) {
           sc_n[nb] = P::prep_scale(sc_raw1[nb], p);
           bf_n[nb] = P::decode(bw_n[nb], 0, sc_n[nb]);
         }
       }
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < kMBW; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = P::mfma(af_c[mb], bf_c[nb], acc[mb][nb]);
+        for (int nb = 0; nb < kNBW; ++nb) acc[mb][nb] = P::mfma(af_c[mb], bf_c[nb], acc[mb][nb]);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        af_c[q] = af_n[q];
-        bf_c[q] = bf_n[q];
-      }
+      for (int q = 0; q < kMBW; ++q) af_c[q] = af_n[q];
+#pragma unroll
+      for (int q = 0; q < kNBW; ++q) bf_c[q] = bf_n[q];
     }
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+    for (int nb = 0; nb < kNBW; ++nb) {
       sc_c[nb] = sc_n[nb];
       sc_raw1[nb] = sc_raw2[nb];
 #pragma unroll
@@ -404,6 +411,7 @@ template <class P>
 __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(P::kBRowBytes == 32, "direct-to-LDS variant: 32 packed bytes per weight row per tile");
+  constexpr int kMBW = 4, kNBW = 4;  // 256 x 256 tile
   constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
   constexpr int kStage = kAStage + kBStage;    // 40 KiB
   constexpr int kStages = 3;
@@ -606,10 +614,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   DQ_GEMM_EPILOGUE
 }
 
-template <class P>
-int launch(const Params& p, hipStream_t stream) {
-  constexpr int kLds = 3 * (kAStage + BN * P::kBRowBytes);
-  auto kern = gemm_kernel<P>;
+template <class P, int kMBW = 4, int kNBW = 4>
+int launch(Params p, hipStream_t stream) {
+  constexpr int kTileM = 64 * kMBW, kTileN = 64 * kNBW;
+  constexpr int kPipe = 3 * (kTileM * kARowBytes + kTileN * P::kBRowBytes);
+  constexpr int kSlabs = 4 * 32 * (32 * kNBW + 4) * 4;  // epilogue staging
+  constexpr int kLds = kPipe > kSlabs ? kPipe : kSlabs;
+  p.tiles_m = (p.M + kTileM - 1) / kTileM;
+  p.tiles_n = (p.N + kTileN - 1) / kTileN;
+  auto kern = gemm_kernel<P, kMBW, kNBW>;
   static bool lds_limit_raised = false;  // once per kernel: legal under stream capture afterwards
   if (!lds_limit_raised) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
@@ -620,9 +633,22 @@ int launch(const Params& p, hipStream_t stream) {
   return 0;
 }
 
+// Tile choice by how many workgroups the 256 CUs get: 256 x 256 when that already gives about one per
+// CU, else 128 x 128, else 128 x 64 (a narrower N tile repeats the weight decode less than a
+// narrower M tile would).
+template <class P>
+int launch_auto(const Params& p, hipStream_t stream) {
+  auto tiles = [&](int bm, int bn) { return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+  if (tiles(256, 256) >= 192) return launch<P, 4, 4>(p, stream);
+  if (tiles(128, 128) >= 192) return launch<P, 2, 2>(p, stream);
+  return launch<P, 2, 1>(p, stream);
+}
+
 template <class P>
 bool dma_eligible(const Params& p) {
-  return (p.K % 128 == 0) && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
+  // the direct-to-LDS kernel has one tile shape (256 x 256): small problems go to the tile-size choice above
+  const long tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  return (p.K % 128 == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
 }
 
 template <class P>

@@ -174,8 +174,8 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
       if (Bias) return gemm::launch_dma<MxPolicy<FMT_, true>>(p, stream);                    \
       return gemm::launch_dma<MxPolicy<FMT_, false>>(p, stream);                             \
     }                                                                                        \
-    if (Bias) return gemm::launch<MxPolicy<FMT_, true>>(p, stream);                          \
-    return gemm::launch<MxPolicy<FMT_, false>>(p, stream);                                   \
+    if (Bias) return gemm::launch_auto<MxPolicy<FMT_, true>>(p, stream);                          \
+    return gemm::launch_auto<MxPolicy<FMT_, false>>(p, stream);                                   \
   } while (0)
   switch (fmt) {
     case FP4_E2M1: DQ_MX(FP4_E2M1);
@@ -192,8 +192,8 @@ int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, in
     if (transposed) return gemm::launch_dma<Fp16Fp4Policy<true>>(p, stream);
     return gemm::launch_dma<Fp16Fp4Policy<false>>(p, stream);
   }
-  if (transposed) return gemm::launch<Fp16Fp4Policy<true>>(p, stream);
-  return gemm::launch<Fp16Fp4Policy<false>>(p, stream);
+  if (transposed) return gemm::launch_auto<Fp16Fp4Policy<true>>(p, stream);
+  return gemm::launch_auto<Fp16Fp4Policy<false>>(p, stream);
 }
 
 int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
@@ -203,8 +203,8 @@ int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void
   p.p1 = K / group;
 #define DQ_W4(MODE_)                                                                        \
   do {                                                                                      \
-    if (layout == LAYOUT_PLAIN) return gemm::launch<W4F16Policy<MODE_, false>>(p, stream);  \
-    return gemm::launch<W4F16Policy<MODE_, true>>(p, stream);                               \
+    if (layout == LAYOUT_PLAIN) return gemm::launch_auto<W4F16Policy<MODE_, false>>(p, stream);  \
+    return gemm::launch_auto<W4F16Policy<MODE_, true>>(p, stream);                               \
   } while (0)
   switch (mode) {
     case W4_UNSIGNED: DQ_W4(W4_UNSIGNED);

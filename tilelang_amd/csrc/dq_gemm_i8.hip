@@ -101,8 +101,8 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
   p.f0 = s_w;
 #define DQ_I2(CONV_)                                                                       \
   do {                                                                                     \
-    if (bitnet_epilogue) return gemm::launch<I2Policy<CONV_, BitnetOut>>(p, stream);       \
-    return gemm::launch<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);                   \
+    if (bitnet_epilogue) return gemm::launch_auto<I2Policy<CONV_, BitnetOut>>(p, stream);       \
+    return gemm::launch_auto<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);                   \
   } while (0)
   switch (convention) {
     case I2_UNSIGNED: DQ_I2(I2_UNSIGNED);
@@ -118,15 +118,15 @@ int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_s
   Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
   if (a_packed) {
     if (!is_signed) DQ_FAIL("int4 gemm: packed A is built for signed int4 only");
-    if (transposed) return gemm::launch<I4Policy<true, true, Int32Out<8, true>>>(p, stream);
-    return gemm::launch<I4Policy<true, true, Int32Out<8, false>>>(p, stream);
+    if (transposed) return gemm::launch_auto<I4Policy<true, true, Int32Out<8, true>>>(p, stream);
+    return gemm::launch_auto<I4Policy<true, true, Int32Out<8, false>>>(p, stream);
   }
   if (is_signed) {
-    if (transposed) return gemm::launch<I4Policy<true, false, Int32Out<4, true>>>(p, stream);
-    return gemm::launch<I4Policy<true, false, Int32Out<4, false>>>(p, stream);
+    if (transposed) return gemm::launch_auto<I4Policy<true, false, Int32Out<4, true>>>(p, stream);
+    return gemm::launch_auto<I4Policy<true, false, Int32Out<4, false>>>(p, stream);
   }
-  if (transposed) return gemm::launch<I4Policy<false, false, Int32Out<0, true>>>(p, stream);
-  return gemm::launch<I4Policy<false, false, Int32Out<0, false>>>(p, stream);
+  if (transposed) return gemm::launch_auto<I4Policy<false, false, Int32Out<0, true>>>(p, stream);
+  return gemm::launch_auto<I4Policy<false, false, Int32Out<0, false>>>(p, stream);
 }
 
 }  // namespace dq
