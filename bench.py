@@ -26,6 +26,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12        # B/s
 MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense
 MFMA_I8_PEAK = 5.0e15    # OP/s dense
+# HBM bytes per launch of the headline GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
+# same counters read for a plain 128 MiB copy kernel (59241.6 x 2 KiB read + 56 KiB written)
+GEMV_HBM_TRAFFIC = 121384141
 
 
 def _time_launches(torch, fns, steps, warmup):
@@ -200,6 +203,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=12)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="skip the per-configuration table")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain elementwise copy of 128 MiB a few times: under `rocprofv3 --pmc FETCH_SIZE` / "
+                         "`WRITE_SIZE` its counters give the factor that turns counter units into bytes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards by output rows N "
@@ -221,7 +227,15 @@ def main():
     us = head["us"]
     gbs = head["bytes"] / (us * 1e-6) / 1e9
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": gbs * 1e9 / HBM_PEAK,
-            "traffic": None, "kernel": "w4a16_gemv_kernel<1,1,4,scale,g128>", "algorithmic_bytes": head["bytes"]}
+            "traffic": GEMV_HBM_TRAFFIC, "kernel": "w4a16_gemv_kernel<1,1,4,scale,g128,wide>", "algorithmic_bytes": head["bytes"]}
+
+    if args.copy_calibration:
+        src = torch.full((128 << 20,), 3, dtype=torch.uint8, device=dev).view(torch.int32)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.add(src, 1, out=dst)  # reads 128 MiB, writes 128 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     shapes = []
     if not args.headline_only:
