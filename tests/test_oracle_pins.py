@@ -2,18 +2,23 @@
 brute force over finite domains, round trips, and reduction to integer / float64 arithmetic."""
 
 import itertools
+import json
+import os
 
 import numpy as np
 import pytest
 
 from oracle import dq_oracle as orc
 
-E2M1 = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0]
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_known_answers.json")) as _f:
+    GOLDEN = json.load(_f)
+E2M1 = GOLDEN["e2m1_value_table"]["values_by_code"]
+assert len(E2M1) == 16
 
 
 # ---- golden vectors from the reference's tests ---------------------------------------------------
 
-@pytest.mark.parametrize("nbit,values", [(2, [-2, -1, 0, 1]), (4, list(range(-8, 8))), (8, [-128, -17, -1, 0, 1, 42, 127])])
+@pytest.mark.parametrize("nbit,values", [(c["nbit"], c["values"]) for c in GOLDEN["signed_subword_decode"]["cases"]])
 def test_sign_extend_known_answers(nbit, values):
     """testing/python/issue/test_tilelang_u32_signed_decode.py:26-30: pack (value & mask) << (pos * nbit), decode."""
     mask = (1 << nbit) - 1
@@ -33,11 +38,12 @@ def test_sign_extend_known_answers(nbit, values):
 
 def test_e2m1_encode_pack_known_answer():
     """testing/python/quantize/test_tilelang_quantize_nvfp4_scale_layout.py:881-887."""
-    values = np.array([[0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.5, -1.0]], dtype=np.float32)
+    kat = GOLDEN["e2m1_encode_pack"]
+    values = np.array([kat["values"]], dtype=np.float32)
     codes = orc.encode_fp4_e2m1_values(values)
-    assert codes.tolist() == [[0x0, 0x1, 0x2, 0x3, 0x4, 0x5, 0x6, 0x7, 0x9, 0xA]]
+    assert codes.tolist() == [kat["codes"]]
     packed = orc.pack_fp4_e2m1_codes(codes)
-    assert packed.tolist() == [[0x10, 0x32, 0x54, 0x76, 0xA9]]
+    assert packed.tolist() == [kat["packed_low_nibble_first"]]
     np.testing.assert_array_equal(orc.decode_fp4_e2m1(packed), values)
 
 
