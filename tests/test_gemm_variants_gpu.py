@@ -115,7 +115,8 @@ def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384), (1500, 2000, 256), (3590, 3580, 128)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384), (1500, 2000, 256), (3590, 3580, 128),
+                                   (3590, 3580, 768)])  # the last one: direct-to-LDS kernel
 def test_bitnet_gemm_int32_exact(cuda, convention, M, N, K):
     """tilelang_bitnet_158_int8xint2_prefill.py:360-381 (256^3, B in {0,1}) generalised to all codes, exact."""
     rng = np.random.default_rng(M + K)

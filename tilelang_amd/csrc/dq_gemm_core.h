@@ -392,8 +392,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
 }
 
 // ---- direct-to-LDS variant ---------------------------------------------------------------------
-// For policies whose A needs no transform (P::kPlainA) and whose scales are either absent or one
-// byte per 32 k (P::kScaleBytes): the A and packed-B tiles, and the scale bytes, travel
+// For policies whose A needs no transform on its way to LDS (any per-fragment transform is P::fix_a,
+// applied after the fragment is read) and whose scales are either absent or one byte per 32 k
+// (P::kScaleBytes): the A and packed-B tiles, and the scale bytes, travel
 // global -> LDS with global_load_lds_dwordx4 / _dword, two tiles ahead of the MFMAs, without
 // passing through registers.  A lane's 16 bytes land at LDS base + lane * 16 whatever its source
 // address, so the XOR swizzle of the A rows is applied by permuting the SOURCE addresses.  These
@@ -437,13 +438,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   for (int i = 0; i < 8; ++i) {
     const int c = (wave * 8 + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
     const int row = c >> 3, pp = c & 7;
-    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * 2) + (unsigned)((pp ^ a_swz(row)) << 4);
+    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * (kARowBytes / P::kKPerBlock)) + (unsigned)((pp ^ a_swz(row)) << 4);
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int c = (wave * 2 + i) * 64 + lane;  // B chunk: row c / 2, physical piece c % 2
     const int row = c >> 1, pp = c & 1;
-    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K >> 1) + (unsigned)(((pp + (row >> 3)) & 1) << 4);
+    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K * P::kBRowBytes / P::kKPerBlock) + (unsigned)(((pp + (row >> 3)) & 1) << 4);
   }
   const unsigned s_voff = (unsigned)min(n0 + tid, N - 1) * (unsigned)(K >> 5);
 
@@ -484,7 +485,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   }
   using frag_t = typename P::frag_t;
   auto read_a1 = [&](const unsigned char* base, int j, int mb) -> frag_t {
-    return *reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4));
+    return P::fix_a(*reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4)));
   };
   auto read_b1 = [&](const unsigned char* base, int nb, uint32_t (&bw)[kBWords]) {
     const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb]);
@@ -648,7 +649,7 @@ template <class P>
 bool dma_eligible(const Params& p) {
   // the direct-to-LDS kernel has one tile shape (256 x 256): small problems go to the tile-size choice above
   const long tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  return (p.K % 128 == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
+  return (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
 }
 
 template <class P>
@@ -689,6 +690,9 @@ struct PlainA {
   static constexpr bool kPlainA = true;  // stage_a is the identity: A may go global -> LDS directly
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return v; }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
+  // direct-to-LDS kernel: transform of an A fragment after it is read from LDS (A lands untouched)
+  template <class F>
+  __device__ static __forceinline__ F fix_a(F f) { return f; }
 };
 
 }  // namespace gemm

@@ -50,6 +50,13 @@ struct I2Policy : I8Mfma, gemm::NoScale, EPI {
   static constexpr bool kAPacked = false;
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return transpose4x4_bytes(v); }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
+  // direct-to-LDS kernel: A lands in LDS untouched and each 16-byte fragment is transposed after the read
+  static constexpr bool kScaleBytes = false;
+  __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
+  using gemm::NoScale::prep_scale;
+  __device__ static __forceinline__ frag_t fix_a(frag_t f) {
+    return __builtin_bit_cast(frag_t, transpose4x4_bytes(__builtin_bit_cast(uint4_t, f)));
+  }
   __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
     frag_t o;
 #pragma unroll
@@ -101,8 +108,12 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
   p.f0 = s_w;
 #define DQ_I2(CONV_)                                                                       \
   do {                                                                                     \
-    if (bitnet_epilogue) return gemm::launch_auto<I2Policy<CONV_, BitnetOut>>(p, stream);       \
-    return gemm::launch_auto<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);                   \
+    if (gemm::dma_eligible<I2Policy<CONV_, BitnetOut>>(p)) {                               \
+      if (bitnet_epilogue) return gemm::launch_dma<I2Policy<CONV_, BitnetOut>>(p, stream); \
+      return gemm::launch_dma<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);             \
+    }                                                                                      \
+    if (bitnet_epilogue) return gemm::launch_auto<I2Policy<CONV_, BitnetOut>>(p, stream);  \
+    return gemm::launch_auto<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);              \
   } while (0)
   switch (convention) {
     case I2_UNSIGNED: DQ_I2(I2_UNSIGNED);
