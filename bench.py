@@ -56,7 +56,7 @@ def _time_launches(torch, fns, steps, warmup):
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         if graph is not None:
-            for _ in range(3):  # untimed replays: warm the instantiated graph and the clocks
+            for _ in range(10):  # untimed replays: warm the instantiated graph and let the clocks settle
                 graph.replay()
             stream.synchronize()
             e0.record(stream)
@@ -199,7 +199,7 @@ def cpu_baseline_w4a16(N, K, rows, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=60)
+    ap.add_argument("--steps", type=int, default=240)
     ap.add_argument("--warmup", type=int, default=12)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="skip the per-configuration table")

@@ -102,8 +102,27 @@ __global__ __launch_bounds__(256) void w4a16_gemv_kernel(const half_t* __restric
     goff[p] = (uint32_t)(slot * groups_per_row + (G128 ? (chunk >> 2) : ((chunk << 5) >> gshift))) * 2u;
   }
 
+  // One row per pass, four row groups, group size 128: the four lanes of a quad share their scale
+  // group, so lane l fetches the scale (zero) of row (l & 3) of the batch for all four of them and
+  // the batch needs one scale load per lane instead of four.
+  constexpr bool kPack = WIDE && R == 4 && G128 && HAS_SCALE;
+  uint32_t pack_off[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) pack_off[p] = (uint32_t)(min(p * tpr + ct, c16 - 1) >> 2) * 2u;
+  unsigned short sc_pack[NP], zp_pack[NP];
+
   uint4_t bq[R][NP];
   half_t sc[R][NP], zp[R][NP];
+  auto issue_pack = [&](int b) {
+    const int row = min(row0 + b * R + (lane & 3), N - 1);
+    const uint8_t* sp = reinterpret_cast<const uint8_t*>(S) + (size_t)row * groups_per_row * 2;
+    const uint8_t* zq = reinterpret_cast<const uint8_t*>(Z) + (size_t)row * groups_per_row * 2;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      sc_pack[p] = *reinterpret_cast<const unsigned short*>(sp + pack_off[p]);
+      if constexpr (HAS_ZEROS) zp_pack[p] = *reinterpret_cast<const unsigned short*>(zq + pack_off[p]);
+    }
+  };
   auto issue_group = [&](int u, int b) {
     // groups past N (N is a multiple of rpp) are clamped to the last one and dropped at the store
     const int rb = min(row0 + (b * R + u) * rpp, N - rpp);
@@ -113,8 +132,11 @@ __global__ __launch_bounds__(256) void w4a16_gemv_kernel(const half_t* __restric
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       bq[u][p] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(bp + boff[p]));
-      if constexpr (HAS_SCALE) sc[u][p] = *reinterpret_cast<const half_t*>(sp + goff[p]);
-      if constexpr (HAS_ZEROS) zp[u][p] = *reinterpret_cast<const half_t*>(zq + goff[p]);
+      if constexpr (HAS_SCALE && !kPack) sc[u][p] = *reinterpret_cast<const half_t*>(sp + goff[p]);
+      if constexpr (HAS_ZEROS && !kPack) zp[u][p] = *reinterpret_cast<const half_t*>(zq + goff[p]);
+    }
+    if constexpr (kPack) {
+      if (u == 0) issue_pack(b);
     }
   };
 
@@ -159,6 +181,23 @@ __global__ __launch_bounds__(256) void w4a16_gemv_kernel(const half_t* __restric
   auto process_batch = [&](int b, auto refill_tag) {
     constexpr bool kRefill = decltype(refill_tag)::value;
     float acc[NV];
+    if constexpr (kPack) {
+      // hand every lane of a quad the scale of each of the four rows (quad_perm broadcast of lane u)
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+        const int s32 = sc_pack[p], z32 = HAS_ZEROS ? zp_pack[p] : 0;
+        const int sb[4] = {__builtin_amdgcn_update_dpp(0, s32, 0x00, 0xF, 0xF, true), __builtin_amdgcn_update_dpp(0, s32, 0x55, 0xF, 0xF, true),
+                           __builtin_amdgcn_update_dpp(0, s32, 0xAA, 0xF, 0xF, true), __builtin_amdgcn_update_dpp(0, s32, 0xFF, 0xF, 0xF, true)};
+#pragma unroll
+        for (int u = 0; u < R; ++u) sc[u][p] = __builtin_bit_cast(half_t, (unsigned short)sb[u & 3]);
+        if constexpr (HAS_ZEROS) {
+          const int zb[4] = {__builtin_amdgcn_update_dpp(0, z32, 0x00, 0xF, 0xF, true), __builtin_amdgcn_update_dpp(0, z32, 0x55, 0xF, 0xF, true),
+                             __builtin_amdgcn_update_dpp(0, z32, 0xAA, 0xF, 0xF, true), __builtin_amdgcn_update_dpp(0, z32, 0xFF, 0xF, 0xF, true)};
+#pragma unroll
+          for (int u = 0; u < R; ++u) zp[u][p] = __builtin_bit_cast(half_t, (unsigned short)zb[u & 3]);
+        }
+      }
+    }
 #pragma unroll
     for (int u = 0; u < R; ++u) {
 #pragma unroll
