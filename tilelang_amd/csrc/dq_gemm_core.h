@@ -34,6 +34,10 @@
 #define DQ_SWZ_SHIFT 1
 #endif
 
+#ifndef DQ_DMA_MBW
+#define DQ_DMA_MBW 4  // wave tile rows / 32 of the direct-to-LDS kernel (2 = 128 x 256 tiles, two workgroups per CU)
+#endif
+
 namespace dq {
 namespace gemm {
 
@@ -408,13 +412,21 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
 
-template <class P>
-__global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
+// kMBW = 4: 256 x 256 tile, one workgroup per CU (the default).  kMBW = 2: 128 x 256 tile, two
+// workgroups per CU (76 KiB of LDS and 256 registers each) that fill each other's barrier stalls;
+// measured 13 % slower on the 4096 x 8192 x 8192 MXFP4 problem (twice the decode work per MFMA,
+// and the 256-register budget spills), so it is kept as a build option only.
+template <class P, int kMBW>
+__global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(P::kBRowBytes == 32, "direct-to-LDS variant: 32 packed bytes per weight row per tile");
-  constexpr int kMBW = 4, kNBW = 4;  // 256 x 256 tile
+  static_assert(kMBW == 2 || kMBW == 4, "wave tile of 64 or 128 rows");
+  constexpr int kNBW = 4;
+  constexpr int BM = 64 * kMBW;                // shadows the 256-row default
+  constexpr int kAStage = BM * kARowBytes;     // 32 or 16 KiB
+  constexpr int kAOps = 2 * kMBW;              // A DMA instructions per wave per tile
   constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
-  constexpr int kStage = kAStage + kBStage;    // 40 KiB
+  constexpr int kStage = kAStage + kBStage;    // 40 or 24 KiB
   constexpr int kStages = 3;
   constexpr int kRing = kStages * kStage;      // scale ring: 4 slots x 1 KiB (256 rows x 4 scale bytes = 2 tiles)
   constexpr int kBWords = 4;
@@ -433,10 +445,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   const unsigned lds0 = (unsigned)(size_t)smem;  // LDS byte address of the dynamic segment
 
   // ---- per-lane source offsets: LDS chunk c (16 bytes) of a tile <- which global 16 bytes --------
-  unsigned a_voff[8], b_voff[2];
+  unsigned a_voff[kAOps], b_voff[2];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int c = (wave * 8 + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
+  for (int i = 0; i < kAOps; ++i) {
+    const int c = (wave * kAOps + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
     const int row = c >> 3, pp = c & 7;
     a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * (kARowBytes / P::kKPerBlock)) + (unsigned)((pp ^ a_swz(row)) << 4);
   }
@@ -448,10 +460,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   }
   const unsigned s_voff = (unsigned)min(n0 + tid, N - 1) * (unsigned)(K >> 5);
 
-  // One tile = 11 DMA instructions per thread: op 0 the scale dword (rows tid, tiles 2p and 2p+1; issued
-  // with every tile, i.e. twice per pair, which keeps the loop branch-free), ops 1..8 the A chunks, ops
-  // 9..10 the packed-B chunks.
-  constexpr int kTileOps = 11;
+  // One tile = 3 + kAOps DMA instructions per thread: op 0 the scale dword (rows tid, tiles 2p and 2p+1;
+  // issued with every tile, i.e. twice per pair, which keeps the loop branch-free), then the A chunks,
+  // then the two packed-B chunks.
+  constexpr int kTileOps = 3 + kAOps;
   auto issue_op = [&](int op, int kb, int stage) {
     const unsigned sbase = lds0 + stage * kStage;
     if (op == 0) {
@@ -459,21 +471,21 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
         const int pair = kb >> 1;
         dma4(lds0 + kRing + (pair & 3) * 1024 + wave * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
       }
-    } else if (op <= 8) {
+    } else if (op <= kAOps) {
       const int i = op - 1;
-      dma16(sbase + (wave * 8 + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
+      dma16(sbase + (wave * kAOps + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
     } else {
-      const int i = op - 9;
+      const int i = op - 1 - kAOps;
       dma16(sbase + kAStage + (wave * 2 + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * 32);
     }
   };
   constexpr int kWaitOps = P::kScaleBytes ? kTileOps : kTileOps - 1;  // outstanding DMA instructions of one tile
 
   // ---- fragment read offsets (same LDS geometry as the register-staged kernel) --------------------
-  int a_row_off[4], a_row_sw[4], b_off[4], s_off[4];
+  int a_row_off[kMBW], a_row_sw[kMBW], b_off[4], s_off[4];
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    const int row = wm * 128 + mb * 32 + r;
+  for (int mb = 0; mb < kMBW; ++mb) {
+    const int row = wm * (32 * kMBW) + mb * 32 + r;
     a_row_off[mb] = row * 128;
     a_row_sw[mb] = a_swz(row);
   }
@@ -497,9 +509,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
     return P::prep_scale(e, p);
   };
 
-  typename P::acc_t acc[4][4];
+  typename P::acc_t acc[kMBW][4];
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
+  for (int mb = 0; mb < kMBW; ++mb)
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
@@ -515,7 +527,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
 
   typename P::Scale sc_c[4];
   uint32_t bw_c[4][kBWords];
-  frag_t af_c[4], bf_c[4], af_n[4], bf_n[4];
+  frag_t af_c[kMBW], bf_c[4], af_n[kMBW], bf_n[4];
 
   // One iteration = tile kb out of `stage`, as 16 chunks of 4 MFMAs (one A fragment against the four
   // B fragments) kept in order by scheduling barriers; every chunk carries side work that issues in
@@ -534,24 +546,39 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
     const int stage2 = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3
     const unsigned char* base = smem + stage * kStage;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (q == 0) {
+    for (int q = 0; q < kMBW; ++q) {
+      if constexpr (kMBW == 4) {
+        if (q == 0) {
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-          read_b1(base, nb, bw_c[nb]);
-          sc_c[nb] = read_scale1(kb, nb);
+          for (int nb = 0; nb < 4; ++nb) {
+            read_b1(base, nb, bw_c[nb]);
+            sc_c[nb] = read_scale1(kb, nb);
+          }
+        } else if (q == 1) {
+          af_n[0] = read_a1(base, 0, 0);
+          af_n[1] = read_a1(base, 0, 1);
+        } else if (q == 2) {
+          af_n[2] = read_a1(base, 0, 2);
+          af_n[3] = read_a1(base, 0, 3);
+          bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]);
+          bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]);
+        } else {
+          bf_n[2] = P::decode(bw_c[2], 0, sc_c[2]);
+          bf_n[3] = P::decode(bw_c[3], 0, sc_c[3]);
         }
-      } else if (q == 1) {
-        af_n[0] = read_a1(base, 0, 0);
-        af_n[1] = read_a1(base, 0, 1);
-      } else if (q == 2) {
-        af_n[2] = read_a1(base, 0, 2);
-        af_n[3] = read_a1(base, 0, 3);
-        bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]);
-        bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]);
       } else {
-        bf_n[2] = P::decode(bw_c[2], 0, sc_c[2]);
-        bf_n[3] = P::decode(bw_c[3], 0, sc_c[3]);
+        if (q == 0) {
+#pragma unroll
+          for (int nb = 0; nb < 4; ++nb) {
+            read_b1(base, nb, bw_c[nb]);
+            sc_c[nb] = read_scale1(kb, nb);
+          }
+          af_n[0] = read_a1(base, 0, 0);
+          af_n[1] = read_a1(base, 0, 1);
+        } else {
+#pragma unroll
+          for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
+        }
       }
       if (has_next2) issue_op(q, kb + 2, stage2);
       if (!first) {
@@ -561,27 +588,29 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      af_c[q] = af_n[q];
-      bf_c[q] = bf_n[q];
-    }
+    for (int q = 0; q < kMBW; ++q) af_c[q] = af_n[q];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) bf_c[q] = bf_n[q];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int chunk = 4 + j * 4 + q;
+      for (int q = 0; q < kMBW; ++q) {
+        const int chunk = kMBW + j * kMBW + q;
         af_n[q] = read_a1(base, j + 1, q);
-        bf_n[q] = P::decode(bw_c[q], j + 1, sc_c[q]);
+#pragma unroll
+        for (int e = 0; e < 4 / kMBW; ++e) {
+          const int nb = q * (4 / kMBW) + e;
+          bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
+        }
         if (has_next2 && chunk < kTileOps) issue_op(chunk, kb + 2, stage2);
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        af_c[q] = af_n[q];
-        bf_c[q] = bf_n[q];
-      }
+      for (int q = 0; q < kMBW; ++q) af_c[q] = af_n[q];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bf_c[q] = bf_n[q];
     }
     // tile kb+1 must have landed before the next iteration reads it; tile kb+2 (issued during this
     // iteration) may still be in flight
@@ -608,7 +637,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel_dma(const Params p) {
   }
   // step 3 of the last tile
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
+  for (int q = 0; q < kMBW; ++q)
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
 
@@ -652,10 +681,12 @@ bool dma_eligible(const Params& p) {
   return (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
 }
 
-template <class P>
-int launch_dma(const Params& p, hipStream_t stream) {
-  constexpr int kLds = 3 * (kAStage + BN * P::kBRowBytes) + 4 * 1024;
-  auto kern = gemm_kernel_dma<P>;
+template <class P, int kMBW>
+int launch_dma_tile(Params p, hipStream_t stream) {
+  constexpr int kLds = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + 4 * 1024;
+  p.tiles_m = (p.M + 64 * kMBW - 1) / (64 * kMBW);
+  p.tiles_n = (p.N + BN - 1) / BN;
+  auto kern = gemm_kernel_dma<P, kMBW>;
   static bool lds_limit_raised = false;
   if (!lds_limit_raised) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
@@ -664,6 +695,11 @@ int launch_dma(const Params& p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(kThreads), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
+}
+
+template <class P>
+int launch_dma(const Params& p, hipStream_t stream) {
+  return launch_dma_tile<P, DQ_DMA_MBW>(p, stream);
 }
 
 inline Params make_params(const void* A, const void* B, const void* S, const void* Z, const void* Bias, void* C, int M,
