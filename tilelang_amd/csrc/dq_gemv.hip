@@ -314,7 +314,7 @@ int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, 
   int r = rows_hint & 15, nb = rows_hint >> 4;
   if (r == 0) r = (((long)N / (4 * rpp)) >= 1024 ? 4 : 2);
   if (r != 2 && r != 4) r = 2;
-  if (r * np * mrows > 8) r = 2;  // keep registers bounded
+  if (r * np * mrows > 16) r = 2;  // keep registers bounded
   if (r * mrows > 16) return 1;
   if (nb == 0) {
     const long wgs1 = ((long)N + r * rpp - 1) / (r * rpp);
