@@ -47,7 +47,8 @@ enum dq_w4_mode {
 
 enum dq_w4_layout {
   DQ_LAYOUT_PLAIN = 0,      /* nibble e of each 32-bit word is element e                         */
-  DQ_LAYOUT_INTERLEAVED = 1 /* words pre-permuted by interleave_weight(.., 4, "float16"),
+  DQ_LAYOUT_INTERLEAVED = 1 /* words pre-permuted by interleave_weight (.., 4, "float16") for uint4,
+                               (.., 2, "int8") for 2-bit codes,
                                examples/dequantize_gemm/quantize/utils.py:71-125              */
 };
 
@@ -111,11 +112,14 @@ enum dq_i2_convention {
 
 /* int8 x 2-bit: C[M,N] = A[M,K] int8 . decode(B[N,K/4])^T, exact int32 accumulation.  out_kind 0: C is
  * int32.  out_kind 1: C is fp16 = (float(acc) / s_a[m]) / s_w, the BitLinear epilogue
- * (examples/bitnet-1.58b/utils_quant.py:165-170), s_a fp32 [M].  B is the plain layout: byte j holds
- * codes 4j..4j+3 at bits 0,2,4,6.  Replaces `call(A, B, C, stream)` of examples/bitnet-1.58b/
- * kernel_benchmark/tilelang_bitnet_158_int8xint2_prefill.py:188-296.  Requires K % 128 == 0. */
-int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a,
-                        float s_w, int out_kind, dq_stream_t stream);
+ * (examples/bitnet-1.58b/utils_quant.py:165-170), s_a fp32 [M].  layout DQ_LAYOUT_PLAIN: byte j holds
+ * codes 4j..4j+3 at bits 0,2,4,6; DQ_LAYOUT_INTERLEAVED: every 32-bit word pre-permuted by
+ * interleave_weight(qw, 2, "int8"), which is what the reference's kernels are fed
+ * (examples/bitnet-1.58b/kernel_benchmark/tilelang_bitnet_158_int8xint2_decode.py:196-234,249-251).
+ * Replaces `call(A, B, C, stream)` of tilelang_bitnet_158_int8xint2_prefill.py:188-296 and
+ * tilelang_bitnet_158_int8xint2_decode.py:66-175.  Requires K % 128 == 0. */
+int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout,
+                        const void* s_a, float s_w, int out_kind, dq_stream_t stream);
 
 /* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T.
  * is_signed 1: two's-complement nibbles (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:10-21,

@@ -117,26 +117,34 @@ def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384), (1500, 2000, 256), (3590, 3580, 128),
                                    (3590, 3580, 768)])  # the last one: direct-to-LDS kernel
-def test_bitnet_gemm_int32_exact(cuda, convention, M, N, K):
-    """tilelang_bitnet_158_int8xint2_prefill.py:360-381 (256^3, B in {0,1}) generalised to all codes, exact."""
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_bitnet_gemm_int32_exact(cuda, convention, M, N, K, interleaved):
+    """tilelang_bitnet_158_int8xint2_prefill.py:360-381 (256^3, B in {0,1}) generalised to all codes, exact;
+    with the weights interleaved as the reference feeds them (fast_decoding) and plain."""
     rng = np.random.default_rng(M + K)
     A = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
     B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
     C = torch.zeros((M, N), dtype=torch.int32, device=cuda)
-    tl.bitnet_158_int8xint2_prefill(M, N, K, convention=convention)(_dev(A, cuda), _dev(B, cuda).view(torch.int8), C)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 2, "int8")
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention=convention)(_dev(A, cuda), Bdev, C)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
 
 
-def test_bitnet_reference_example_inputs(cuda):
-    """The reference's own check: A in [0,4), B in {0,1} compressed with general_compress (no interleave here)."""
-    M = N = K = 256
+@pytest.mark.parametrize("M", [256, 1])
+def test_bitnet_reference_example_inputs(cuda, M):
+    """The reference's own check, with its own call sequence (prefill.py:360-381 at 256^3, decode.py:237-258 at
+    1x256x256): A in [0,4), B in {0,1}, general_compress then interleave_weight(qw, 2, int8), default arguments."""
+    N = K = 256
     torch.manual_seed(42)
     A = torch.randint(0, 4, (M, K), dtype=torch.int8)
     W = torch.randint(0, 2, (N, K), dtype=torch.int8)
-    qw = quantize.general_compress(W, source_bits=2)
+    qw = quantize.interleave_weight(quantize.general_compress(W, source_bits=2), 2, "int8")
     C = torch.zeros((M, N), dtype=torch.int32, device=cuda)
-    tl.bitnet_158_int8xint2_prefill(M, N, K)(A.to(cuda), qw.to(cuda), C)
+    factory = tl.bitnet_158_int8xint2_prefill if M > 1 else tl.bitnet_158_int8xint2_decode
+    factory(M, N, K, "int8", "int32", "int32")(A.to(cuda), qw.to(cuda), C)
     torch.cuda.synchronize()
     ref = torch.matmul(A.float(), W.float().T).to(torch.int32)
     assert torch.equal(C.cpu(), ref)
@@ -149,11 +157,14 @@ def test_bitlinear_config5(cuda, M):
     N = K = 1024
     d = workloads.bitnet(M, N, K, seed=M)
     out = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]))(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["s_a"], cuda))
+    Bil = quantize.interleave_weight(_dev(d["B"], cuda).view(torch.int8), 2, "int8")
+    out_il = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), interleaved=True)(_dev(d["A"], cuda), Bil, _dev(d["s_a"], cuda))
     torch.cuda.synchronize()
     ref = orc.ref_bitnet(d["A"], d["B"], d["s_a"], d["s_w"], "offset")
     np.testing.assert_allclose(out.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+    assert torch.equal(out, out_il)
     acc = torch.zeros((M, N), dtype=torch.int32, device=cuda)
-    tl.bitnet_158_int8xint2_prefill(M, N, K, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), acc)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=False, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), acc)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(acc.cpu().numpy(), d["A"].astype(np.int64) @ d["W"].astype(np.int64).T)
 
@@ -164,7 +175,7 @@ def test_bitnet_full_size_checksum(cuda):
     M, N, K = 2048, 8192, 8192
     d = workloads.bitnet(M, N, K, seed=0)
     acc = torch.zeros((M, N), dtype=torch.int32, device=cuda)
-    tl.bitnet_158_int8xint2_prefill(M, N, K, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), acc)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=False, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), acc)
     torch.cuda.synchronize()
     got = acc.cpu().numpy().astype(np.int64)
     wsum = d["W"].astype(np.int64).sum(axis=0)
@@ -176,13 +187,17 @@ def test_bitnet_full_size_checksum(cuda):
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
 @pytest.mark.parametrize("M,N,K", [(1, 256, 256), (1, 1000, 8192), (2, 130, 4096), (3, 64, 2048), (4, 4096, 8192), (1, 96, 16384), (2, 40, 16384)])
-def test_bitnet_decode_gemv_exact(cuda, convention, M, N, K):
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_bitnet_decode_gemv_exact(cuda, convention, M, N, K, interleaved):
     """tilelang_bitnet_158_int8xint2_decode.py:237-258 (1x256x256) generalised: all codes, int8 range, exact."""
     rng = np.random.default_rng(M * 7 + K)
     A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
     B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
     C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
-    tl.bitnet_158_int8xint2_decode(M, N, K, convention=convention)(_dev(A, cuda), _dev(B, cuda).view(torch.int8), C)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 2, "int8")
+    tl.bitnet_158_int8xint2_decode(M, N, K, fast_decoding=interleaved, convention=convention)(_dev(A, cuda), Bdev, C)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
 
@@ -192,7 +207,7 @@ def test_bitnet_decode_full_size(cuda):
     M, N, K = 1, 8192, 8192
     d = workloads.bitnet(M, N, K, seed=1)
     C = torch.zeros((M, N), dtype=torch.int32, device=cuda)
-    tl.bitnet_158_int8xint2_decode(M, N, K, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), C)
+    tl.bitnet_158_int8xint2_decode(M, N, K, fast_decoding=False, convention="offset")(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), C)
     out = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]))(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["s_a"], cuda))
     torch.cuda.synchronize()
     ref = d["A"].astype(np.int64) @ d["W"].astype(np.int64).T

@@ -28,10 +28,10 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
 int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream);
 int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                 int mode, int layout, hipStream_t stream);
-int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
-            int bitnet_epilogue, hipStream_t stream);
-int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
-            int out_kind, hipStream_t stream);
+int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
+            float s_w, int bitnet_epilogue, hipStream_t stream);
+int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
+            float s_w, int out_kind, hipStream_t stream);
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
             hipStream_t stream);
 
@@ -164,18 +164,19 @@ extern "C" int call_dequant_gemm_w4_fp16(const void* A, const void* B, const voi
 }
 
 extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention,
-                                   const void* s_a, float s_w, int out_kind, dq_stream_t stream) {
+                                   int layout, const void* s_a, float s_w, int out_kind, dq_stream_t stream) {
   const char* fn = "call_gemm_int8xint2";
   if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
   if (convention < I2_UNSIGNED || convention > I2_TWOS) DQ_FAIL("%s: unknown code convention %d", fn, convention);
+  if (layout != LAYOUT_PLAIN && layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
   if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
   if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);
   if (out_kind == 1 && !(s_w != 0.f)) DQ_FAIL("%s: s_w must be non-zero", fn);
   if (M <= 4) {  // decode: the streaming dot4 kernel
-    const int rc = i2_gemv(A, B, C, M, N, K, convention, s_a, s_w, out_kind, (hipStream_t)stream);
+    const int rc = i2_gemv(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
-  return i2_gemm(A, B, C, M, N, K, convention, s_a, s_w, out_kind, (hipStream_t)stream);
+  return i2_gemm(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
 }
 
 extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed,

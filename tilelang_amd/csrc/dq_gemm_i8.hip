@@ -43,19 +43,24 @@ struct BitnetOut {
 };
 
 // ---- int8 x 2-bit ---------------------------------------------------------------------------------
-// packed byte j of a row holds codes 4j..4j+3 at bits 0, 2, 4, 6.
-template <int CONV, class EPI>
+// Plain layout: packed byte j of a row holds codes 4j..4j+3 at bits 0, 2, 4, 6; (w >> 2i) & 0x03030303
+// then yields elements (i, 4+i, 8+i, 12+i) of a 16-code word, and A is transposed to match.
+// INTERLEAVED: words pre-permuted by interleave_weight(qw, 2, "int8") (examples/bitnet-1.58b/
+// kernel_benchmark/tilelang_bitnet_158_int8xint2_decode.py:196-234: element e at byte e % 4, slot
+// e / 4), the layout the reference's kernels consume; the same shift-and-mask yields elements
+// 4i..4i+3 in natural order and A needs no transform.
+template <int CONV, class EPI, bool INTERLEAVED>
 struct I2Policy : I8Mfma, gemm::NoScale, EPI {
   static constexpr int kBRowBytes = 32;
   static constexpr bool kAPacked = false;
-  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return transpose4x4_bytes(v); }
+  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : transpose4x4_bytes(v); }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
   // direct-to-LDS kernel: A lands in LDS untouched and each 16-byte fragment is transposed after the read
   static constexpr bool kScaleBytes = false;
   __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
   using gemm::NoScale::prep_scale;
   __device__ static __forceinline__ frag_t fix_a(frag_t f) {
-    return __builtin_bit_cast(frag_t, transpose4x4_bytes(__builtin_bit_cast(uint4_t, f)));
+    return INTERLEAVED ? f : __builtin_bit_cast(frag_t, transpose4x4_bytes(__builtin_bit_cast(uint4_t, f)));
   }
   __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
     frag_t o;
@@ -102,18 +107,23 @@ struct I4Policy : I8Mfma, gemm::NoScale, EPI {
 
 }  // namespace
 
-int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
-            int bitnet_epilogue, hipStream_t stream) {
+int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
+            float s_w, int bitnet_epilogue, hipStream_t stream) {
   Params p = gemm::make_params(A, B, s_a, nullptr, nullptr, C, M, N, K);
   p.f0 = s_w;
-#define DQ_I2(CONV_)                                                                       \
-  do {                                                                                     \
-    if (gemm::dma_eligible<I2Policy<CONV_, BitnetOut>>(p)) {                               \
-      if (bitnet_epilogue) return gemm::launch_dma<I2Policy<CONV_, BitnetOut>>(p, stream); \
-      return gemm::launch_dma<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);             \
-    }                                                                                      \
-    if (bitnet_epilogue) return gemm::launch_auto<I2Policy<CONV_, BitnetOut>>(p, stream);  \
-    return gemm::launch_auto<I2Policy<CONV_, Int32Out<0, false>>>(p, stream);              \
+#define DQ_I2L(CONV_, IL_)                                                                      \
+  do {                                                                                          \
+    if (gemm::dma_eligible<I2Policy<CONV_, BitnetOut, IL_>>(p)) {                               \
+      if (bitnet_epilogue) return gemm::launch_dma<I2Policy<CONV_, BitnetOut, IL_>>(p, stream); \
+      return gemm::launch_dma<I2Policy<CONV_, Int32Out<0, false>, IL_>>(p, stream);             \
+    }                                                                                           \
+    if (bitnet_epilogue) return gemm::launch_auto<I2Policy<CONV_, BitnetOut, IL_>>(p, stream);  \
+    return gemm::launch_auto<I2Policy<CONV_, Int32Out<0, false>, IL_>>(p, stream);              \
+  } while (0)
+#define DQ_I2(CONV_)                                        \
+  do {                                                      \
+    if (layout == LAYOUT_INTERLEAVED) DQ_I2L(CONV_, true);  \
+    DQ_I2L(CONV_, false);                                   \
   } while (0)
   switch (convention) {
     case I2_UNSIGNED: DQ_I2(I2_UNSIGNED);
@@ -122,6 +132,7 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
     default: DQ_FAIL("int2 gemm: unknown code convention %d", convention);
   }
 #undef DQ_I2
+#undef DQ_I2L
 }
 
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,

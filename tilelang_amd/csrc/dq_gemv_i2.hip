@@ -34,7 +34,7 @@ template <int MROWS, int NP, int R>
 __global__ __launch_bounds__(256) void i2_gemv_kernel(const int8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                        void* __restrict__ C, const float* __restrict__ s_a, float s_w,
                                                        int out_kind, int M, int N, int K, int tpr_shift, int nb,
-                                                       uint32_t flip_mask, int zsub) {
+                                                       uint32_t flip_mask, int zsub, int interleaved) {
   __shared__ int red[kMaxRowsPerWg * 4 * MROWS];
 
   const int tid = threadIdx.x;
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void i2_gemv_kernel(const int8_t* __restrict__
       for (int j = 0; j < 4; ++j) {
         uint4_t d = *reinterpret_cast<const uint4_t*>(ap + j * 16);
         if (!valid) d = uint4_t{0u, 0u, 0u, 0u};
-        d = transpose4x4_bytes(d);
+        if (!interleaved) d = transpose4x4_bytes(d);  // interleaved words decode to natural order
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           a[p][m][j * 4 + i] = d[i];
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void i2_gemv_kernel(const int8_t* __restrict__
 
 template <int MROWS, int NP>
 int launch_i2_gemv(const void* A, const void* B, void* C, const void* s_a, float s_w, int out_kind, int M, int N, int K,
-                   int tpr_shift, uint32_t flip, int zsub, hipStream_t stream) {
+                   int tpr_shift, uint32_t flip, int zsub, int interleaved, hipStream_t stream) {
   constexpr int R = 4 / NP;
   const int rpp = 256 >> tpr_shift;
   const long wgs1 = ((long)N + R * rpp - 1) / (R * rpp);
@@ -166,7 +166,7 @@ int launch_i2_gemv(const void* A, const void* B, void* C, const void* s_a, float
   const int rows_per_wg = nb * R * rpp;
   hipLaunchKernelGGL((i2_gemv_kernel<MROWS, NP, R>), dim3((N + rows_per_wg - 1) / rows_per_wg), dim3(256), 0, stream,
                      (const int8_t*)A, (const uint8_t*)B, C, (const float*)s_a, s_w, out_kind, M, N, K, tpr_shift, nb,
-                     flip, zsub);
+                     flip, zsub, interleaved);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }
@@ -174,8 +174,9 @@ int launch_i2_gemv(const void* A, const void* B, void* C, const void* s_a, float
 }  // namespace
 
 // Returns 1 when this kernel does not cover the shape (caller uses the MFMA GEMM).
-int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, const void* s_a, float s_w,
-            int out_kind, hipStream_t stream) {
+int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
+            float s_w, int out_kind, hipStream_t stream) {
+  const int interleaved = layout == LAYOUT_INTERLEAVED;
   if (M > 4 || K % 64 != 0) return 1;
   const int c16 = K / 64;
   int tpr_shift = 5;
@@ -189,11 +190,11 @@ int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int conv
   int zsub = 0;
   if (convention == I2_OFFSET) zsub = 2;
   else if (convention == I2_TWOS) { flip = 0xAAAAAAAAu; zsub = 2; }
-  if (mrows == 1 && np == 1) return launch_i2_gemv<1, 1>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, stream);
-  if (mrows == 1 && np == 2) return launch_i2_gemv<1, 2>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, stream);
-  if (mrows == 2 && np == 1) return launch_i2_gemv<2, 1>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, stream);
-  if (mrows == 2 && np == 2) return launch_i2_gemv<2, 2>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, stream);
-  if (mrows == 4 && np == 1) return launch_i2_gemv<4, 1>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, stream);
+  if (mrows == 1 && np == 1) return launch_i2_gemv<1, 1>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, interleaved, stream);
+  if (mrows == 1 && np == 2) return launch_i2_gemv<1, 2>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, interleaved, stream);
+  if (mrows == 2 && np == 1) return launch_i2_gemv<2, 1>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, interleaved, stream);
+  if (mrows == 2 && np == 2) return launch_i2_gemv<2, 2>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, interleaved, stream);
+  if (mrows == 4 && np == 1) return launch_i2_gemv<4, 1>(A, B, C, s_a, s_w, out_kind, M, N, K, tpr_shift, flip, zsub, interleaved, stream);
   return 1;
 }
 

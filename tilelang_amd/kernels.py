@@ -420,8 +420,9 @@ def bitnet_158_int8xint2_prefill(
     """BitNet W2A8 GEMM: ``C[M,N] int32 = A[M,K] int8 @ decode(B[N,K/4]).T``, exact; ``kernel(A, B, C)``.
 
     Same arguments as ``bitnet_158_int8xint2_prefill`` of examples/bitnet-1.58b/kernel_benchmark/
-    tilelang_bitnet_158_int8xint2_prefill.py:72-85.  B is the plain packing (``general_compress(W, 2)``,
-    no ``interleave_weight``).  ``convention``: ``"unsigned"`` (what the example's kernel decodes),
+    tilelang_bitnet_158_int8xint2_prefill.py:72-85.  As there, ``fast_decoding=True`` takes B as
+    ``interleave_weight(general_compress(W, 2), 2, "int8")`` (:372-374); ``fast_decoding=False`` takes the plain
+    packing ``general_compress(W, 2)``.  ``convention``: ``"unsigned"`` (what the example's kernel decodes),
     ``"offset"`` (``w = c - 2``, ternary weights stored as ``w + 2``) or ``"twos"``.
     """
     if _dtype(in_dtype) != torch.int8 or _dtype(out_dtype) != torch.int32:
@@ -429,20 +430,22 @@ def bitnet_158_int8xint2_prefill(
     if K % 128 != 0:
         raise ValueError(f"bitnet_158_int8xint2_prefill: K={K} must be a multiple of 128")
     conv = _I2_CONVENTIONS[convention]
+    layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
     params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 4), packed=True),
               KernelParam("C", torch.int32, (M, N))]
 
     def launch(ptrs, stream):
-        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, None, 1.0, 0, stream)
+        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, layout, None, 1.0, 0, stream)
 
     return KernelAdapter("bitnet_158_int8xint2_prefill", params, [], launch, _lib.last_error)
 
 
-def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "offset") -> KernelAdapter:
+def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "offset", interleaved: bool = False) -> KernelAdapter:
     """BitLinear forward after activation quantisation: ``out[M,N] fp16 = ((A int8 @ W.T) / s_a[m]) / s_w``.
 
     The matmul plus ``post_quant_process`` of examples/bitnet-1.58b/utils_quant.py:165-170,199-209 in one
     kernel.  ``out = kernel(A, B, s_a)`` with ``s_a`` fp32 ``[M]`` (the per-row activation scale).
+    ``interleaved``: B went through ``interleave_weight(.., 2, "int8")``.
     """
     if K % 128 != 0:
         raise ValueError(f"bitlinear_int8xint2: K={K} must be a multiple of 128")
@@ -451,7 +454,8 @@ def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "o
               KernelParam("s_a", torch.float32, (M,)), KernelParam("out", torch.float16, (M, N))]
 
     def launch(ptrs, stream):
-        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv, ptrs[2], float(s_w), 1, stream)
+        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv,
+                                                      LAYOUT_INTERLEAVED if interleaved else LAYOUT_PLAIN, ptrs[2], float(s_w), 1, stream)
 
     return KernelAdapter("bitlinear_int8xint2", params, [-1], launch, _lib.last_error)
 
@@ -472,7 +476,7 @@ def bitnet_158_int8xint2_decode(
 
     Same arguments as ``bitnet_158_int8xint2_decode`` of examples/bitnet-1.58b/kernel_benchmark/
     tilelang_bitnet_158_int8xint2_decode.py:66-76.  M <= 4 runs the streaming dot4 kernel, larger M the
-    MFMA GEMM.  B is the plain packing (no ``interleave_weight``); ``convention`` as in
+    MFMA GEMM.  ``fast_decoding`` (B interleaved or plain) and ``convention`` as in
     :func:`bitnet_158_int8xint2_prefill`.
     """
     k = bitnet_158_int8xint2_prefill(M, N, K, in_dtype, out_dtype, accum_dtype, fast_decoding, convention=convention)
