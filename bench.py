@@ -137,6 +137,23 @@ def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev):
     return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
 
 
+def bench_activation_quant(torch, tl, M, K, steps, warmup, dev):
+    """BitLinear activation quantiser (fp16 rows -> int8 + fp32 scale), the step before the W2A8 GEMM."""
+    nc = _copies(3 * M * K, hi=12)
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    xs = [torch.randn((M, K), generator=gen, dtype=torch.float32).to(torch.float16).to(dev) for _ in range(nc)]
+    kern = tl.bitnet_activation_quant(M, K)
+    out = [None]
+
+    def mk(i):
+        def f():
+            out[0] = kern(xs[i], skip_tensor_validation=True)
+        return f
+
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
+    return {"us": ms * 1e3, "bytes": 3 * M * K + 4 * M, "flops": 2 * M * K, "graph": graphed}
+
+
 def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev):
     """W4A8 (int8 x int4, Ct[N,M] int32) or int4 x int4 (C[M,N] int32), exact."""
     if a_packed:
@@ -255,6 +272,8 @@ def main():
         for m in (1, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, k if m == 1 else kg, 2, dev)
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        r = bench_activation_quant(torch, tl, 2048, 8192, k, 2, dev)
+        shapes.append(_row("bitnet_activation_quant M=2048 K=8192", r, "hbm", MFMA_I8_PEAK))
         r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, False, kg, 2, dev)
         shapes.append(_row("w4a8_gemm M=4096 N=4096 K=4096 (Ct int32)", r, "mfma", MFMA_I8_PEAK))
         r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, True, kg, 2, dev)

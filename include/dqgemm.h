@@ -121,6 +121,12 @@ enum dq_i2_convention {
 int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout,
                         const void* s_a, float s_w, int out_kind, dq_stream_t stream);
 
+/* BitLinear activation quantiser (the caller-side step before call_gemm_int8xint2): per row of X[M,K] fp16,
+ * S[m] = (1 / max(max_k |x|, 1e-5)) * 127 in fp32 (torch's `Qp / tensor` = reciprocal, then product) and Q[m,k] = clamp(round_half_even(float(x) * S[m]), -128, 127) int8,
+ * bit-identical to BitLinearBitBLAS.activation_quant (examples/bitnet-1.58b/utils_quant.py:156-163), which it
+ * replaces.  Requires K % 8 == 0. */
+int call_bitnet_activation_quant(const void* X, void* Q, void* S, int M, int K, dq_stream_t stream);
+
 /* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T.
  * is_signed 1: two's-complement nibbles (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:10-21,
  * `call(A, B, Ct)` :109-147); 0: unsigned nibbles (example_dequant_gemm_fine_grained.py int8 path).

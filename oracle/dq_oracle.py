@@ -535,11 +535,17 @@ def weight_quant(weight: np.ndarray):
 
 
 def activation_quant(x: np.ndarray, num_bits: int = 8):
-    """Per-row int8 activations.  Follows examples/bitnet-1.58b/utils_quant.py:156-163.  Returns (x_q, s[M,1])."""
+    """Per-row int8 activations.  Follows examples/bitnet-1.58b/utils_quant.py:156-163.  Returns (x_q, s[M,1]).
+
+    ``Qp / tensor`` with a Python scalar on the left is torch's ``Tensor.__rtruediv__``, i.e.
+    ``tensor.reciprocal() * Qp``: two fp32 roundings, not one division (pinned against torch's own ops on the
+    CPU in tests/test_oracle_pins.py).
+    """
     xf = np.asarray(x, dtype=np.float32)
     qn, qp = -(2 ** (num_bits - 1)), 2 ** (num_bits - 1) - 1
-    s = np.float32(qp) / np.maximum(np.abs(xf).max(axis=-1, keepdims=True), np.float32(1e-5))
-    return np.clip(np.rint(xf * s), qn, qp).astype(np.int8), s.astype(np.float32)
+    amax = np.maximum(np.abs(xf).max(axis=-1, keepdims=True), np.float32(1e-5)).astype(np.float32)
+    s = ((np.float32(1.0) / amax).astype(np.float32) * np.float32(qp)).astype(np.float32)
+    return np.clip(np.rint(xf * s), qn, qp).astype(np.int8), s
 
 
 def post_quant_process(acc: np.ndarray, si: np.ndarray, sw) -> np.ndarray:

@@ -1,0 +1,52 @@
+"""GPU parity of the BitLinear caller path: activation quantiser (bit-exact) and the module's forward."""
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from tilelang_amd import bitlinear
+from oracle import dq_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,K", [(1, 128), (3, 8192), (64, 1024), (257, 4096), (5, 8 * 37)])
+def test_activation_quant_bit_exact(cuda, M, K):
+    """examples/bitnet-1.58b/utils_quant.py:156-163: int8 codes and fp32 scales identical to the restatement."""
+    rng = np.random.default_rng(M * 131 + K)
+    x = (rng.standard_normal((M, K), dtype=np.float32) * rng.uniform(0.01, 30.0, size=(M, 1)).astype(np.float32)).astype(np.float16)
+    x[0, : min(K, 16)] = np.array([0.5, -0.5, 1.5, 2.5, -2.5, 0.0, 1e-4, -1e-4] * 2, dtype=np.float16)[: min(K, 16)]  # ties
+    if M > 2:
+        x[2, :] = 0  # all-zero row: the 1e-5 clamp decides the scale
+    xq, s = tl.bitnet_activation_quant(M, K)(torch.from_numpy(x).to(cuda))
+    torch.cuda.synchronize()
+    ref_q, ref_s = orc.activation_quant(x)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), ref_s.reshape(-1).view(np.uint32))
+    np.testing.assert_array_equal(xq.cpu().numpy(), ref_q)
+    # and against torch's own ops, the way the reference computes it
+    tq, ts = bitlinear.activation_quant_reference(torch.from_numpy(x))
+    assert torch.equal(xq.cpu(), tq) and torch.equal(s.cpu(), ts.reshape(-1))
+
+
+@pytest.mark.parametrize("interleave", [True, False])
+@pytest.mark.parametrize("batch", [(1,), (7,), (2, 130)])
+def test_bitlinear_forward(cuda, interleave, batch):
+    """Module forward against forward_fp32_simulated of utils_quant.py:189-205 restated with the oracle."""
+    in_f, out_f = 1024, 768
+    rng = np.random.default_rng(len(batch) * 17 + int(interleave))
+    W = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
+    bias = rng.standard_normal(out_f).astype(np.float16)
+    x = rng.standard_normal(batch + (in_f,), dtype=np.float32).astype(np.float16)
+
+    layer = tl.BitLinear(in_f, out_f, interleave=interleave).to(cuda)
+    layer.load_float_weight(torch.from_numpy(W), torch.from_numpy(bias))
+    out = layer(torch.from_numpy(x).to(cuda))
+    torch.cuda.synchronize()
+    assert out.shape == batch + (out_f,) and out.dtype == torch.float16
+
+    wq, sw = orc.weight_quant(W)
+    xq, sa = orc.activation_quant(x.reshape(-1, in_f))
+    acc = xq.astype(np.int64) @ wq.astype(np.int64).T
+    ref = orc.post_quant_process(acc, sa, sw).astype(np.float32) + bias.astype(np.float32)[None, :]
+    np.testing.assert_allclose(out.float().cpu().numpy().reshape(-1, out_f), ref, rtol=1e-2, atol=1e-2)

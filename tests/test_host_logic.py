@@ -56,6 +56,38 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     assert "multiple of 64" in lib.get_last_error().decode()
     assert lib.call_dequant_gemm_bf16_mxfp4(a, a, a, vp(0), a, 64, 64, 128, 16, 0, 127, vp(0)) == -1
     assert "scale_size" in lib.get_last_error().decode()
+    assert lib.call_gemm_int8xint2(a, a, a, 8, 64, 256, 0, 7, vp(0), 1.0, 0, vp(0)) == -1
+    assert "unknown weight layout" in lib.get_last_error().decode()
+    assert lib.call_gemm_int8xint2(a, a, a, 8, 64, 256, 5, 0, vp(0), 1.0, 0, vp(0)) == -1
+    assert "unknown code convention" in lib.get_last_error().decode()
+    assert lib.call_bitnet_activation_quant(a, a, vp(0), 4, 256, vp(0)) == -1
+    assert "S is expected to have non-NULL" in lib.get_last_error().decode()
+    assert lib.call_bitnet_activation_quant(a, a, a, 4, 100, vp(0)) == -1
+    assert "multiple of 8" in lib.get_last_error().decode()
+
+
+def test_bitlinear_weight_packing_matches_oracle():
+    """BitLinear.load_float_weight: ternary codes w + 2, four per byte, interleaved for the fast decoder; decoding
+    the packed buffer with the oracle gives back weight_quant(W) (utils_quant.py:149-154)."""
+    import numpy as np
+    from oracle import dq_oracle as orc
+    from tilelang_amd import bitlinear
+
+    rng = np.random.default_rng(3)
+    W = (rng.standard_normal((48, 256), dtype=np.float32) * 0.05).astype(np.float32)
+    wq_ref, sw_ref = orc.weight_quant(W)
+    assert torch.equal(bitlinear.weight_quant(torch.from_numpy(W)), torch.from_numpy(wq_ref))
+    for interleave in (False, True):
+        layer = bitlinear.BitLinear(256, 48, interleave=interleave)
+        layer.load_float_weight(torch.from_numpy(W))
+        packed = layer.qweight.numpy().view(np.uint8)
+        if interleave:
+            words = np.ascontiguousarray(packed).view(np.uint32)
+            dec = orc.fast_decode_i2_to_i8(words, signed=True).reshape(48, 256)
+        else:
+            dec = orc.decode_i2(packed, "offset")
+        np.testing.assert_array_equal(dec, wq_ref)
+        assert abs(float(layer.sw) - float(sw_ref)) <= 1e-6 * float(sw_ref)
 
 
 # ---- adapter ----------------------------------------------------------------------------------------

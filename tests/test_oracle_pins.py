@@ -267,6 +267,22 @@ def test_ref_mxfp4_exact_scaling_and_identity():
     np.testing.assert_array_equal(W0, orc.decode_fp4_e2m1(B) * 4)
 
 
+def test_activation_quant_matches_torch_ops():
+    """utils_quant.py:156-163 executed with torch's own CPU ops (the reference's statements verbatim in
+    tilelang_amd.bitlinear.activation_quant_reference): scales bit-identical, codes identical, ties included."""
+    import torch
+    from tilelang_amd import bitlinear
+
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((96, 1024), dtype=np.float32) * rng.uniform(0.01, 30.0, size=(96, 1)).astype(np.float32)).astype(np.float16)
+    x[0, :8] = np.array([0.5, -0.5, 1.5, 2.5, -2.5, 0.0, 1e-4, -1e-4], dtype=np.float16)
+    x[1, :] = 0
+    q, s = orc.activation_quant(x)
+    tq, ts = bitlinear.activation_quant_reference(torch.from_numpy(x))
+    np.testing.assert_array_equal(s.view(np.uint32), ts.numpy().view(np.uint32))
+    np.testing.assert_array_equal(q, tq.numpy())
+
+
 def test_bitlinear_quantisers_and_epilogue():
     rng = np.random.default_rng(5)
     x = rng.standard_normal((3, 16)).astype(np.float32) * 3

@@ -10,6 +10,7 @@ from .adapter import KernelAdapter, KernelParam  # noqa: F401
 from .kernels import (  # noqa: F401
     bitlinear_int8xint2,
     bitnet_158_int8xint2_decode,
+    bitnet_activation_quant,
     bitnet_158_int8xint2_prefill,
     dequantize_gemv,
     dequantize_w4,
@@ -20,6 +21,7 @@ from .kernels import (  # noqa: F401
     matmul_w4_fine_grained,
     matmul_w4a16,
 )
+from .bitlinear import BitLinear  # noqa: F401
 from .profiler import Profiler, TensorSupplyType, do_bench  # noqa: F401
 
 __version__ = "0.1.0"

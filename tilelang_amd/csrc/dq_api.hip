@@ -32,6 +32,7 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int bitnet_epilogue, hipStream_t stream);
 int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int out_kind, hipStream_t stream);
+int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
             hipStream_t stream);
 
@@ -177,6 +178,17 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
     if (rc <= 0) return rc;
   }
   return i2_gemm(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+}
+
+extern "C" int call_bitnet_activation_quant(const void* X, void* Q, void* S, int M, int K, dq_stream_t stream) {
+  const char* fn = "call_bitnet_activation_quant";
+  if (!X) DQ_FAIL("%s: X is expected to have non-NULL data pointer", fn);
+  if (!Q) DQ_FAIL("%s: Q is expected to have non-NULL data pointer", fn);
+  if (!S) DQ_FAIL("%s: S is expected to have non-NULL data pointer", fn);
+  if (M <= 0 || K <= 0) DQ_FAIL("%s: M and K must be positive (got %d, %d)", fn, M, K);
+  if (K % 8 != 0) DQ_FAIL("%s: K=%d must be a multiple of 8", fn, K);
+  if (!aligned16(X) || ((uintptr_t)Q & 7) != 0) DQ_FAIL("%s: X must be 16-byte and Q 8-byte aligned", fn);
+  return activation_quant(X, Q, S, M, K, (hipStream_t)stream);
 }
 
 extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed,

@@ -460,6 +460,24 @@ def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "o
     return KernelAdapter("bitlinear_int8xint2", params, [-1], launch, _lib.last_error)
 
 
+def bitnet_activation_quant(M: int, K: int) -> KernelAdapter:
+    """BitLinear activation quantiser: ``x_q, s = kernel(x)`` with ``x`` fp16 ``[M, K]``, ``x_q`` int8 ``[M, K]``,
+    ``s`` fp32 ``[M]``: ``s = 127 / max(|x|.max(-1), 1e-5)``, ``x_q = clamp(round(x.float() * s), -128, 127)``.
+
+    One fused kernel for ``BitLinearBitBLAS.activation_quant`` of examples/bitnet-1.58b/utils_quant.py:156-163
+    (there ``s`` is ``[M, 1]``); bit-identical results.
+    """
+    if K % 8 != 0:
+        raise ValueError(f"bitnet_activation_quant: K={K} must be a multiple of 8")
+    params = [KernelParam("x", torch.float16, (M, K)), KernelParam("x_q", torch.int8, (M, K)),
+              KernelParam("s", torch.float32, (M,))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_bitnet_activation_quant(ptrs[0], ptrs[1], ptrs[2], M, K, stream)
+
+    return KernelAdapter("bitnet_activation_quant", params, [1, 2], launch, _lib.last_error)
+
+
 def bitnet_158_int8xint2_decode(
     M: int,
     N: int,
