@@ -11,7 +11,7 @@ from oracle import dq_oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("M,K", [(1, 128), (3, 8192), (64, 1024), (257, 4096), (5, 8 * 37)])
+@pytest.mark.parametrize("M,K", [(1, 128), (3, 8192), (64, 1024), (257, 4096), (5, 8 * 37), (2, 16384), (2, 16384 + 2048), (1500, 512)])
 def test_activation_quant_bit_exact(cuda, M, K):
     """examples/bitnet-1.58b/utils_quant.py:156-163: int8 codes and fp32 scales identical to the restatement."""
     rng = np.random.default_rng(M * 131 + K)
