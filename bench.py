@@ -27,8 +27,8 @@ HBM_PEAK = 8.0e12        # B/s
 MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense
 MFMA_I8_PEAK = 5.0e15    # OP/s dense
 # HBM bytes per launch of the headline GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
-# same counters read for a plain 128 MiB copy kernel (59241.6 x 2 KiB read + 56 KiB written)
-GEMV_HBM_TRAFFIC = 121384141
+# same counters read for a plain 128 MiB copy kernel (59240.5 x 2 KiB read + 56 KiB written)
+GEMV_HBM_TRAFFIC = 121381888
 
 
 def _time_launches(torch, fns, steps, warmup):
