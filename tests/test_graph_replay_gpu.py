@@ -1,0 +1,70 @@
+"""HIP graph capture of the entry points: the library never allocates or synchronises and sets kernel attributes
+only on a kernel's first (eager) launch, so its launches can be captured; every replay must reproduce the eager
+result bit for bit."""
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from tilelang_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(x, cuda):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(cuda)
+
+
+def test_graph_replays_match_eager(cuda):
+    M1, N1, K1 = 1, 2048, 4096
+    d1 = workloads.w4a16(M1, N1, K1, 128, seed=1)
+    gemv = tl.dequantize_gemv(M1, N1, K1, group_size=128, source_format="int", with_scaling=True)
+    A1, B1, S1 = _dev(d1["A"], cuda), _dev(d1["B"], cuda).view(torch.int8), _dev(d1["Scale"], cuda)
+    C1 = torch.empty((M1, N1), dtype=torch.float16, device=cuda)
+
+    M2, N2, K2 = 16, 1024, 2048
+    d2 = workloads.w4a16(M2, N2, K2, 128, seed=2, zeros_range=(6, 10))
+    batch = tl.dequantize_gemv(M2, N2, K2, group_size=128, source_format="uint", with_scaling=True, with_zeros=True)
+    A2, B2, S2, Z2 = _dev(d2["A"], cuda), _dev(d2["B"], cuda).view(torch.int8), _dev(d2["Scale"], cuda), _dev(d2["Zeros"], cuda)
+    C2 = torch.empty((M2, N2), dtype=torch.float16, device=cuda)
+
+    M3, N3, K3 = 256, 512, 512
+    d3 = workloads.mxfp4(M3, N3, K3, seed=3, scale_bias=127)
+    gemm = tl.matmul_bf16_mxfp4(M3, N3, K3, weight_format="e2m1", scale_bias=127)
+    A3, B3, S3 = _dev(d3["A"], cuda).view(torch.bfloat16), _dev(d3["B"], cuda), _dev(d3["Scale"], cuda)
+    bias = torch.empty((M3, N3), dtype=torch.bfloat16, device=cuda)
+
+    M4, N4, K4 = 8, 512, 1024
+    d4 = workloads.bitnet(M4, N4, K4, seed=4)
+    quant = tl.bitnet_activation_quant(M4, K4)
+    lin = tl.bitlinear_int8xint2(M4, N4, K4, float(d4["s_w"]))
+    X4 = torch.randn((M4, K4), dtype=torch.float16, device=cuda)
+    B4 = _dev(d4["B"], cuda).view(torch.int8)
+
+    def run():
+        gemv(A1, B1, S1, C1)
+        batch(A2, B2, S2, Z2, C2)
+        c3 = gemm(A3, B3, S3, bias)
+        xq, sa = quant(X4)
+        return c3, lin(xq, B4, sa)
+
+    c3_e, o4_e = run()  # eager: first launches set the kernel attributes
+    torch.cuda.synchronize()
+    eager = [C1.clone(), C2.clone(), c3_e.clone(), o4_e.clone()]
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            c3_g, o4_g = run()
+    for _ in range(3):
+        C1.fill_(float("nan"))
+        C2.fill_(float("nan"))
+        c3_g.fill_(float("nan"))
+        o4_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip([C1, C2, c3_g, o4_g], eager):
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
