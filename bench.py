@@ -225,8 +225,8 @@ def main():
                          "`WRITE_SIZE` its counters give the factor that turns counter units into bytes")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards by output rows N "
-                 "with no communication, see DESIGN.md)")
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path would shard by output rows N, "
+                 "each GPU holding its rows of the weights and a replica of the activations, with no communication)")
 
     import torch
 
