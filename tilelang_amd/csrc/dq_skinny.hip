@@ -249,7 +249,7 @@ __global__ void w4_dequant_kernel(const uint8_t* __restrict__ B, const half_t* _
   }
 }
 
-template <int MB, int RB, int WAVES, int U, bool ALL_MODES>
+template <int MB, int RB, int WAVES, int U>
 int launch_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                   int mode, int layout, int KT, hipStream_t stream) {
   const dim3 grid((N + RB * 16 - 1) / (RB * 16), (M + 16 * MB - 1) / (16 * MB));
@@ -281,25 +281,15 @@ int launch_skinny(const void* A, const void* B, const void* S, const void* Z, vo
     if (layout == LAYOUT_PLAIN) DQ_LAUNCH(MODE_, true); \
     else DQ_LAUNCH(MODE_, false);             \
   } while (0)
-  if constexpr (ALL_MODES) {
-    switch (mode) {
-      case W4_UNSIGNED: DQ_LAUNCH_MODE(W4_UNSIGNED); break;
-      case W4_SIGNED: DQ_LAUNCH_MODE(W4_SIGNED); break;
-      case W4_OFFSET8: DQ_LAUNCH_MODE(W4_OFFSET8); break;
-      case W4_SCALE: DQ_LAUNCH_MODE(W4_SCALE); break;
-      case W4_USCALE: DQ_LAUNCH_MODE(W4_USCALE); break;
-      case W4_ZEROS_ORIGINAL: DQ_LAUNCH_MODE(W4_ZEROS_ORIGINAL); break;
-      case W4_ZEROS_RESCALE: DQ_LAUNCH_MODE(W4_ZEROS_RESCALE); break;
-      default: DQ_FAIL("w4a16: unknown mode %d", mode);
-    }
-  } else {
-    // tuning variants: the two modes of the measured configurations, plain layout only
-    if (layout != LAYOUT_PLAIN) DQ_FAIL("w4a16: kernel variant supports the plain layout only");
-    switch (mode) {
-      case W4_SCALE: DQ_LAUNCH(W4_SCALE, true); break;
-      case W4_ZEROS_ORIGINAL: DQ_LAUNCH(W4_ZEROS_ORIGINAL, true); break;
-      default: DQ_FAIL("w4a16: kernel variant supports modes SCALE and ZEROS_ORIGINAL only (got %d)", mode);
-    }
+  switch (mode) {
+    case W4_UNSIGNED: DQ_LAUNCH_MODE(W4_UNSIGNED); break;
+    case W4_SIGNED: DQ_LAUNCH_MODE(W4_SIGNED); break;
+    case W4_OFFSET8: DQ_LAUNCH_MODE(W4_OFFSET8); break;
+    case W4_SCALE: DQ_LAUNCH_MODE(W4_SCALE); break;
+    case W4_USCALE: DQ_LAUNCH_MODE(W4_USCALE); break;
+    case W4_ZEROS_ORIGINAL: DQ_LAUNCH_MODE(W4_ZEROS_ORIGINAL); break;
+    case W4_ZEROS_RESCALE: DQ_LAUNCH_MODE(W4_ZEROS_RESCALE); break;
+    default: DQ_FAIL("w4a16: unknown mode %d", mode);
   }
 #undef DQ_LAUNCH_MODE
 #undef DQ_LAUNCH
@@ -334,24 +324,15 @@ int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, voi
   }
   const size_t budget = 72 * 1024;
   switch (variant) {
-#define DQ_V(ID, MB_, RB_, W_, U_, ALL_)                                                                  \
+#define DQ_V(ID, MB_, RB_, W_, U_)                                                                  \
   case ID:                                                                                                \
-    return launch_skinny<MB_, RB_, W_, U_, ALL_>(A, B, S, Z, C, M, N, K, group, mode, layout,             \
+    return launch_skinny<MB_, RB_, W_, U_>(A, B, S, Z, C, M, N, K, group, mode, layout,             \
                                                  pick_kt(M < 16 * MB_ ? M : 16 * MB_, K, budget), stream)
-    //   id  MB RB  W  U  all-modes
-    DQ_V(0, 1, 1, 4, 8, true);
-    DQ_V(1, 1, 1, 1, 8, false);
-    DQ_V(2, 1, 1, 2, 8, false);
-    DQ_V(3, 1, 2, 4, 4, false);
-    DQ_V(4, 2, 2, 4, 4, true);
-    DQ_V(5, 4, 4, 4, 2, true);
-    DQ_V(6, 1, 1, 4, 4, false);
-    DQ_V(7, 1, 1, 8, 8, false);
-    DQ_V(8, 1, 1, 8, 4, false);
-    DQ_V(9, 1, 2, 8, 4, false);
-    DQ_V(10, 1, 4, 4, 2, true);
-    DQ_V(11, 1, 1, 16, 4, false);
-    DQ_V(12, 1, 1, 8, 2, false);
+    //   id  MB RB  W  U
+    DQ_V(0, 1, 1, 4, 8);
+    DQ_V(4, 2, 2, 4, 4);
+    DQ_V(5, 4, 4, 4, 2);
+    DQ_V(10, 1, 4, 4, 2);
 #undef DQ_V
     default: DQ_FAIL("w4a16: unknown kernel variant %d", variant);
   }
