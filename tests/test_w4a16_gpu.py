@@ -158,6 +158,16 @@ def test_streaming_small_batch_kernel(cuda, variant, mode):
     _run_gemv(cuda, 16, 256, 4096, 128, mode, variant=variant)
 
 
+@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
+@pytest.mark.parametrize("M", [1, 4, 9, 16])
+def test_register_resident_kernel(cuda, M, mode, variant=40):
+    """Activations resident in registers (M <= 16, K = 2048 / 4096 / 8192): one row block per workgroup and
+    several, both layouts."""
+    _run_gemv(cuda, M, 16 * 37, 4096, 128, mode, variant=variant)
+    _run_gemv(cuda, M, 48, 8192, 128, mode, variant=variant, interleaved=(mode in ("scale", "original")))
+    _run_gemv(cuda, M, 16 * 600, 2048, 128, mode, variant=variant)  # more row blocks than workgroups
+
+
 def test_multi_tile_k(cuda):
     """K large enough that the activations are staged in several LDS tiles."""
     _run_gemv(cuda, 16, 256, 8192, 128, "scale")

@@ -13,6 +13,8 @@ static char g_error_buf[kErrorBufSize];
 char* error_buf() { return g_error_buf; }
 
 // kernels (defined in the .hip files next to this one)
+int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                 int mode, int layout, hipStream_t stream);
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, hipStream_t stream);
 int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
@@ -89,8 +91,15 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   // prefill-sized M: the 256 x 256 MFMA GEMM (same tile-exact decoders)
   if (variant < 0 && M > 64) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread
-  // (r = 0: its own choice).  30..35: a configuration of the direct-to-LDS small-batch kernel.  0..12: a
+  // (r = 0: its own choice).  30..35: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with register-resident
+  // activations (M <= 16).  0..12: a
   // configuration of the tiled MFMA kernel (covers every shape).
+  if (variant == 40 || (variant < 0 && M >= 3 && M <= 16)) {
+    // a handful of rows: activations resident in registers (shapes it does not cover fall through)
+    const int rc = w4a16_regres(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+    if (variant == 40) DQ_FAIL("%s: the register-resident kernel does not cover M=%d N=%d K=%d group=%d", fn, M, N, K, group);
+  }
   if (variant >= 30 && variant < 40) {
     const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant - 30, (hipStream_t)stream);
     if (rc > 0) DQ_FAIL("%s: the streaming small-batch kernel does not cover N=%d K=%d group=%d", fn, N, K, group);
