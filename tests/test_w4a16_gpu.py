@@ -147,7 +147,7 @@ def test_kernel_variants(cuda, variant):
     _run_gemv(cuda, 1, 1000, 2048 + 128, 128, "original", variant=variant)
 
 
-@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35])
+@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35, 36])
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
 def test_streaming_small_batch_kernel(cuda, variant, mode):
     """The direct-to-LDS kernel: ragged M and N, a single K step, fewer steps than ring stages, many steps,

@@ -88,10 +88,11 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
   if (K % 128 != 0) DQ_FAIL("%s: K=%d must be a multiple of 128", fn, K);
   if (!aligned16(A) || !aligned16(C)) DQ_FAIL("%s: A and C must be 16-byte aligned", fn);
-  // prefill-sized M: the 256 x 256 MFMA GEMM (same tile-exact decoders)
-  if (variant < 0 && M > 64) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
+  // prefill-sized M: the tiled MFMA GEMM (same tile-exact decoders); up to 128 rows the streaming kernel
+  // below (two passes over the weights) is still the faster one.  50: the GEMM whatever M.
+  if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread
-  // (r = 0: its own choice).  30..35: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with register-resident
+  // (r = 0: its own choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with register-resident
   // activations (M <= 16).  0..12: a
   // configuration of the tiled MFMA kernel (covers every shape).
   if (variant == 40 || (variant < 0 && M >= 3 && M <= 16)) {
@@ -114,7 +115,7 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (variant < 0 && M > 4) {
     // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
     const bool wide = N >= 128 * 200;
-    const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : 2);
+    const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : 6);
     const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, config, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }

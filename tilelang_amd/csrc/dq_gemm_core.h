@@ -34,6 +34,9 @@
 #define DQ_SWZ_SHIFT 1
 #endif
 
+#ifndef DQ_DMA_NBW
+#define DQ_DMA_NBW 4  // wave tile columns / 32 of the direct-to-LDS kernel (2 = eight waves, two per SIMD)
+#endif
 #ifndef DQ_DMA_MBW
 #define DQ_DMA_MBW 4  // wave tile rows / 32 of the direct-to-LDS kernel (2 = 128 x 256 tiles, two workgroups per CU)
 #endif
@@ -416,15 +419,18 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
 // workgroups per CU (76 KiB of LDS and 256 registers each) that fill each other's barrier stalls;
 // measured 13 % slower on the 4096 x 8192 x 8192 MXFP4 problem (twice the decode work per MFMA,
 // and the 256-register budget spills), so it is kept as a build option only.
-template <class P, int kMBW>
-__global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
+template <class P, int kMBW, int kNBW>
+__global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(P::kBRowBytes == 32, "direct-to-LDS variant: 32 packed bytes per weight row per tile");
   static_assert(kMBW == 2 || kMBW == 4, "wave tile of 64 or 128 rows");
-  constexpr int kNBW = 4;
+  static_assert(kNBW == 2 || kNBW == 4, "wave tile of 64 or 128 columns");
+  constexpr int kWavesN = 8 / kNBW;            // waves across the 256 tile columns
+  constexpr int kWaves = 2 * kWavesN;          // 4, or 8 (two per SIMD)
   constexpr int BM = 64 * kMBW;                // shadows the 256-row default
   constexpr int kAStage = BM * kARowBytes;     // 32 or 16 KiB
-  constexpr int kAOps = 2 * kMBW;              // A DMA instructions per wave per tile
+  constexpr int kAOps = 8 * kMBW / kWaves;     // A DMA instructions per wave per tile
+  constexpr int kBOps = 8 / kWaves;            // packed-B DMA instructions per wave per tile
   constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
   constexpr int kStage = kAStage + kBStage;    // 40 or 24 KiB
   constexpr int kStages = 3;
@@ -434,7 +440,7 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / kWavesN, wn = wave % kWavesN;
   const int g = lane >> 5, r = lane & 31;
   const int M = p.M, N = p.N, K = p.K;
 
@@ -445,7 +451,7 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
   const unsigned lds0 = (unsigned)(size_t)smem;  // LDS byte address of the dynamic segment
 
   // ---- per-lane source offsets: LDS chunk c (16 bytes) of a tile <- which global 16 bytes --------
-  unsigned a_voff[kAOps], b_voff[2];
+  unsigned a_voff[kAOps], b_voff[kBOps];
 #pragma unroll
   for (int i = 0; i < kAOps; ++i) {
     const int c = (wave * kAOps + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
@@ -453,36 +459,36 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
     a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * (kARowBytes / P::kKPerBlock)) + (unsigned)((pp ^ a_swz(row)) << 4);
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int c = (wave * 2 + i) * 64 + lane;  // B chunk: row c / 2, physical piece c % 2
+  for (int i = 0; i < kBOps; ++i) {
+    const int c = (wave * kBOps + i) * 64 + lane;  // B chunk: row c / 2, physical piece c % 2
     const int row = c >> 1, pp = c & 1;
     b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K * P::kBRowBytes / P::kKPerBlock) + (unsigned)(((pp + (row >> 3)) & 1) << 4);
   }
-  const unsigned s_voff = (unsigned)min(n0 + tid, N - 1) * (unsigned)(K >> 5);
+  const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(K >> 5);  // waves 4..7 repeat 0..3
 
   // One tile = 3 + kAOps DMA instructions per thread: op 0 the scale dword (rows tid, tiles 2p and 2p+1;
   // issued with every tile, i.e. twice per pair, which keeps the loop branch-free), then the A chunks,
   // then the two packed-B chunks.
-  constexpr int kTileOps = 3 + kAOps;
+  constexpr int kTileOps = 1 + kAOps + kBOps;
   auto issue_op = [&](int op, int kb, int stage) {
     const unsigned sbase = lds0 + stage * kStage;
     if (op == 0) {
       if constexpr (P::kScaleBytes) {
         const int pair = kb >> 1;
-        dma4(lds0 + kRing + (pair & 3) * 1024 + wave * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
+        dma4(lds0 + kRing + (pair & 3) * 1024 + (wave & 3) * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
       }
     } else if (op <= kAOps) {
       const int i = op - 1;
       dma16(sbase + (wave * kAOps + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
     } else {
       const int i = op - 1 - kAOps;
-      dma16(sbase + kAStage + (wave * 2 + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * 32);
+      dma16(sbase + kAStage + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * 32);
     }
   };
   constexpr int kWaitOps = P::kScaleBytes ? kTileOps : kTileOps - 1;  // outstanding DMA instructions of one tile
 
   // ---- fragment read offsets (same LDS geometry as the register-staged kernel) --------------------
-  int a_row_off[kMBW], a_row_sw[kMBW], b_off[4], s_off[4];
+  int a_row_off[kMBW], a_row_sw[kMBW], b_off[kNBW], s_off[kNBW];
 #pragma unroll
   for (int mb = 0; mb < kMBW; ++mb) {
     const int row = wm * (32 * kMBW) + mb * 32 + r;
@@ -490,8 +496,8 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
     a_row_sw[mb] = a_swz(row);
   }
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    const int row = wn * 128 + nb * 32 + r;
+  for (int nb = 0; nb < kNBW; ++nb) {
+    const int row = wn * (32 * kNBW) + nb * 32 + r;
     b_off[nb] = kAStage + row * 32 + (((g + (row >> 3)) & 1) << 4);
     s_off[nb] = kRing + row * 4 + g;
   }
@@ -509,11 +515,11 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
     return P::prep_scale(e, p);
   };
 
-  typename P::acc_t acc[kMBW][4];
+  typename P::acc_t acc[kMBW][kNBW];
 #pragma unroll
   for (int mb = 0; mb < kMBW; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < kNBW; ++nb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
@@ -525,9 +531,9 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
   __syncthreads();
 
-  typename P::Scale sc_c[4];
-  uint32_t bw_c[4][kBWords];
-  frag_t af_c[kMBW], bf_c[4], af_n[kMBW], bf_n[4];
+  typename P::Scale sc_c[kNBW];
+  uint32_t bw_c[kNBW][kBWords];
+  frag_t af_c[kMBW], bf_c[kNBW], af_n[kMBW], bf_n[kNBW];
 
   // One iteration = tile kb out of `stage`, as 16 chunks of 4 MFMAs (one A fragment against the four
   // B fragments) kept in order by scheduling barriers; every chunk carries side work that issues in
@@ -550,7 +556,7 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
       if constexpr (kMBW == 4) {
         if (q == 0) {
 #pragma unroll
-          for (int nb = 0; nb < 4; ++nb) {
+          for (int nb = 0; nb < kNBW; ++nb) {
             read_b1(base, nb, bw_c[nb]);
             sc_c[nb] = read_scale1(kb, nb);
           }
@@ -560,16 +566,16 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
         } else if (q == 2) {
           af_n[2] = read_a1(base, 0, 2);
           af_n[3] = read_a1(base, 0, 3);
-          bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]);
-          bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]);
+#pragma unroll
+          for (int nb = 0; nb < kNBW / 2; ++nb) bf_n[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
         } else {
-          bf_n[2] = P::decode(bw_c[2], 0, sc_c[2]);
-          bf_n[3] = P::decode(bw_c[3], 0, sc_c[3]);
+#pragma unroll
+          for (int nb = kNBW / 2; nb < kNBW; ++nb) bf_n[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
         }
       } else {
         if (q == 0) {
 #pragma unroll
-          for (int nb = 0; nb < 4; ++nb) {
+          for (int nb = 0; nb < kNBW; ++nb) {
             read_b1(base, nb, bw_c[nb]);
             sc_c[nb] = read_scale1(kb, nb);
           }
@@ -577,20 +583,20 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
           af_n[1] = read_a1(base, 0, 1);
         } else {
 #pragma unroll
-          for (int nb = 0; nb < 4; ++nb) bf_n[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
+          for (int nb = 0; nb < kNBW; ++nb) bf_n[nb] = P::decode(bw_c[nb], 0, sc_c[nb]);
         }
       }
-      if (has_next2) issue_op(q, kb + 2, stage2);
+      if (has_next2 && q < kTileOps) issue_op(q, kb + 2, stage2);
       if (!first) {
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
+        for (int nb = 0; nb < kNBW; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int q = 0; q < kMBW; ++q) af_c[q] = af_n[q];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) bf_c[q] = bf_n[q];
+    for (int q = 0; q < kNBW; ++q) bf_c[q] = bf_n[q];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
 #pragma unroll
@@ -598,19 +604,17 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
         const int chunk = kMBW + j * kMBW + q;
         af_n[q] = read_a1(base, j + 1, q);
 #pragma unroll
-        for (int e = 0; e < 4 / kMBW; ++e) {
-          const int nb = q * (4 / kMBW) + e;
-          bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
-        }
+        for (int nb = 0; nb < kNBW; ++nb)  // the kNBW decodes of a step spread evenly over its kMBW chunks
+          if (nb * kMBW / kNBW == q) bf_n[nb] = P::decode(bw_c[nb], j + 1, sc_c[nb]);
         if (has_next2 && chunk < kTileOps) issue_op(chunk, kb + 2, stage2);
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
+        for (int nb = 0; nb < kNBW; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int q = 0; q < kMBW; ++q) af_c[q] = af_n[q];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) bf_c[q] = bf_n[q];
+      for (int q = 0; q < kNBW; ++q) bf_c[q] = bf_n[q];
     }
     // tile kb+1 must have landed before the next iteration reads it; tile kb+2 (issued during this
     // iteration) may still be in flight
@@ -639,7 +643,7 @@ __global__ __launch_bounds__(kThreads, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(c
 #pragma unroll
   for (int q = 0; q < kMBW; ++q)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
+    for (int nb = 0; nb < kNBW; ++nb) acc[q][nb] = P::mfma(af_c[q], bf_c[nb], acc[q][nb]);
 
   DQ_GEMM_EPILOGUE
 }
@@ -681,25 +685,28 @@ bool dma_eligible(const Params& p) {
   return (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
 }
 
-template <class P, int kMBW>
+template <class P, int kMBW, int kNBW>
 int launch_dma_tile(Params p, hipStream_t stream) {
-  constexpr int kLds = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + 4 * 1024;
+  constexpr int kWaves = 16 / kNBW;
+  constexpr int kPipe = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + 4 * 1024;
+  constexpr int kSlabs = kWaves * 32 * (32 * kNBW + 4) * 4;  // epilogue staging
+  constexpr int kLds = kPipe > kSlabs ? kPipe : kSlabs;
   p.tiles_m = (p.M + 64 * kMBW - 1) / (64 * kMBW);
   p.tiles_n = (p.N + BN - 1) / BN;
-  auto kern = gemm_kernel_dma<P, kMBW>;
+  auto kern = gemm_kernel_dma<P, kMBW, kNBW>;
   static bool lds_limit_raised = false;
   if (!lds_limit_raised) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
     lds_limit_raised = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(kThreads), kLds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(64 * kWaves), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }
 
 template <class P>
 int launch_dma(const Params& p, hipStream_t stream) {
-  return launch_dma_tile<P, DQ_DMA_MBW>(p, stream);
+  return launch_dma_tile<P, DQ_DMA_MBW, DQ_DMA_NBW>(p, stream);
 }
 
 inline Params make_params(const void* A, const void* B, const void* S, const void* Z, const void* Bias, void* C, int M,

@@ -1,4 +1,4 @@
-// W4A16 small-batch kernel for gfx950 (4 <= M <= 64 activation rows), direct-to-LDS streaming.
+// W4A16 small-batch kernel for gfx950 (blocks of up to 64 activation rows), direct-to-LDS streaming.
 //
 // Replaces the batched use of the kernel generated from
 // examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:83-153 (group scales / zeros as in
@@ -21,9 +21,14 @@
 //     labelled k = chunk + g * 32 + j * 8 + {0,4,1,5,2,6,3,7}[e]; the matching activation
 //     operand is one ds_read_b128 plus, for the plain layout, four v_perm_b32;
 //   * all vector-memory loads of the loop are these DMA instructions, issued from inline assembly
-//     and tracked by hand with s_waitcnt vmcnt; one workgroup barrier per step.
+//     and tracked by hand with s_waitcnt vmcnt; one workgroup barrier per step;
+//   * the LDS reads, the decode and the MFMAs of consecutive 32-k sub-steps are software-pipelined
+//     (two sub-steps deep, across the step boundary), so that a wave's MFMAs issue among the VALU work
+//     of its next sub-step.
 //
 // K is not split: every wave owns its output tile, results are bit-identical from run to run.
+#include <type_traits>
+
 #include "dq_common.h"
 
 namespace dq {
@@ -49,25 +54,37 @@ struct StreamGeom {
   static constexpr int kStage = kSOff + 1024;
 };
 
-template <int MB, int RBW, int NST, int MODE, bool APERM>
-__global__ __launch_bounds__(256) void w4a16_stream_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ B,
-                                                            const half_t* __restrict__ S, const half_t* __restrict__ Z,
-                                                            half_t* __restrict__ C, int M, int N, int K) {
+// KSPLIT = 2: eight waves, two per SIMD; waves 4..7 own the same rows as waves 0..3 and take the second
+// 128-k half of every step (the two partial sums meet once, through LDS, after the K loop).  The
+// LDS traffic and the decode work per workgroup are those of KSPLIT = 1; what the second wave per
+// SIMD buys is that one wave's MFMAs run under the other's decode and waits.
+template <int MB, int RBW, int NST, int KSPLIT, int MODE, bool APERM>
+__global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t* __restrict__ A,
+                                                                     const uint8_t* __restrict__ B,
+                                                                     const half_t* __restrict__ S,
+                                                                     const half_t* __restrict__ Z, half_t* __restrict__ C,
+                                                                     int M, int N, int K) {
   extern __shared__ __align__(16) unsigned char smem[];
   using G = StreamGeom<MB, RBW>;
+  static_assert(KSPLIT == 1 || KSPLIT == 2, "one or two waves per SIMD");
+  static_assert((2 * RBW) % KSPLIT == 0 && (2 * MB) % KSPLIT == 0, "whole DMA instructions per wave");
   constexpr int kRowsPerWg = G::kRowsPerWg;
   constexpr int kWBytes = G::kWBytes;
-  constexpr int kWOps = 2 * RBW;                        // weight DMA instructions per wave per stage
+  constexpr int kWOps = 2 * RBW / KSPLIT;               // weight DMA instructions per wave per stage
   constexpr bool kScale = MODE >= W4_SCALE;
   constexpr bool kZeros = MODE >= W4_ZEROS_ORIGINAL;
-  constexpr int kAOps = 2 * MB;                         // activation DMA instructions per wave per stage
+  constexpr int kAOps = 2 * MB / KSPLIT;                // activation DMA instructions per wave per stage
   constexpr int kOps = kWOps + kAOps + (kScale ? 1 : 0);    // DMA instructions per wave per stage
   constexpr int kWaitOps = (NST - 2) * kOps;            // younger instructions when the next stage must have landed
-  static_assert(kWaitOps <= 63, "vmcnt is a 6-bit counter");
+  static_assert((NST - 1) * kOps <= 63, "vmcnt is a 6-bit counter");
+  constexpr int kU = 2 / KSPLIT;                        // 128-k halves of a step per wave
+  constexpr int kSub = 4 * kU;                          // sub-steps (32 k) of a step per wave
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 3;                              // which rows
+  const int kh = wave >> 2;                             // which half of a step (KSPLIT = 2)
   const int g = lane >> 4;
   const int r = lane & 15;
   const int n0 = blockIdx.x * kRowsPerWg;
@@ -92,10 +109,10 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(const half_t* __restr
     a_voff[i] = (unsigned)(m0 + min(row, mrows - 1)) * (unsigned)(K * 2) + (unsigned)((pos ^ (row & 15)) << 4);
   }
   // waves 0, 1: scales of rows 0..63 / 64..127 from the workgroup's first row; waves 2, 3: zeros (or,
-  // without zeros, the scales again).  Every wave issues the same number of DMA instructions; with 64
-  // rows per workgroup the second half is simply not read.
-  const unsigned s_voff = (unsigned)min(n0 + (wave & 1) * 64 + lane, N - 1) * (unsigned)(groups_per_row * 2);
-  const unsigned char* s_src = reinterpret_cast<const unsigned char*>((wave >= 2 && kZeros) ? Z : S);
+  // without zeros, the scales again); waves 4..7 repeat 0..3.  Every wave issues the same number of
+  // DMA instructions; with 64 rows per workgroup the second half is simply not read.
+  const unsigned s_voff = (unsigned)min(n0 + (wn & 1) * 64 + lane, N - 1) * (unsigned)(groups_per_row * 2);
+  const unsigned char* s_src = reinterpret_cast<const unsigned char*>((wn >= 2 && kZeros) ? Z : S);
 
   auto issue_stage = [&](int step, int slot) {
     const unsigned sb = lds0 + slot * G::kStage;
@@ -105,22 +122,23 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(const half_t* __restr
     for (int i = 0; i < kAOps; ++i)
       dma16(sb + kWBytes + (wave * kAOps + i) * 1024, a_voff[i],
             reinterpret_cast<const unsigned char*>(A) + (size_t)step * (kStepK * 2));
-    if constexpr (kScale) dma4(sb + G::kSOff + wave * 256, s_voff, s_src + (size_t)step * 4);
+    if constexpr (kScale) dma4(sb + G::kSOff + wn * 256, s_voff, s_src + (size_t)step * 4);
   };
 
-  // ---- fragment read offsets inside a stage -----------------------------------------------------
-  int w_off[RBW][2], sc_off[RBW], y_off[2][4];
+  // ---- fragment read offsets inside a stage (ui: the wave's ui-th half of a step) -----------------
+  int w_off[RBW][kU], sc_off[RBW][kU], y_off[kU][4];
 #pragma unroll
-  for (int rb = 0; rb < RBW; ++rb) {
-    const int row = wave * (16 * RBW) + rb * 16 + r;
-    sc_off[rb] = G::kSOff + row * 4;
+  for (int ui = 0; ui < kU; ++ui) {
+    const int u = KSPLIT == 2 ? kh : ui;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) w_off[rb][u] = row * 128 + ((((u << 2) + g) ^ ((row >> 1) & 7)) << 4);
+    for (int rb = 0; rb < RBW; ++rb) {
+      const int row = wn * (16 * RBW) + rb * 16 + r;
+      sc_off[rb][ui] = G::kSOff + row * 4 + u * 2;
+      w_off[rb][ui] = row * 128 + ((((u << 2) + g) ^ ((row >> 1) & 7)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y_off[ui][j] = kWBytes + r * 512 + (u << 8) + ((((g << 2) + j) ^ r) << 4);
   }
-#pragma unroll
-  for (int u = 0; u < 2; ++u)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) y_off[u][j] = kWBytes + r * 512 + (u << 8) + ((((g << 2) + j) ^ r) << 4);
 
   float4_t acc[RBW][MB];
 #pragma unroll
@@ -128,75 +146,160 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(const half_t* __restr
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  // All LDS operands of a step are fetched up front (registers are plentiful, waves per SIMD are
-  // not): the reads of chunk 1 and of the later activation pieces return while chunk 0 is decoded.
-  auto compute = [&](const unsigned char* sb) {
-    uint4_t w[2][RBW], yraw[2][4][MB];
-    half_t sc[2][RBW], zp[2][RBW];
+  // ---- software pipeline over the sub-steps (32 k each) of every step -----------------------------
+  // Sub-step t goes through R(t): its LDS reads are requested, D(t): the weight dwords are decoded and,
+  // for the plain layout, one operand is permuted to the other's element order (whichever of the two
+  // takes fewer v_perm_b32), M(t): the RBW x MB MFMAs.  Slot t of the instruction stream holds
+  // R(t+2), D(t+1) and M(t) between two scheduling barriers, so the MFMAs of one sub-step issue among
+  // the independent VALU work of the next and no operand is waited for right after it was requested.
+  // The pipeline runs across steps: the last two slots of a step read from the NEXT stage, so the
+  // workgroup barrier that publishes that stage (and releases the current one for the DMA engine)
+  // sits in front of them.
+  constexpr bool kPermW = APERM && RBW < MB;   // bring the decoded weights to natural k order
+  constexpr bool kPermA = APERM && !kPermW;    // or the activations to the decoder's order
+  uint4_t w_c[kU][RBW], w_n[kU][RBW], yraw[2][MB];
+  half_t sc_c[kU][RBW], zp_c[kU][RBW], sc_n[kU][RBW], zp_n[kU][RBW];
+  half8_t x_m[RBW], y_m[MB], x_d[RBW], y_d[MB];
+  auto read_weights = [&](const unsigned char* sb) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int ui = 0; ui < kU; ++ui)
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb) {
-        w[u][rb] = *reinterpret_cast<const uint4_t*>(sb + w_off[rb][u]);
-        sc[u][rb] = kScale ? *reinterpret_cast<const half_t*>(sb + sc_off[rb] + u * 2) : (half_t)1.f;
-        zp[u][rb] = kZeros ? *reinterpret_cast<const half_t*>(sb + sc_off[rb] + 512 + u * 2) : (half_t)0.f;
+        w_n[ui][rb] = *reinterpret_cast<const uint4_t*>(sb + w_off[rb][ui]);
+        sc_n[ui][rb] = kScale ? *reinterpret_cast<const half_t*>(sb + sc_off[rb][ui]) : (half_t)1.f;
+        zp_n[ui][rb] = kZeros ? *reinterpret_cast<const half_t*>(sb + sc_off[rb][ui] + 512) : (half_t)0.f;
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          yraw[u][j][mb] = *reinterpret_cast<const uint4_t*>(sb + y_off[u][j] + mb * (16 * 512));
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        half8_t y[MB];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          y[mb] = __builtin_bit_cast(half8_t, APERM ? permute_k8_16bit(yraw[u][j][mb]) : yraw[u][j][mb]);
-#pragma unroll
-        for (int rb = 0; rb < RBW; ++rb) {
-          const half8_t x = decode_w4<MODE>(w[u][rb][j], sc[u][rb], zp[u][rb]);
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y[mb], acc[rb][mb], 0, 0, 0);
-        }
-      }
+  };
+  auto decode = [&](uint32_t w, half_t sc, half_t zp) -> half8_t {
+    const half8_t x = decode_w4<MODE>(w, sc, zp);
+    if constexpr (kPermW) {
+      const uint4_t d = __builtin_bit_cast(uint4_t, x);  // (n0,n4) (n1,n5) (n2,n6) (n3,n7)
+      uint4_t o;
+      o[0] = __builtin_amdgcn_perm(d[1], d[0], 0x05040100u);
+      o[1] = __builtin_amdgcn_perm(d[3], d[2], 0x05040100u);
+      o[2] = __builtin_amdgcn_perm(d[1], d[0], 0x07060302u);
+      o[3] = __builtin_amdgcn_perm(d[3], d[2], 0x07060302u);
+      return __builtin_bit_cast(half8_t, o);
+    } else {
+      return x;
     }
   };
-
-  // ---- prologue: stages 0 .. NST-2 in flight, stage 0 landed --------------------------------------
+  // slots s_begin .. s_end-1 of a step whose stage is sb_cur; kCur: the step exists (false only
+  // while the pipeline fills before step 0), kNext: so does the next one, staged at sb_nxt
+  auto run_slots = [&](auto s_begin, auto s_end, const unsigned char* sb_cur, const unsigned char* sb_nxt, auto cur_tag,
+                       auto next_tag) {
+    constexpr bool kCur = decltype(cur_tag)::value, kNext = decltype(next_tag)::value;
 #pragma unroll
-  for (int s = 0; s < NST - 1; ++s)
-    if (s < KS) issue_stage(s, s);
-  if (KS >= NST - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
+    for (int s = decltype(s_begin)::value; s < decltype(s_end)::value; ++s) {
+      const int s2 = s + 2, s1 = s + 1;
+      if (s2 < kSub) {  // R(t+2)
+        if constexpr (kCur) {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            yraw[s & 1][mb] = *reinterpret_cast<const uint4_t*>(sb_cur + y_off[s2 >> 2][s2 & 3] + mb * (16 * 512));
+        }
+      } else if constexpr (kNext) {
+        if (s2 == kSub) read_weights(sb_nxt);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          yraw[s & 1][mb] = *reinterpret_cast<const uint4_t*>(sb_nxt + y_off[0][s2 - kSub] + mb * (16 * 512));
+      }
+      if (s1 < kSub ? kCur : kNext) {  // D(t+1)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          y_d[mb] = __builtin_bit_cast(half8_t, kPermA ? permute_k8_16bit(yraw[s1 & 1][mb]) : yraw[s1 & 1][mb]);
+#pragma unroll
+        for (int rb = 0; rb < RBW; ++rb) {
+          if (s1 < kSub) x_d[rb] = decode(w_c[(s1 >> 2) % kU][rb][s1 & 3], sc_c[(s1 >> 2) % kU][rb], zp_c[(s1 >> 2) % kU][rb]);
+          else x_d[rb] = decode(w_n[0][rb][0], sc_n[0][rb], zp_n[0][rb]);
+        }
+      }
+      if constexpr (kCur) {  // M(t)
+#pragma unroll
+        for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x_m[rb], y_m[mb], acc[rb][mb], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) x_m[rb] = x_d[rb];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) y_m[mb] = y_d[mb];
+    }
+  };
+  auto next_weights_become_current = [&]() {
+#pragma unroll
+    for (int ui = 0; ui < kU; ++ui)
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) {
+        w_c[ui][rb] = w_n[ui][rb];
+        sc_c[ui][rb] = sc_n[ui][rb];
+        zp_c[ui][rb] = zp_n[ui][rb];
+      }
+  };
+  using SlotFirst = std::integral_constant<int, 0>;
+  using SlotNext = std::integral_constant<int, kSub - 2>;  // first slot that reads the next stage
+  using SlotEnd = std::integral_constant<int, kSub>;
+
+  // ---- prologue: stages 0 .. NST-1 in flight, stage 0 landed, pipeline filled -----------------------
+#pragma unroll
+  for (int st = 0; st < NST; ++st)
+    if (st < KS) issue_stage(st, st);
+  if (KS >= NST) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kOps) : "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  run_slots(SlotNext{}, SlotEnd{}, smem, smem, std::false_type{}, std::true_type{});
+  next_weights_become_current();
 
-  // Step `step` multiplies out of slot step % NST.  The slot of step - 1 was released by the barrier
-  // that ended that step, so the DMA of step + NST - 1 goes there first thing.  At the end of the
-  // step the stages younger than step + 1 are the NST - 2 issued last (kWaitOps instructions); in the
-  // tail, where nothing is issued any more, the wave simply drains its counter.
+  // Step `step` multiplies out of slot step % NST.  Before its last two slots the next stage must
+  // have landed: the stages younger than it are the NST - 2 issued last (kWaitOps instructions), or, in
+  // the tail where fewer are in flight, the wave simply drains its counter.  After the barrier no wave
+  // reads stage `step` any more (the barrier also waits for the LDS reads in flight), so the DMA of
+  // step + NST goes there.
   int slot = 0;
-  for (int step = 0; step < KS; ++step) {
-    const int nxt = step + NST - 1;
-    if (nxt < KS) issue_stage(nxt, slot == 0 ? NST - 1 : slot - 1);
-    compute(smem + slot * G::kStage);
-    if (nxt < KS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
+  for (int step = 0; step + 1 < KS; ++step) {
+    const int slot1 = slot + 1 == NST ? 0 : slot + 1;
+    const unsigned char* sb_cur = smem + slot * G::kStage;
+    run_slots(SlotFirst{}, SlotNext{}, sb_cur, sb_cur, std::true_type{}, std::true_type{});
+    if (step + NST - 1 < KS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    slot = slot + 1 == NST ? 0 : slot + 1;
+    if (step + NST < KS) issue_stage(step + NST, slot);
+    run_slots(SlotNext{}, SlotEnd{}, sb_cur, smem + slot1 * G::kStage, std::true_type{}, std::true_type{});
+    next_weights_become_current();
+    slot = slot1;
+  }
+  run_slots(SlotFirst{}, SlotEnd{}, smem + slot * G::kStage, smem, std::true_type{}, std::false_type{});
+
+  if constexpr (KSPLIT == 2) {
+    // waves 4..7 hand their half of the K sum to waves 0..3: [wn][rb][mb][lane] float4
+    __syncthreads();  // every wave is done with the stages
+    float4_t* red = reinterpret_cast<float4_t*>(smem) + wn * (RBW * MB * 64) + lane;
+    if (kh == 1) {
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red[(rb * MB + mb) * 64] = acc[rb][mb];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+#pragma unroll
+    for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const float4_t o = red[(rb * MB + mb) * 64];
+        acc[rb][mb] = float4_t{acc[rb][mb][0] + o[0], acc[rb][mb][1] + o[1], acc[rb][mb][2] + o[2], acc[rb][mb][3] + o[3]};
+      }
   }
 
-  // acc[rb][mb][i] = C[m0 + mb*16 + r][n0 + wave*16*RBW + rb*16 + g*4 + i]
+  // acc[rb][mb][i] = C[m0 + mb*16 + r][n0 + wn*16*RBW + rb*16 + g*4 + i]
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int m = mb * 16 + r;
-      const int n = n0 + wave * (16 * RBW) + rb * 16 + g * 4;
+      const int n = n0 + wn * (16 * RBW) + rb * 16 + g * 4;
       if (m >= mrows || n >= N) continue;
       const float4_t v = acc[rb][mb];
       half_t* dst = C + (size_t)(m0 + m) * N + n;
@@ -212,17 +315,17 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(const half_t* __restr
     }
 }
 
-template <int MB, int RBW, int NST>
+template <int MB, int RBW, int NST, int KSPLIT>
 int launch_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int mode,
                   int layout, hipStream_t stream) {
   constexpr int kLds = NST * StreamGeom<MB, RBW>::kStage;
   constexpr int kRowsPerWg = StreamGeom<MB, RBW>::kRowsPerWg;
   static_assert(kLds <= 160 * 1024, "LDS budget");
   const dim3 grid((N + kRowsPerWg - 1) / kRowsPerWg, (M + 16 * MB - 1) / (16 * MB));
-  const dim3 block(256);
+  const dim3 block(256 * KSPLIT);
 #define DQ_LAUNCH2(MODE_, APERM_)                                                                                    \
   do {                                                                                                               \
-    auto kern = w4a16_stream_kernel<MB, RBW, NST, MODE_, APERM_>;                                                         \
+    auto kern = w4a16_stream_kernel<MB, RBW, NST, KSPLIT, MODE_, APERM_>;                                                         \
     static bool lds_limit_raised = false; /* once per kernel: legal under stream capture afterwards */            \
     if (!lds_limit_raised) {                                                                                         \
       DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                          \
@@ -256,7 +359,9 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 }  // namespace
 
 // config 0, 1, 2: 16, 32, 64 activation rows and 128 weight rows per workgroup; 3, 4, 5: 16, 32, 16
-// activation rows and 64 weight rows.  Returns 1 when the shape is not
+// activation rows and 64 weight rows; 6: as 2 with eight waves (measured at N = 28672, K = 8192, M = 64:
+// 60 us against 63 us; the eight-wave forms of 0 and 1 were slower than the four-wave ones and are
+// not built).  Returns 1 when the shape is not
 // covered (the caller falls back to a kernel without these restrictions): the group size must be
 // 128 when the mode reads scales, K a multiple of 256, and every operand below 4 GiB (32-bit
 // lane offsets).
@@ -266,12 +371,13 @@ int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, voi
   if (mode >= W4_SCALE && group != 128) return 1;
   if ((size_t)N * K / 2 >= (1ull << 32) || (size_t)M * K * 2 >= (1ull << 32)) return 1;
   switch (config) {
-    case 0: return launch_stream<1, 2, 6>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 1: return launch_stream<2, 2, 4>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 2: return launch_stream<4, 2, 3>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 3: return launch_stream<1, 1, 4>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 4: return launch_stream<2, 1, 3>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 5: return launch_stream<1, 1, 6>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 0: return launch_stream<1, 2, 6, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 1: return launch_stream<2, 2, 4, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 2: return launch_stream<4, 2, 3, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 3: return launch_stream<1, 1, 4, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 4: return launch_stream<2, 1, 3, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 5: return launch_stream<1, 1, 6, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 6: return launch_stream<4, 2, 3, 2>(A, B, S, Z, C, M, N, K, mode, layout, stream);
     default: DQ_FAIL("w4a16 stream kernel: unknown configuration %d", config);
   }
 }
