@@ -418,7 +418,10 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
 // kMBW = 4: 256 x 256 tile, one workgroup per CU (the default).  kMBW = 2: 128 x 256 tile, two
 // workgroups per CU (76 KiB of LDS and 256 registers each) that fill each other's barrier stalls;
 // measured 13 % slower on the 4096 x 8192 x 8192 MXFP4 problem (twice the decode work per MFMA,
-// and the 256-register budget spills), so it is kept as a build option only.
+// and the 256-register budget spills), so it is kept as a build option only.  kNBW = 2: the same
+// 256 x 256 tile on eight waves (two per SIMD, wave tile 128 x 64): no spills and the same decode work,
+// but every A fragment is read from LDS by twice as many waves; measured 4 % slower on that
+// problem (410 us against 393 us), also a build option only (-DDQ_DMA_NBW=2).
 template <class P, int kMBW, int kNBW>
 __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
