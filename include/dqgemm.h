@@ -100,7 +100,7 @@ int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int
 /* fp16 x uint4 with the integer decoders: C[M,N] fp16 = A[M,K] fp16 . dequant(B, Scale, Zeros)^T with
  * the dequantised tile rounded to fp16 exactly as call_dequantize_w4 does.  Replaces `call(A, B, C)` of
  * examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:45-88 (mode DQ_W4_UNSIGNED) and serves
- * W4A16 at M > 64.  Requires K % 64 == 0; group rules as for call_dequantize_gemv_w4a16. */
+ * W4A16 at M > 128.  Requires K % 64 == 0; group rules as for call_dequantize_gemv_w4a16. */
 int call_dequant_gemm_w4_fp16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M,
                               int N, int K, int group, int mode, int layout, dq_stream_t stream);
 
