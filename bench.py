@@ -154,6 +154,24 @@ def bench_activation_quant(torch, tl, M, K, steps, warmup, dev):
     return {"us": ms * 1e3, "bytes": 3 * M * K + 4 * M, "flops": 2 * M * K, "graph": graphed}
 
 
+def bench_mxfp4_quant(torch, tl, N, K, steps, warmup, dev):
+    """MXFP4 weight quantiser (bf16 -> e2m1 codes + one scale byte per 32), the producer of the GEMM's B and Scale."""
+    nbytes = 2 * N * K + N * K // 2 + N * K // 32
+    nc = _copies(nbytes, hi=6)
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    ws = [(torch.randn((N, K), generator=gen, dtype=torch.float32) * 0.05).to(torch.bfloat16).to(dev) for _ in range(nc)]
+    kern = tl.quantize_bf16_mxfp4(N, K)
+    out = [None]
+
+    def mk(i):
+        def f():
+            out[0] = kern(ws[i], skip_tensor_validation=True)
+        return f
+
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * N * K, "graph": graphed}
+
+
 def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev):
     """W4A8 (int8 x int4, Ct[N,M] int32) or int4 x int4 (C[M,N] int32), exact."""
     if a_packed:
@@ -272,6 +290,8 @@ def main():
         for m in (1, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, k if m == 1 else kg, 2, dev)
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        r = bench_mxfp4_quant(torch, tl, 8192, 8192, k, 2, dev)
+        shapes.append(_row("mxfp4_quantize N=8192 K=8192", r, "hbm", MFMA_BF16_PEAK))
         r = bench_activation_quant(torch, tl, 2048, 8192, k, 2, dev)
         shapes.append(_row("bitnet_activation_quant M=2048 K=8192", r, "hbm", MFMA_I8_PEAK))
         r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, False, kg, 2, dev)

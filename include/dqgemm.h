@@ -127,6 +127,15 @@ int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int
  * replaces.  Requires K % 8 == 0. */
 int call_bitnet_activation_quant(const void* X, void* Q, void* S, int M, int K, dq_stream_t stream);
 
+/* MXFP4 weight quantiser (the producer of call_dequant_gemm_bf16_mxfp4's B and Scale, which the reference's
+ * example draws at random, examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:99-103,286-290):
+ * W[N,K] bf16 -> B[N,K/2] e2m1 codes, two per byte, even k in the low nibble, and Scale[N,K/32] one byte per 32 k.
+ * Per block: e = max(floor(log2(max|w|)) - 2, -127), Scale = clamp(e + scale_bias, 0, 255), codes =
+ * encode_fp4_e2m1_values(w / 2^(Scale - scale_bias)) of examples/dequantize_gemm/quantize/nvfp4.py:120-138
+ * (thresholds 0.25 .. 5.0, a value on a threshold goes up, saturation at 6, no negative zero).
+ * scale_bias as in call_dequant_gemm_bf16_mxfp4 (127: E8M0).  Requires K % 32 == 0. */
+int call_quantize_bf16_mxfp4(const void* W, void* B, void* Scale, int N, int K, int scale_bias, dq_stream_t stream);
+
 /* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T.
  * is_signed 1: two's-complement nibbles (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:10-21,
  * `call(A, B, Ct)` :109-147); 0: unsigned nibbles (example_dequant_gemm_fine_grained.py int8 path).

@@ -26,7 +26,13 @@ Parity unpinned by any reference test or fixture (no in-tree caller exists; the
 contract is the closed form plus the operation order of the device snippets):
 ``dequant_u4_scale`` / ``dequant_u4_scale_zeros`` rounding order
 (examples/dequantize_gemm/quantize/lop3.py:41-81,136-176,233-271,326-363) and the
-BitNet 2-bit code convention (``decode_i2``, zero_point choice).
+BitNet 2-bit code convention (``decode_i2``, zero_point choice).  ``quantize_mxfp4``: the
+reference has no MXFP4 quantiser (its example draws codes and scales at random), so the block
+scale rule is the OCP Microscaling v1.0 conversion and only the element rule
+(``encode_fp4_e2m1_values``) is the reference's own: parity unpinned for the scale choice, which
+is pinned by closed forms instead (exact powers of two, round trip through ``mxfp4_dequant``,
+idempotence, the block maximum always landing in e2m1's top binade).  ``gen_quant4_quantize`` is
+pinned by its closed form (absmax scale, rint, clamp) against torch's own ops on the CPU.
 """
 
 from __future__ import annotations
@@ -520,6 +526,55 @@ def ref_bitnet_int(A_i8, packed, convention: str = "offset"):
     and ..._prefill.py:360-381 (torch matmul of the unpacked operands).
     """
     return _matmul_int(np.asarray(A_i8, dtype=np.int8), decode_i2(packed, convention)).astype(np.int32)
+
+
+# --------------------------------------------------------------------------------------
+# weight quantisers (the producers of the packed operands)
+# --------------------------------------------------------------------------------------
+
+
+def quantize_mxfp4(w: np.ndarray, scale_bias: int = 127, scale_size: int = 32):
+    """bf16-representable ``w[N, K]`` -> (packed e2m1 codes uint8 [N, K/2], scale bytes uint8 [N, K/scale_size]).
+
+    Block scale: ``e = max(floor(log2(max|w|)) - 2, -127)`` (OCP Microscaling Formats v1.0, section 6.3: shared
+    exponent = exponent of the block maximum minus the exponent of the element format's largest value, 6 = 1.5 * 2^2;
+    an all-zero block takes the smallest exponent, as the published ``microxcaling`` library does),
+    ``byte = clamp(e + scale_bias, 0, 255)``.  Elements: ``encode_fp4_e2m1_values(w / 2**(byte - scale_bias))``
+    (examples/dequantize_gemm/quantize/nvfp4.py:120-138), packed low nibble first (``:141-157``).  The layout is
+    the one examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:99-103 consumes.
+    """
+    w = np.asarray(w, dtype=np.float32)
+    N, K = w.shape
+    blocks = w.reshape(N, K // scale_size, scale_size)
+    amax = np.abs(blocks).max(axis=-1)
+    # floor(log2(amax)) from the exponent field (exact); bf16 subnormals and zero give exponent field 0
+    expf = (amax.view(np.uint32) >> 23).astype(np.int32) & 0xFF
+    e = np.maximum(expf - 127 - 2, -127)
+    byte = np.clip(e + scale_bias, 0, 255)
+    e_used = np.clip(byte - scale_bias, -127, 126)
+    scaled = blocks * np.exp2(-e_used.astype(np.float64))[..., None].astype(np.float32)  # exact: power of two
+    codes = encode_fp4_e2m1_values(scaled.reshape(N, K))
+    return pack_fp4_e2m1_codes(codes), byte.astype(np.uint8)
+
+
+def gen_quant4_quantize(w: np.ndarray, groupsize: int = -1):
+    """The deterministic part of ``gen_quant4`` (examples/dequantize_gemm/quantize/utils.py:1-47) for a given
+    fp16 ``w[K, N]``: per (group of ``groupsize`` consecutive k, column n) ``s = max|w| * 2 / 16`` in fp16,
+    ``q = clamp(rint(w / s) + 8, 0, 16)``, ``ref = (q - 8).half() * s``.  Returns ``(ref[K, N] fp16,
+    s[K/groupsize, N] fp16, q - 8 [K, N] int32)`` — the reference's ``linear.weight.T``, ``s`` and last value.
+
+    ``maxq`` is 16 there, not 15: the element with the largest magnitude of a group, when positive, quantises to
+    ``q = 16``, which does not fit a nibble (the reference never packs this function's output).
+    """
+    w = np.asarray(w, dtype=np.float16)
+    K, N = w.shape
+    g = K if groupsize == -1 else groupsize
+    wg = w.reshape(K // g, g, N)
+    s = (np.abs(wg).max(axis=1, keepdims=True).astype(np.float16) * np.float16(2 / 16)).astype(np.float16)
+    q = np.rint((wg / s).astype(np.float16).astype(np.float32)).astype(np.int32) + 8
+    q = np.clip(q, 0, 16)
+    ref = ((q - 8).astype(np.float16) * s).astype(np.float16)
+    return ref.reshape(K, N), s.reshape(K // g, N), (q - 8).reshape(K, N)
 
 
 # --------------------------------------------------------------------------------------

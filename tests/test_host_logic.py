@@ -64,6 +64,12 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     assert "S is expected to have non-NULL" in lib.get_last_error().decode()
     assert lib.call_bitnet_activation_quant(a, a, a, 4, 100, vp(0)) == -1
     assert "multiple of 8" in lib.get_last_error().decode()
+    assert lib.call_quantize_bf16_mxfp4(a, vp(0), a, 4, 64, 127, vp(0)) == -1
+    assert "B is expected to have non-NULL" in lib.get_last_error().decode()
+    assert lib.call_quantize_bf16_mxfp4(a, a, a, 4, 48, 127, vp(0)) == -1
+    assert "multiple of 32" in lib.get_last_error().decode()
+    assert lib.call_quantize_bf16_mxfp4(a, a, a, 4, 64, 300, vp(0)) == -1
+    assert "scale_bias" in lib.get_last_error().decode()
 
 
 def test_bitlinear_weight_packing_matches_oracle():

@@ -317,3 +317,102 @@ def test_torch_restatement_matches_numpy_oracle():
     got = ref_torch.ref_bitnet(torch.from_numpy(bn["A"]), torch.from_numpy(bn["B"]), torch.from_numpy(bn["s_a"]), float(bn["s_w"]))
     want = orc.ref_bitnet(bn["A"], bn["B"], bn["s_a"], bn["s_w"], "offset")
     np.testing.assert_allclose(got.numpy().astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
+def _bf16_pred(x):
+    """Largest bf16 value below the positive bf16 value x."""
+    bits = orc.f32_to_bf16_bits(np.asarray(x, dtype=np.float32))
+    return orc.bf16_bits_to_f32((bits - 1).astype(np.uint16))
+
+
+def test_quantize_mxfp4_closed_forms():
+    """Block scale and element codes where the mathematics fixes them: a block whose maximum is 6 * 2^e or
+    4 * 2^e keeps exponent e (codes 7 / 6); every e2m1 threshold goes up, its bf16 predecessor goes down; an
+    all-zero block takes the smallest exponent; the sign bit is never set on a zero magnitude."""
+    for e in (-20, -8, -1, 0, 3, 17):
+        blk = np.zeros((1, 32), dtype=np.float32)
+        blk[0, 5] = 6.0 * 2.0**e
+        blk[0, 6] = -4.0 * 2.0**e
+        blk[0, 7] = 7.5 * 2.0**e   # same binade as 6: saturates
+        blk[0, 8] = -1e-30         # rounds to zero: no negative zero
+        B, S = orc.quantize_mxfp4(blk, scale_bias=127)
+        codes = orc.unpack_u4(B)[0]
+        assert S[0, 0] == 127 + e
+        assert list(codes[5:9]) == [7, 8 | 6, 7, 0]
+    thresholds = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], dtype=np.float32)
+    blk = np.zeros((1, 32), dtype=np.float32)
+    blk[0, 0] = 6.0                                  # pins the block exponent at 0
+    blk[0, 1:8] = thresholds
+    blk[0, 8:15] = _bf16_pred(thresholds)
+    blk[0, 15:22] = -thresholds
+    B, S = orc.quantize_mxfp4(blk)
+    codes = orc.unpack_u4(B)[0]
+    assert S[0, 0] == 127
+    assert list(codes[1:8]) == [1, 2, 3, 4, 5, 6, 7]
+    assert list(codes[8:15]) == [0, 1, 2, 3, 4, 5, 6]
+    assert list(codes[15:22]) == [9, 10, 11, 12, 13, 14, 15]
+    B, S = orc.quantize_mxfp4(np.zeros((2, 64), dtype=np.float32), scale_bias=127)
+    assert (B == 0).all() and (S == 0).all()
+    B, S = orc.quantize_mxfp4(np.zeros((2, 64), dtype=np.float32), scale_bias=0)   # raw-exponent mode clamps at 0
+    assert (B == 0).all() and (S == 0).all()
+
+
+def test_quantize_mxfp4_round_trip_and_idempotence():
+    """quantize(dequantize(codes, scales)) gives the codes and scales back whenever every block holds a code of
+    e2m1's top binade (4 or 6), and quantize is idempotent on arbitrary data."""
+    rng = np.random.default_rng(11)
+    N, K = 16, 256
+    codes = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    codes[codes == 8] = 0                                       # negative zero is never produced
+    top = rng.integers(0, 32, size=(N, K // 32))
+    for n in range(N):
+        for b in range(K // 32):
+            codes[n, b * 32 + top[n, b]] = rng.choice([6, 7, 14, 15])
+    scale = rng.integers(100, 140, size=(N, K // 32)).astype(np.uint8)
+    packed = orc.pack_fp4_e2m1_codes(codes)
+    w = orc.mxfp4_dequant(packed, scale, fmt="e2m1", scale_size=32, scale_bias=127)
+    B, S = orc.quantize_mxfp4(w, scale_bias=127)
+    np.testing.assert_array_equal(S, scale)
+    np.testing.assert_array_equal(B, packed)
+
+    x = orc.round_to_bf16((rng.standard_normal((N, K)) * np.exp2(rng.integers(-12, 12, size=(N, 1)))).astype(np.float32))
+    B1, S1 = orc.quantize_mxfp4(x)
+    d = orc.mxfp4_dequant(B1, S1, fmt="e2m1", scale_size=32, scale_bias=127)
+    B2, S2 = orc.quantize_mxfp4(d)
+    np.testing.assert_array_equal(B2, B1)
+    # the block maximum always lands in e2m1's top binade (scaled value in [4, 8) -> code 6 or 7), which is what
+    # makes the second pass choose the same exponent
+    assert ((orc.unpack_u4(B1).reshape(N, K // 32, 32) & 7).max(axis=-1) >= 6).all()
+    np.testing.assert_array_equal(S2, S1)
+    # error bound: half a step of the binade the scaled value falls in, or the saturation gap of the top binade
+    step = np.exp2(S1.astype(np.float64) - 127)[:, :, None]
+    err = np.abs(x.reshape(N, K // 32, 32) - d.reshape(N, K // 32, 32))
+    assert (err <= 2.0 * step + 1e-30).all()
+
+
+def test_gen_quant4_quantize_properties():
+    """The deterministic part of gen_quant4: scale = group absmax / 8 exactly; the largest element of a group
+    quantises to +-8; weights already on the grid come back unchanged; error at most half a step otherwise."""
+    rng = np.random.default_rng(5)
+    K, N, g = 256, 24, 64
+    w = rng.standard_normal((K, N)).astype(np.float16)
+    ref, s, q = orc.gen_quant4_quantize(w, g)
+    absmax = np.abs(w.reshape(K // g, g, N)).max(axis=1)
+    np.testing.assert_array_equal((s.astype(np.float32) * 8).astype(np.float16), absmax)
+    assert np.abs(q).max() == 8 and (np.abs(q.reshape(K // g, g, N)).max(axis=1) == 8).all()
+    step = np.repeat(s.astype(np.float32), g, axis=0)
+    # half a step, plus the fp16 roundings of w / s (before the rint) and of q * s: each below 2^-8 of a step
+    assert (np.abs(w.astype(np.float32) - ref.astype(np.float32)) <= 0.51 * step).all()
+    # on-grid weights: j * s0 with max |j| = 8 in every group
+    j = rng.integers(-8, 9, size=(K, N))
+    j.reshape(K // g, g, N)[:, 0, :] = 8
+    s0 = np.float16(0.0078125) * rng.integers(1, 64, size=(K // g, N)).astype(np.float16)
+    w_grid = (j.astype(np.float16) * np.repeat(s0, g, axis=0)).astype(np.float16)
+    ref, s, q = orc.gen_quant4_quantize(w_grid, g)
+    np.testing.assert_array_equal(s, s0)
+    np.testing.assert_array_equal(q, j)
+    np.testing.assert_array_equal(ref, w_grid)
+    # the whole-K group of groupsize = -1
+    ref, s, q = orc.gen_quant4_quantize(w, -1)
+    assert s.shape == (1, N) and np.abs(q).max() == 8
+

@@ -20,6 +20,7 @@ from .kernels import (  # noqa: F401
     matmul_nt_int4,
     matmul_w4_fine_grained,
     matmul_w4a16,
+    quantize_bf16_mxfp4,
 )
 from .bitlinear import BitLinear  # noqa: F401
 from .profiler import Profiler, TensorSupplyType, do_bench  # noqa: F401

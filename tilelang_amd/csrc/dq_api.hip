@@ -35,6 +35,7 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
 int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int out_kind, hipStream_t stream);
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
+int mxfp4_quant(const void* W, void* B, void* S, int N, int K, int scale_bias, hipStream_t stream);
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
             hipStream_t stream);
 
@@ -199,6 +200,19 @@ extern "C" int call_bitnet_activation_quant(const void* X, void* Q, void* S, int
   if (K % 8 != 0) DQ_FAIL("%s: K=%d must be a multiple of 8", fn, K);
   if (!aligned16(X) || ((uintptr_t)Q & 7) != 0) DQ_FAIL("%s: X must be 16-byte and Q 8-byte aligned", fn);
   return activation_quant(X, Q, S, M, K, (hipStream_t)stream);
+}
+
+extern "C" int call_quantize_bf16_mxfp4(const void* W, void* B, void* Scale, int N, int K, int scale_bias,
+                                        dq_stream_t stream) {
+  const char* fn = "call_quantize_bf16_mxfp4";
+  if (!W) DQ_FAIL("%s: W is expected to have non-NULL data pointer", fn);
+  if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
+  if (!Scale) DQ_FAIL("%s: Scale is expected to have non-NULL data pointer", fn);
+  if (N <= 0 || K <= 0) DQ_FAIL("%s: N and K must be positive (got %d, %d)", fn, N, K);
+  if (K % 32 != 0) DQ_FAIL("%s: K=%d must be a multiple of 32 (one scale per 32 elements)", fn, K);
+  if (scale_bias < 0 || scale_bias > 254) DQ_FAIL("%s: scale_bias=%d must be in 0..254", fn, scale_bias);
+  if (!aligned16(W) || ((uintptr_t)B & 3) != 0) DQ_FAIL("%s: W must be 16-byte and B 4-byte aligned", fn);
+  return mxfp4_quant(W, B, Scale, N, K, scale_bias, (hipStream_t)stream);
 }
 
 extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed,

@@ -1,5 +1,8 @@
-// BitLinear activation quantiser for gfx950: per-row absmax -> int8.
+// Quantisers that feed the dequantize-GEMM kernels on gfx950: the BitLinear activation quantiser
+// (per-row absmax -> int8) and the MXFP4 weight quantiser (bf16 -> e2m1 codes + one shared
+// power-of-two scale per 32 elements), further down.
 //
+// BitLinear activation quantiser.
 // Replaces BitLinearBitBLAS.activation_quant of examples/bitnet-1.58b/utils_quant.py:156-163 (a
 // torch.compile'd elementwise + row reduction):
 //     s[m]   = (1 / max(max_k |x[m, k]|, 1e-5)) * 127      (fp32; what torch's `Qp / tensor` computes)
@@ -106,6 +109,79 @@ __global__ __launch_bounds__(256) void activation_quant_kernel(const half_t* __r
   }
 }
 
+
+// ---- MXFP4 weight quantiser ---------------------------------------------------------------------
+// bf16 W[N, K] -> the operands of the MXFP4 GEMM (examples/dequantize_gemm/
+// example_dequant_gemm_bf16_mxfp4_cdna4.py:99-103): e2m1 codes, two per byte along K with the even
+// k in the low nibble, and one scale byte per 32 consecutive k.  Per block of 32:
+//     e      = max(floor(log2(max |w|)) - 2, -127)         (2 = exponent of e2m1's largest value, 6;
+//                                                           an all-zero block gets -127)
+//     byte   = clamp(e + scale_bias, 0, 255)
+//     code_i = e2m1(w_i / 2^(byte - scale_bias)),  magnitudes rounded at the thresholds 0.25, 0.75,
+//              1.25, 1.75, 2.5, 3.5, 5.0 (a value on a threshold goes up), saturating at 6; the sign
+//              bit is set only for non-zero magnitudes
+// The element rule is encode_fp4_e2m1_values of examples/dequantize_gemm/quantize/nvfp4.py:120-138;
+// the block scale is the OCP Microscaling v1.0 conversion (largest power of two that keeps the block
+// maximum inside e2m1's range after rounding down the exponent).  The division by a power of two is
+// exact, so codes and scale bytes are reproducible bit for bit.
+// A lane owns 8 consecutive elements (one 16-byte load, one packed dword out), the four lanes of a
+// quad own a block and agree on its maximum with two DPP steps.  HBM traffic: 2 bytes in,
+// 1/2 + 1/32 byte out per element.
+__device__ __forceinline__ uint32_t quad_max_u32(uint32_t v) {
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true));  // quad_perm(1,0,3,2)
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true));  // quad_perm(2,3,0,1)
+  return v;
+}
+
+template <int U>
+__global__ __launch_bounds__(256) void mxfp4_quant_kernel(const uint4_t* __restrict__ W, uint32_t* __restrict__ B,
+                                                          uint8_t* __restrict__ S, size_t pieces, int scale_bias) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t p0 = (size_t)blockIdx.x * 256 + threadIdx.x; p0 < pieces; p0 += stride * U) {
+    uint4_t raw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t p = p0 + u * stride;
+      // pieces is a multiple of 4 and p0 keeps the quad aligned: a quad is inside or outside as a whole
+      raw[u] = p < pieces ? __builtin_nontemporal_load(W + p) : uint4_t{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const size_t p = p0 + u * stride;
+      // non-negative floats order like their bit patterns: the block maximum in integer arithmetic
+      uint32_t amax = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) amax = max(amax, max(raw[u][i] & 0x7FFFu, (raw[u][i] >> 16) & 0x7FFFu));
+      amax = quad_max_u32(amax);
+      const int e = max((int)(amax >> 7) - 129, -127);       // exponent field - 127 - 2
+      const int byte = min(max(e + scale_bias, 0), 255);
+      const int e_used = min(max(byte - scale_bias, -127), 126);
+      // 2^-e_used (a normal float) times 1 + 2^-10: the products below stay exact (8 significant bits times 11),
+      // values on a threshold move just above it and nothing else crosses one (neighbouring bf16 values are at
+      // least 2^-8 apart, relatively), so the converter's round-to-nearest-even becomes "a threshold goes up"
+      const float inv = __builtin_bit_cast(float, (uint32_t)(127 - e_used) << 23) * 1.0009765625f;
+      uint32_t packed = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float lo = __builtin_bit_cast(float, raw[u][i] << 16) * inv;          // the bf16 pair as fp32
+        const float hi = __builtin_bit_cast(float, raw[u][i] & 0xFFFF0000u) * inv;
+        // v_cvt_scalef32_pk_fp4_f32: two e2m1 codes (saturating, round to nearest even) into byte i
+        if (i == 0) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, lo, hi, 1.0f, 0);
+        if (i == 1) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, lo, hi, 1.0f, 1);
+        if (i == 2) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, lo, hi, 1.0f, 2);
+        if (i == 3) packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, lo, hi, 1.0f, 3);
+      }
+      // no negative zero: keep a nibble's sign bit only where its magnitude bits are not all clear
+      const uint32_t nonzero = ((packed & 0x77777777u) + 0x77777777u) & 0x88888888u;
+      packed &= nonzero | 0x77777777u;
+      if (p < pieces) {
+        B[p] = packed;
+        if ((threadIdx.x & 3) == 0) S[p >> 2] = (uint8_t)byte;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream) {
@@ -121,6 +197,18 @@ int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t 
   else if (per_thread <= 8) DQ_AQ(8, wgs);
   else DQ_AQ(0, M);
 #undef DQ_AQ
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int mxfp4_quant(const void* W, void* B, void* S, int N, int K, int scale_bias, hipStream_t stream) {
+  const size_t pieces = (size_t)N * K / 8;
+  constexpr int kUnroll = 4;
+  const size_t per_wg = 256 * kUnroll;
+  size_t wgs = (pieces + per_wg - 1) / per_wg;
+  if (wgs > 256 * 8) wgs = 256 * 8;  // eight workgroups per CU, each walking the matrix with a grid stride
+  hipLaunchKernelGGL(mxfp4_quant_kernel<kUnroll>, dim3((unsigned)wgs), dim3(256), 0, stream, (const uint4_t*)W,
+                     (uint32_t*)B, (uint8_t*)S, pieces, scale_bias);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }

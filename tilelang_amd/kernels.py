@@ -478,6 +478,28 @@ def bitnet_activation_quant(M: int, K: int) -> KernelAdapter:
     return KernelAdapter("bitnet_activation_quant", params, [1, 2], launch, _lib.last_error)
 
 
+def quantize_bf16_mxfp4(N: int, K: int, scale_bias: int = 127) -> KernelAdapter:
+    """MXFP4 weight quantiser: ``B, Scale = kernel(W)`` with ``W`` bf16 ``[N, K]``, ``B`` uint8 ``[N, K/2]`` (e2m1
+    codes, even k in the low nibble) and ``Scale`` uint8 ``[N, K/32]`` — the operands that
+    :func:`matmul_bf16_mxfp4` takes and that the reference's example draws at random
+    (examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:286-290).
+
+    Per block of 32: ``e = max(floor(log2(max|w|)) - 2, -127)``, ``Scale = clamp(e + scale_bias, 0, 255)``, codes =
+    ``encode_fp4_e2m1_values(w / 2**(Scale - scale_bias))`` (examples/dequantize_gemm/quantize/nvfp4.py:120-138).
+    """
+    if K % 32 != 0:
+        raise ValueError(f"quantize_bf16_mxfp4: K={K} must be a multiple of 32")
+    if not 0 <= scale_bias <= 254:
+        raise ValueError(f"quantize_bf16_mxfp4: scale_bias={scale_bias} must be in 0..254")
+    params = [KernelParam("W", torch.bfloat16, (N, K)), KernelParam("B", torch.uint8, (N, K // 2)),
+              KernelParam("Scale", torch.uint8, (N, K // 32))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_quantize_bf16_mxfp4(ptrs[0], ptrs[1], ptrs[2], N, K, scale_bias, stream)
+
+    return KernelAdapter("quantize_bf16_mxfp4", params, [1, 2], launch, _lib.last_error)
+
+
 def bitnet_158_int8xint2_decode(
     M: int,
     N: int,

@@ -2,8 +2,9 @@
 
 Same names and argument meaning as the helpers the reference's examples import:
 ``general_compress`` / ``interleave_weight`` (examples/dequantize_gemm/quantize/utils.py:50-125),
-``pack_int4`` (examples/gemm_int4/example_tilelang_gemm_int4.py:59-67), and the e2m1
-helpers of examples/dequantize_gemm/quantize/nvfp4.py:120-177.
+``pack_int4`` (examples/gemm_int4/example_tilelang_gemm_int4.py:59-67), the e2m1
+helpers of examples/dequantize_gemm/quantize/nvfp4.py:120-177, and ``gen_quant4``
+(examples/dequantize_gemm/quantize/utils.py:1-47) with a packer from its layout to this library's.
 """
 
 from __future__ import annotations
@@ -112,3 +113,45 @@ def decode_packed_fp4_e2m1(packed: torch.Tensor, cols: int | None = None) -> tor
     lut = torch.tensor(FP4_E2M1_VALUES, device=packed.device, dtype=torch.float32)
     nib = torch.stack((u & 0x0F, u >> 4), dim=-1).reshape(packed.shape[0], cols)
     return lut[nib.long()]
+
+
+def gen_quant4(k: int, n: int, groupsize: int = -1):
+    """Random fp16 ``w[k, n]`` quantised to 4 bits per (group of ``groupsize`` consecutive k, column): returns
+    ``(original_w, linear, s, q)`` like ``gen_quant4`` of examples/dequantize_gemm/quantize/utils.py:1-47 —
+    ``s[k/groupsize, n]`` fp16 = group absmax * 2/16, ``q[k, n]`` int32 = ``clamp(round(w/s) + 8, 0, 16) - 8``,
+    ``linear`` an ``nn.Linear(k, n, bias=False)`` whose weight is the dequantised ``(q.half() * s).T``.
+
+    As in the reference ``maxq`` is 16, so ``q`` reaches +8 (code 16) for a group's largest positive element;
+    :func:`pack_gen_quant4` deals with that when the codes have to fit a nibble.
+    """
+    maxq = 2**4
+    if groupsize == -1:
+        groupsize = k
+    if k % groupsize:
+        raise ValueError(f"gen_quant4: k={k} is not a multiple of groupsize={groupsize}")
+    original_w = torch.randn((k, n), dtype=torch.half, device="cpu")
+    grouped = original_w.reshape(k // groupsize, groupsize, n)
+    s = grouped.abs().amax(dim=1, keepdim=True) * (2 / maxq)
+    q = torch.clamp(torch.round(grouped / s).int() + maxq // 2, 0, maxq)
+    ref = (q - maxq // 2).half() * s
+    linear = torch.nn.Linear(k, n, bias=False)
+    linear.weight.data = ref.reshape(k, n).t()
+    return original_w, linear, s.reshape(k // groupsize, n).contiguous(), (q - maxq // 2).reshape(k, n)
+
+
+def pack_gen_quant4(q: torch.Tensor, s: torch.Tensor, saturate: bool = False):
+    """``gen_quant4``'s ``q[k, n]`` (values -8..8) and ``s[k/g, n]`` -> this library's W4A16 operands
+    ``B[n, k/2]`` int8 (codes ``q + 8``, even k in the low nibble) and ``Scale[n, k/g]`` fp16, for
+    ``dequantize_gemv(..., source_format="int", with_scaling=True)`` (``w = (code - 8) * s``).
+
+    Code 16 (``q = +8``) does not fit a nibble: with ``saturate=False`` that raises, with ``saturate=True`` it is
+    stored as 15 (the dequantised value of that element is then ``7 s`` instead of ``8 s``).
+    """
+    codes = (q.to(torch.int32) + 8).t().contiguous()
+    if int(codes.min()) < 0 or int(codes.max()) > 16:
+        raise ValueError("pack_gen_quant4: q must be in -8..8")
+    if int(codes.max()) > 15:
+        if not saturate:
+            raise ValueError("pack_gen_quant4: code 16 does not fit 4 bits (pass saturate=True to store 15)")
+        codes = codes.clamp(max=15)
+    return general_compress(codes.to(torch.int8), 4), s.t().contiguous().to(torch.float16)
