@@ -67,13 +67,10 @@ struct I2Policy : I8Mfma, gemm::NoScale, EPI {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       uint32_t d = (w[j] >> (2 * i)) & 0x03030303u;
-      if constexpr (CONV == I2_OFFSET) {
-        // per byte c - 2 without a borrow between bytes: ((c | 0x80) - 2) ^ 0x80
-        d = ((d | 0x80808080u) - 0x02020202u) ^ 0x80808080u;
-      } else if constexpr (CONV == I2_TWOS) {
-        // sext2(c) = (c ^ 2) - 2
-        d = (((d ^ 0x02020202u) | 0x80808080u) - 0x02020202u) ^ 0x80808080u;
-      }
+      // each byte of d is a code 0..3: as the selector of v_perm_b32 it picks the code's int8 value out of a
+      // four-byte table (offset binary: c - 2; two's complement: sext2(c)), one instruction per dword
+      if constexpr (CONV == I2_OFFSET) d = __builtin_amdgcn_perm(0u, 0x0100FFFEu, d);
+      else if constexpr (CONV == I2_TWOS) d = __builtin_amdgcn_perm(0u, 0xFFFE0100u, d);
       o[i] = (int)d;
     }
     return o;
