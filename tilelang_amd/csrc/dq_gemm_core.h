@@ -421,7 +421,9 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
 // and the 256-register budget spills), so it is kept as a build option only.  kNBW = 2: the same
 // 256 x 256 tile on eight waves (two per SIMD, wave tile 128 x 64): no spills and the same decode work,
 // but every A fragment is read from LDS by twice as many waves; measured 4 % slower on that
-// problem (410 us against 393 us), also a build option only (-DDQ_DMA_NBW=2).
+// problem (410 us against 393 us), also a build option only (-DDQ_DMA_NBW=2).  Eight waves of 64 x 128
+// (four along the rows, which keeps the LDS traffic of the four-wave form) measured the same 410 us: a
+// second wave per SIMD does not buy MFMA issue slots here.
 template <class P, int kMBW, int kNBW>
 __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
