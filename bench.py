@@ -290,6 +290,8 @@ def main():
         for m in (1, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, k if m == 1 else kg, 2, dev)
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, max(5, k // 4), 2, dev)
+        shapes.append(_row("w4a16_zeros_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
         r = bench_mxfp4_quant(torch, tl, 8192, 8192, k, 2, dev)
         shapes.append(_row("mxfp4_quantize N=8192 K=8192", r, "hbm", MFMA_BF16_PEAK))
         r = bench_activation_quant(torch, tl, 2048, 8192, k, 2, dev)

@@ -88,9 +88,10 @@ def test_fp16_fp4_weights_exact(cuda):
 
 @pytest.mark.parametrize("mode", ["scale", "original", "rescale", "signed"])
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("M,N,K", [(200, 320, 512), (1500, 2000, 256), (3581, 3589, 128)])  # 128x64, 128x128, 256x256 tiles
+@pytest.mark.parametrize("M,N,K", [(200, 320, 512), (1500, 2000, 256), (3581, 3589, 128), (3581, 3589, 768),
+                                   (3584, 3584, 256)])  # 128x64, 128x128, 256x256 tiles; the last two: direct-to-LDS kernel
 def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
-    """W4A16 through the MFMA GEMM (M > 64): same tile-exact decoders as the decode kernel."""
+    """W4A16 through the MFMA GEMM (M > 128): same tile-exact decoders as the decode kernel."""
     group = 128
     d = workloads.w4a16(M, N, K, group, seed=2, scale_range=(0.002, 0.01), zeros_range=(6, 10))
     kw = {"scale": dict(source_format="int"), "original": dict(source_format="uint", with_zeros=True),

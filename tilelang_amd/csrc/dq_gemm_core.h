@@ -400,8 +400,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
 
 // ---- direct-to-LDS variant ---------------------------------------------------------------------
 // For policies whose A needs no transform on its way to LDS (any per-fragment transform is P::fix_a,
-// applied after the fragment is read) and whose scales are either absent or one byte per 32 k
-// (P::kScaleBytes): the A and packed-B tiles, and the scale bytes, travel
+// applied after the fragment is read) and whose scales are absent, one byte per 32 k or one fp16 (plus
+// one fp16 zero) per 128 k (P::kScaleDma): the A and packed-B tiles, and the scales, travel
 // global -> LDS with global_load_lds_dwordx4 / _dword, two tiles ahead of the MFMAs, without
 // passing through registers.  A lane's 16 bytes land at LDS base + lane * 16 whatever its source
 // address, so the XOR swizzle of the A rows is applied by permuting the SOURCE addresses.  These
@@ -439,7 +439,11 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
   constexpr int kStage = kAStage + kBStage;    // 40 or 24 KiB
   constexpr int kStages = 3;
-  constexpr int kRing = kStages * kStage;      // scale ring: 4 slots x 1 KiB (256 rows x 4 scale bytes = 2 tiles)
+  // Scales that travel by DMA (P::kScaleDma): 1 = one byte per 32 k (a dword per row covers a pair of tiles),
+  // 2 = one fp16 per 128 k (a dword per row covers four tiles), 3 = the same for scales and for zeros.
+  // Ring: 4 slots x 1 KiB (256 rows x one dword), a second ring for the zeros.
+  constexpr int kRing = kStages * kStage;
+  constexpr int kSOps = P::kScaleDma == 0 ? 0 : (P::kScaleDma == 3 ? 2 : 1);  // scale DMA instructions per wave per tile
   constexpr int kBWords = 4;
 
   const int tid = threadIdx.x;
@@ -469,28 +473,32 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     const int row = c >> 1, pp = c & 1;
     b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K * P::kBRowBytes / P::kKPerBlock) + (unsigned)(((pp + (row >> 3)) & 1) << 4);
   }
-  const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(K >> 5);  // waves 4..7 repeat 0..3
+  const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(P::kScaleDma == 1 ? (K >> 5) : (K >> 6));  // waves 4..7 repeat 0..3
 
-  // One tile = 3 + kAOps DMA instructions per thread: op 0 the scale dword (rows tid, tiles 2p and 2p+1;
-  // issued with every tile, i.e. twice per pair, which keeps the loop branch-free), then the A chunks,
-  // then the two packed-B chunks.
-  constexpr int kTileOps = 1 + kAOps + kBOps;
+  // One tile = kSOps + kAOps + kBOps DMA instructions per thread: first the scale dword(s) (row tid; issued
+  // with every tile although a dword serves two or four, which keeps the loop branch-free), then the A
+  // chunks, then the packed-B chunks.
+  constexpr int kTileOps = kSOps + kAOps + kBOps;
   auto issue_op = [&](int op, int kb, int stage) {
     const unsigned sbase = lds0 + stage * kStage;
-    if (op == 0) {
-      if constexpr (P::kScaleBytes) {
+    if (op < kSOps) {
+      if constexpr (P::kScaleDma == 1) {
         const int pair = kb >> 1;
         dma4(lds0 + kRing + (pair & 3) * 1024 + (wave & 3) * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
+      } else if constexpr (P::kScaleDma >= 2) {
+        const int quad = kb >> 2;
+        dma4(lds0 + kRing + op * 4096 + (quad & 3) * 1024 + (wave & 3) * 256, s_voff,
+             (const unsigned char*)(op == 0 ? p.S : p.Z) + (size_t)quad * 4);
       }
-    } else if (op <= kAOps) {
-      const int i = op - 1;
+    } else if (op < kSOps + kAOps) {
+      const int i = op - kSOps;
       dma16(sbase + (wave * kAOps + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
     } else {
-      const int i = op - 1 - kAOps;
+      const int i = op - kSOps - kAOps;
       dma16(sbase + kAStage + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * 32);
     }
   };
-  constexpr int kWaitOps = P::kScaleBytes ? kTileOps : kTileOps - 1;  // outstanding DMA instructions of one tile
+  constexpr int kWaitOps = kTileOps;  // outstanding DMA instructions of one tile
 
   // ---- fragment read offsets (same LDS geometry as the register-staged kernel) --------------------
   int a_row_off[kMBW], a_row_sw[kMBW], b_off[kNBW], s_off[kNBW];
@@ -504,7 +512,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   for (int nb = 0; nb < kNBW; ++nb) {
     const int row = wn * (32 * kNBW) + nb * 32 + r;
     b_off[nb] = kAStage + row * 32 + (((g + (row >> 3)) & 1) << 4);
-    s_off[nb] = kRing + row * 4 + g;
+    s_off[nb] = kRing + row * 4 + (P::kScaleDma == 1 ? g : 0);
   }
   using frag_t = typename P::frag_t;
   auto read_a1 = [&](const unsigned char* base, int j, int mb) -> frag_t {
@@ -515,9 +523,14 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     bw[0] = v[0]; bw[1] = v[1]; bw[2] = v[2]; bw[3] = v[3];
   };
   auto read_scale1 = [&](int kb, int nb) -> typename P::Scale {
-    int e = 0;
-    if constexpr (P::kScaleBytes) e = smem[s_off[nb] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2];
-    return P::prep_scale(e, p);
+    if constexpr (P::kScaleDma >= 2) {
+      const unsigned char* at = smem + s_off[nb] + ((kb >> 2) & 3) * 1024 + ((kb >> 1) & 1) * 2;
+      return P::ring_scale(at, at + 4096);
+    } else {
+      int e = 0;
+      if constexpr (P::kScaleDma == 1) e = smem[s_off[nb] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2];
+      return P::prep_scale(e, p);
+    }
   };
 
   typename P::acc_t acc[kMBW][kNBW];
@@ -687,13 +700,14 @@ template <class P>
 bool dma_eligible(const Params& p) {
   // the direct-to-LDS kernel has one tile shape (256 x 256): small problems go to the tile-size choice above
   const long tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  return (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) && ((size_t)p.N * p.K / 2 < (1ull << 32));
+  return P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) &&
+         ((size_t)p.N * p.K / 2 < (1ull << 32));
 }
 
 template <class P, int kMBW, int kNBW>
 int launch_dma_tile(Params p, hipStream_t stream) {
   constexpr int kWaves = 16 / kNBW;
-  constexpr int kPipe = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + 4 * 1024;
+  constexpr int kPipe = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + 8 * 1024;
   constexpr int kSlabs = kWaves * 32 * (32 * kNBW + 4) * 4;  // epilogue staging
   constexpr int kLds = kPipe > kSlabs ? kPipe : kSlabs;
   p.tiles_m = (p.M + 64 * kMBW - 1) / (64 * kMBW);
@@ -727,6 +741,8 @@ inline Params make_params(const void* A, const void* B, const void* S, const voi
 // ---- building blocks shared by the policies -------------------------------------------------------
 
 struct NoScale {
+  static constexpr int kScaleDma = 0;  // no scales to bring in by DMA
+  static bool dma_ok(const Params&) { return true; }
   struct ScaleRaw {};
   struct Scale {};
   __device__ static __forceinline__ ScaleRaw fetch_scale(const Params&, int, int, int) { return {}; }

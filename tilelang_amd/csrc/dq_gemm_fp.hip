@@ -85,7 +85,8 @@ struct MxPolicy : Bf16Mfma, gemm::PlainA {
   static constexpr bool kTransposed = false;
   using out_t = bf16_t;
   using ScaleRaw = int;
-  static constexpr bool kScaleBytes = true;  // one scale byte per 32 k: eligible for the direct-to-LDS kernel
+  static constexpr int kScaleDma = 1;  // one scale byte per 32 k travels by DMA in the direct-to-LDS kernel
+  static bool dma_ok(const Params&) { return true; }
   struct Scale { float f; uint32_t add; };
   __device__ static __forceinline__ ScaleRaw fetch_scale(const Params& p, int row, int kb, int g) {
     return ((const uint8_t*)p.S)[(size_t)row * (p.K >> 5) + kb * 2 + g];
@@ -120,7 +121,6 @@ struct MxPolicy : Bf16Mfma, gemm::PlainA {
 template <bool TRANSPOSED>
 struct Fp16Fp4Policy : F16Mfma, gemm::PlainA, gemm::NoScale {
   static constexpr int kBRowBytes = 32;
-  static constexpr bool kScaleBytes = false;
   __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
   using gemm::NoScale::prep_scale;
   static constexpr bool kTransposed = TRANSPOSED;
@@ -143,8 +143,23 @@ struct W4F16Policy : F16Mfma {
   using out_t = half_t;
   struct ScaleRaw { half_t s, z; };
   using Scale = ScaleRaw;
-  // the plain-layout decoder emits nibble pairs (e, e+4): activations get the same order
+  // direct-to-LDS kernel: with one scale (and zero) per 128 k the fp16 values travel by DMA, a dword per row
+  // (two groups = four tiles of 64 k) at a time; other group sizes stay on the register-staged kernel
+  static constexpr int kScaleDma = MODE >= W4_ZEROS_ORIGINAL ? 3 : (MODE >= W4_SCALE ? 2 : 0);
+  static bool dma_ok(const Params& p) { return kScaleDma == 0 || (p.p0 == 7 && p.K % 256 == 0); }
+  __device__ static __forceinline__ Scale ring_scale(const unsigned char* s_at, const unsigned char* z_at) {
+    Scale r{(half_t)1.f, (half_t)0.f};
+    r.s = *reinterpret_cast<const half_t*>(s_at);
+    if constexpr (kScaleDma == 3) r.z = *reinterpret_cast<const half_t*>(z_at);
+    return r;
+  }
+  __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return Scale{(half_t)1.f, (half_t)0.f}; }
+  // the plain-layout decoder emits nibble pairs (e, e+4): activations get the same order, on their way to LDS
+  // (register-staged kernel) or fragment by fragment after the LDS read (direct-to-LDS kernel)
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : permute_k8_16bit(v); }
+  __device__ static __forceinline__ frag_t fix_a(frag_t f) {
+    return INTERLEAVED ? f : __builtin_bit_cast(frag_t, permute_k8_16bit(__builtin_bit_cast(uint4_t, f)));
+  }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
   __device__ static __forceinline__ ScaleRaw fetch_scale(const Params& p, int row, int kb, int g) {
     ScaleRaw r{(half_t)1.f, (half_t)0.f};
@@ -203,8 +218,12 @@ int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void
   p.p1 = K / group;
 #define DQ_W4(MODE_)                                                                        \
   do {                                                                                      \
-    if (layout == LAYOUT_PLAIN) return gemm::launch_auto<W4F16Policy<MODE_, false>>(p, stream);  \
-    return gemm::launch_auto<W4F16Policy<MODE_, true>>(p, stream);                               \
+    if (layout == LAYOUT_PLAIN) {                                                           \
+      if (gemm::dma_eligible<W4F16Policy<MODE_, false>>(p)) return gemm::launch_dma<W4F16Policy<MODE_, false>>(p, stream); \
+      return gemm::launch_auto<W4F16Policy<MODE_, false>>(p, stream);                       \
+    }                                                                                       \
+    if (gemm::dma_eligible<W4F16Policy<MODE_, true>>(p)) return gemm::launch_dma<W4F16Policy<MODE_, true>>(p, stream); \
+    return gemm::launch_auto<W4F16Policy<MODE_, true>>(p, stream);                          \
   } while (0)
   switch (mode) {
     case W4_UNSIGNED: DQ_W4(W4_UNSIGNED);

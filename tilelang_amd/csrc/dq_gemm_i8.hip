@@ -56,7 +56,6 @@ struct I2Policy : I8Mfma, gemm::NoScale, EPI {
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : transpose4x4_bytes(v); }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
   // direct-to-LDS kernel: A lands in LDS untouched and each 16-byte fragment is transposed after the read
-  static constexpr bool kScaleBytes = false;
   __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
   using gemm::NoScale::prep_scale;
   __device__ static __forceinline__ frag_t fix_a(frag_t f) {
