@@ -18,7 +18,8 @@ def _dev(x, cuda):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 256, 256), (512, 512, 512), (100, 130, 384), (1, 8, 128),
-                                   (1500, 2000, 256), (3581, 3589, 128)])  # the last two: 128x128 and 256x256 tiles
+                                   (1500, 2000, 256), (3581, 3589, 128), (3581, 3589, 768),
+                                   (3584, 3584, 256)])  # 128x128 tiles, 256x256 tiles, and twice the direct-to-LDS kernel
 def test_w4a8_exact(cuda, M, N, K):
     """examples/dequantize_gemm/example_dequant_gemm_w4a8.py: Ct[N,M] int32, all byte values."""
     d = workloads.int8_int4(M, N, K, seed=M)
@@ -59,6 +60,17 @@ def test_fine_grained(cuda, in_dtype):
         torch.cuda.synchronize()
         ref = orc.ref_w4a16(A, B, mode="unsigned")
         np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL * 10)
+
+
+def test_fine_grained_int8_many_tiles(cuda):
+    """The unsigned-nibble int8 path with enough 256 x 256 tiles for the direct-to-LDS kernel, ragged edges."""
+    M, N, K = 3581, 3589, 512
+    rng = np.random.default_rng(4)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    C = tl.matmul_w4_fine_grained(M, N, K, in_dtype="int8")(_dev(A, cuda), _dev(B, cuda).view(torch.int8))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_u4_int8(A, B))
 
 
 @pytest.mark.parametrize("transposed", [True, False])

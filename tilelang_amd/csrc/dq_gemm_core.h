@@ -427,7 +427,7 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
 template <class P, int kMBW, int kNBW>
 __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
   extern __shared__ __align__(16) unsigned char smem[];
-  static_assert(P::kBRowBytes == 32, "direct-to-LDS variant: 32 packed bytes per weight row per tile");
+  static_assert(P::kBRowBytes == 32 || P::kBRowBytes == 64, "direct-to-LDS variant: 32 or 64 packed bytes per weight row per tile");
   static_assert(kMBW == 2 || kMBW == 4, "wave tile of 64 or 128 rows");
   static_assert(kNBW == 2 || kNBW == 4, "wave tile of 64 or 128 columns");
   constexpr int kWavesN = 8 / kNBW;            // waves across the 256 tile columns
@@ -435,7 +435,9 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   constexpr int BM = 64 * kMBW;                // shadows the 256-row default
   constexpr int kAStage = BM * kARowBytes;     // 32 or 16 KiB
   constexpr int kAOps = 8 * kMBW / kWaves;     // A DMA instructions per wave per tile
-  constexpr int kBOps = 8 / kWaves;            // packed-B DMA instructions per wave per tile
+  constexpr int kBPiecesPerRow = P::kBRowBytes / 16;          // 2 or 4
+  constexpr int kBRot = kBPiecesPerRow == 2 ? 3 : 2;          // piece rotation advances every 8 or 4 rows
+  constexpr int kBOps = BN * kBPiecesPerRow / 64 / kWaves;    // packed-B DMA instructions per wave per tile
   constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
   constexpr int kStage = kAStage + kBStage;    // 40 or 24 KiB
   constexpr int kStages = 3;
@@ -444,7 +446,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   // Ring: 4 slots x 1 KiB (256 rows x one dword), a second ring for the zeros.
   constexpr int kRing = kStages * kStage;
   constexpr int kSOps = P::kScaleDma == 0 ? 0 : (P::kScaleDma == 3 ? 2 : 1);  // scale DMA instructions per wave per tile
-  constexpr int kBWords = 4;
+  constexpr int kBWords = P::kBRowBytes / 8;   // dwords per lane and 32-row block: 4 or 8
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -469,9 +471,11 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   }
 #pragma unroll
   for (int i = 0; i < kBOps; ++i) {
-    const int c = (wave * kBOps + i) * 64 + lane;  // B chunk: row c / 2, physical piece c % 2
-    const int row = c >> 1, pp = c & 1;
-    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K * P::kBRowBytes / P::kKPerBlock) + (unsigned)(((pp + (row >> 3)) & 1) << 4);
+    const int c = (wave * kBOps + i) * 64 + lane;  // B chunk: row c / pieces per row, physical piece c % pieces per row
+    const int row = c / kBPiecesPerRow, pp = c % kBPiecesPerRow;
+    // LDS position (piece + rotation) % pieces holds source piece `piece`
+    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K * P::kBRowBytes / P::kKPerBlock) +
+                (unsigned)(((pp - (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);
   }
   const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(P::kScaleDma == 1 ? (K >> 5) : (K >> 6));  // waves 4..7 repeat 0..3
 
@@ -495,13 +499,13 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
       dma16(sbase + (wave * kAOps + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
     } else {
       const int i = op - kSOps - kAOps;
-      dma16(sbase + kAStage + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * 32);
+      dma16(sbase + kAStage + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * P::kBRowBytes);
     }
   };
   constexpr int kWaitOps = kTileOps;  // outstanding DMA instructions of one tile
 
   // ---- fragment read offsets (same LDS geometry as the register-staged kernel) --------------------
-  int a_row_off[kMBW], a_row_sw[kMBW], b_off[kNBW], s_off[kNBW];
+  int a_row_off[kMBW], a_row_sw[kMBW], b_off[kNBW][kBPiecesPerRow / 2], s_off[kNBW];
 #pragma unroll
   for (int mb = 0; mb < kMBW; ++mb) {
     const int row = wm * (32 * kMBW) + mb * 32 + r;
@@ -511,7 +515,11 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
 #pragma unroll
   for (int nb = 0; nb < kNBW; ++nb) {
     const int row = wn * (32 * kNBW) + nb * 32 + r;
-    b_off[nb] = kAStage + row * 32 + (((g + (row >> 3)) & 1) << 4);
+#pragma unroll
+    for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
+      const int piece = g * (kBPiecesPerRow / 2) + h;
+      b_off[nb][h] = kAStage + row * P::kBRowBytes + (((piece + (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);
+    }
     s_off[nb] = kRing + row * 4 + (P::kScaleDma == 1 ? g : 0);
   }
   using frag_t = typename P::frag_t;
@@ -519,8 +527,11 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     return P::fix_a(*reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4)));
   };
   auto read_b1 = [&](const unsigned char* base, int nb, uint32_t (&bw)[kBWords]) {
-    const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb]);
-    bw[0] = v[0]; bw[1] = v[1]; bw[2] = v[2]; bw[3] = v[3];
+#pragma unroll
+    for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
+      const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb][h]);
+      bw[4 * h + 0] = v[0]; bw[4 * h + 1] = v[1]; bw[4 * h + 2] = v[2]; bw[4 * h + 3] = v[3];
+    }
   };
   auto read_scale1 = [&](int kb, int nb) -> typename P::Scale {
     if constexpr (P::kScaleDma >= 2) {
@@ -700,8 +711,10 @@ template <class P>
 bool dma_eligible(const Params& p) {
   // the direct-to-LDS kernel has one tile shape (256 x 256): small problems go to the tile-size choice above
   const long tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  return P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && ((size_t)p.M * p.K * 2 < (1ull << 32)) &&
-         ((size_t)p.N * p.K / 2 < (1ull << 32));
+  // 32-bit lane offsets: A rows are 128 bytes per K block, packed B rows kBRowBytes
+  const size_t a_bytes = (size_t)p.M * (p.K / P::kKPerBlock) * kARowBytes;
+  const size_t b_bytes = (size_t)p.N * (p.K / P::kKPerBlock) * P::kBRowBytes;
+  return P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
 }
 
 template <class P, int kMBW, int kNBW>

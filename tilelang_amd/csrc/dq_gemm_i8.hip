@@ -91,6 +91,14 @@ struct I4Policy : I8Mfma, gemm::NoScale, EPI {
     return SIGNED ? (w & 0xF0F0F0F0u) : ((w >> 4) & 0x0F0F0F0Fu);
   }
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return split_even_odd_bytes(v); }
+  // direct-to-LDS kernel (int8 A only: a packed A is expanded on its way to LDS): the byte shuffle moves behind
+  // the LDS read, fragment by fragment
+  static bool dma_ok(const Params&) { return !A_PACKED; }
+  __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
+  using gemm::NoScale::prep_scale;
+  __device__ static __forceinline__ frag_t fix_a(frag_t f) {
+    return __builtin_bit_cast(frag_t, split_even_odd_bytes(__builtin_bit_cast(uint4_t, f)));
+  }
   __device__ static __forceinline__ void expand_a(uint4_t v, uint4_t& lo, uint4_t& hi) {
     lo = uint4_t{even(v[0]), odd(v[0]), even(v[1]), odd(v[1])};
     hi = uint4_t{even(v[2]), odd(v[2]), even(v[3]), odd(v[3])};
@@ -139,12 +147,19 @@ int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_s
     if (transposed) return gemm::launch_auto<I4Policy<true, true, Int32Out<8, true>>>(p, stream);
     return gemm::launch_auto<I4Policy<true, true, Int32Out<8, false>>>(p, stream);
   }
+#define DQ_I4(SIGNED_, SHIFT_, TRANS_)                                        \
+  do {                                                                        \
+    using Pol = I4Policy<SIGNED_, false, Int32Out<SHIFT_, TRANS_>>;           \
+    if (gemm::dma_eligible<Pol>(p)) return gemm::launch_dma<Pol>(p, stream);  \
+    return gemm::launch_auto<Pol>(p, stream);                                 \
+  } while (0)
   if (is_signed) {
-    if (transposed) return gemm::launch_auto<I4Policy<true, false, Int32Out<4, true>>>(p, stream);
-    return gemm::launch_auto<I4Policy<true, false, Int32Out<4, false>>>(p, stream);
+    if (transposed) DQ_I4(true, 4, true);
+    DQ_I4(true, 4, false);
   }
-  if (transposed) return gemm::launch_auto<I4Policy<false, false, Int32Out<0, true>>>(p, stream);
-  return gemm::launch_auto<I4Policy<false, false, Int32Out<0, false>>>(p, stream);
+  if (transposed) DQ_I4(false, 0, true);
+  DQ_I4(false, 0, false);
+#undef DQ_I4
 }
 
 }  // namespace dq
