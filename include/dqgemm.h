@@ -57,7 +57,7 @@ enum dq_w4_layout {
 /* C[M,N] fp16 = A[M,K] fp16 . dequant(B[N,K/2], Scale[N,K/group], Zeros[N,K/group])^T,
  * fp32 accumulation.  Replaces `call(A, B, C, stream)` of the kernel generated from
  * examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:83-153 (M = 1) and its
- * batched use (M up to 64 per pass; larger M loops over blocks of 64 rows).
+ * batched use (decode kernels up to M = 128; larger M goes to the tiled GEMM of call_dequant_gemm_w4_fp16).
  * Requires K % 128 == 0, group % 32 == 0, K % group == 0 (group = K when there is one
  * scale per row).  Scale / Zeros may be NULL for modes that do not read them.
  * `variant` < 0 selects the kernel configuration heuristically. */

@@ -92,10 +92,10 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   // prefill-sized M: the tiled MFMA GEMM (same tile-exact decoders); up to 128 rows the streaming kernel
   // below (two passes over the weights) is still the faster one.  50: the GEMM whatever M.
   if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
-  // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread
-  // (r = 0: its own choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with register-resident
-  // activations (M <= 16).  0..12: a
-  // configuration of the tiled MFMA kernel (covers every shape).
+  // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread (r = 0: its own
+  // choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with
+  // register-resident activations (M <= 16).  0, 4, 5, 10: a configuration of the tiled MFMA fallback kernel
+  // (covers every shape).
   if (variant == 40 || (variant < 0 && M >= 3 && M <= 16)) {
     // a handful of rows: activations resident in registers (shapes it does not cover fall through)
     const int rc = w4a16_regres(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
