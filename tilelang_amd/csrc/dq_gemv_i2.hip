@@ -160,7 +160,9 @@ int launch_i2_gemv(const void* A, const void* B, void* C, const void* s_a, float
   constexpr int R = 4 / NP;
   const int rpp = 256 >> tpr_shift;
   const long wgs1 = ((long)N + R * rpp - 1) / (R * rpp);
-  int nb = (int)((wgs1 + 1791) / 1792);
+  // about two workgroups per CU, each walking several batches: at N = K = 8192 one batch per workgroup (1024
+  // workgroups) measured 7.4 us, two 6.3 us, four 6.2 us, eight 8.6 us
+  int nb = (int)((wgs1 + 511) / 512);
   while (nb > 1 && nb * R * rpp > kMaxRowsPerWg) --nb;
   if (nb < 1) nb = 1;
   const int rows_per_wg = nb * R * rpp;
