@@ -186,8 +186,9 @@ __global__ __launch_bounds__(256) void mxfp4_quant_kernel(const uint4_t* __restr
 
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream) {
   const int per_thread = (K / 8 + 255) / 256;  // 16-byte pieces per thread
-  // register-resident rows: at most 2 workgroups per CU in flight, each walking several rows
-  const int wgs = M < 512 ? M : 512;
+  // register-resident rows: up to eight workgroups per CU, each walking rows with a grid stride (M = 2048,
+  // K = 8192: 11.0 us with one row per workgroup, 12.9 us with 512 workgroups of four rows, 17.7 us with 256)
+  const int wgs = M < 2048 ? M : 2048;
 #define DQ_AQ(NV_, GRID_)                                                                                              \
   hipLaunchKernelGGL(activation_quant_kernel<NV_>, dim3(GRID_), dim3(256), 0, stream, (const half_t*)X, (int8_t*)Q, \
                      (float*)S, M, K)
