@@ -319,6 +319,9 @@ int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, 
   if (nb == 0) {
     const long wgs1 = ((long)N + r * rpp - 1) / (r * rpp);
     nb = (int)((wgs1 + 1791) / 1792);
+    // long rows on a short matrix (N = 4096, K = 11008: 7.3 us with 1024 workgroups of one batch, 6.7 us with
+    // 512 of two): let a workgroup overlap its second batch's loads with the first one's arithmetic
+    if (np >= 2 && wgs1 >= 512 && wgs1 <= 1024) nb = 2;
   }
   while (nb > 1 && (nb * r * rpp > kMaxRowsPerWg || nb * r > kMaxRowsPerWg)) --nb;
   if (nb < 1) nb = 1;
