@@ -526,22 +526,26 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   auto read_a1 = [&](const unsigned char* base, int j, int mb) -> frag_t {
     return P::fix_a(*reinterpret_cast<const frag_t*>(base + a_row_off[mb] + ((((g << 2) + j) ^ a_row_sw[mb]) << 4)));
   };
+  // 32 rows further down the rotation of the packed-B pieces repeats ((32 >> kBRot) % kBPiecesPerRow == 0)
+  // and the scale rows are 4 bytes apart: block nb sits at a constant distance from block 0, so one
+  // address per tile serves all kNBW reads through their immediate offsets
+  static_assert((32 >> kBRot) % kBPiecesPerRow == 0, "B rotation must repeat every 32 rows");
   auto read_b1 = [&](const unsigned char* base, int nb, uint32_t (&bw)[kBWords]) {
 #pragma unroll
     for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
-      const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[nb][h]);
+      const uint4_t v = *reinterpret_cast<const uint4_t*>(base + b_off[0][h] + nb * (32 * P::kBRowBytes));
       bw[4 * h + 0] = v[0]; bw[4 * h + 1] = v[1]; bw[4 * h + 2] = v[2]; bw[4 * h + 3] = v[3];
     }
   };
   // the LDS read of a scale and the arithmetic on it are separate steps, so that the read can be issued a
   // chunk ahead of its first use
   auto read_scale_byte = [&](int kb, int nb) -> int {
-    if constexpr (P::kScaleDma == 1) return smem[s_off[nb] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2];
+    if constexpr (P::kScaleDma == 1) return (smem + s_off[0] + ((kb >> 1) & 3) * 1024 + (kb & 1) * 2)[nb * 128];
     else return 0;
   };
   auto read_scale1 = [&](int kb, int nb) -> typename P::Scale {
     if constexpr (P::kScaleDma >= 2) {
-      const unsigned char* at = smem + s_off[nb] + ((kb >> 2) & 3) * 1024 + ((kb >> 1) & 1) * 2;
+      const unsigned char* at = smem + s_off[0] + ((kb >> 2) & 3) * 1024 + ((kb >> 1) & 1) * 2 + nb * 128;
       return P::ring_scale(at, at + 4096);
     } else {
       return P::prep_scale(read_scale_byte(kb, nb), p);
@@ -579,11 +583,11 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   //   chunks  0..10  also issue one DMA instruction each of tile kb+2 into stage (kb+2) % 3, which
   //                  was last read in iteration kb-1 and is free since the barrier that ended it.
   // Tile kb+2 is not read before iteration kb+2: its loads have almost two iterations to land.
-  // A chunk with its side work cut into three pieces that sit between the chunk's four MFMAs, each piece
+  // A chunk with its side work cut into four pieces, one behind each of the chunk's four MFMAs, each piece
   // fenced by scheduling barriers: left to itself the scheduler issues one MFMA, then all of the side work
   // (about 50 cycles, longer than the 32 the MFMA runs), then the other three back to back, and the matrix
   // pipe idles once per chunk.
-  auto chunk4 = [&](int q, auto do_mfma_tag, auto&& side_a, auto&& side_b, auto&& side_c) {
+  auto chunk4 = [&](int q, auto do_mfma_tag, auto&& side_a, auto&& side_b, auto&& side_c, auto&& side_d) {
     constexpr bool do_mfma = decltype(do_mfma_tag)::value;
     if constexpr (do_mfma) acc[q][0] = P::mfma(af_c[q], bf_c[0], acc[q][0]);
     side_a();
@@ -595,6 +599,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     side_c();
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (do_mfma) acc[q][3] = P::mfma(af_c[q], bf_c[3], acc[q][3]);
+    side_d();
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -614,19 +619,18 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
         if constexpr (P::kScaleDma >= 2) sc_c[nb] = read_scale1(kb, nb);
         else sc_byte[nb] = read_scale_byte(kb, nb);
       };
-      auto finish_scales = [&]() {
-        if constexpr (P::kScaleDma < 2) {
-#pragma unroll
-          for (int nb = 0; nb < 4; ++nb) sc_c[nb] = P::prep_scale(sc_byte[nb], p);
-        }
+      auto finish_scale = [&](int nb) {
+        if constexpr (P::kScaleDma < 2) sc_c[nb] = P::prep_scale(sc_byte[nb], p);
       };
-      chunk4(0, DoMfma{}, [&] { fetch_b(0); fetch_b(1); }, [&] { dma(0); }, [&] { fetch_b(2); fetch_b(3); });
-      chunk4(1, DoMfma{}, [&] { af_n[0] = read_a1(base, 0, 0); }, [&] { dma(1); },
-             [&] { af_n[1] = read_a1(base, 0, 1); finish_scales(); });
-      chunk4(2, DoMfma{}, [&] { af_n[2] = read_a1(base, 0, 2); bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]); }, [&] { dma(2); },
-             [&] { af_n[3] = read_a1(base, 0, 3); bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]); });
+      auto nothing = [] {};
+      chunk4(0, DoMfma{}, [&] { fetch_b(0); fetch_b(1); }, [&] { dma(0); }, [&] { fetch_b(2); fetch_b(3); },
+             [&] { af_n[0] = read_a1(base, 0, 0); });
+      chunk4(1, DoMfma{}, [&] { af_n[1] = read_a1(base, 0, 1); finish_scale(0); }, [&] { dma(1); },
+             [&] { af_n[2] = read_a1(base, 0, 2); finish_scale(1); }, [&] { finish_scale(2); });
+      chunk4(2, DoMfma{}, [&] { af_n[3] = read_a1(base, 0, 3); finish_scale(3); }, [&] { dma(2); },
+             [&] { bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]); }, [&] { bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]); });
       chunk4(3, DoMfma{}, [&] { bf_n[2] = P::decode(bw_c[2], 0, sc_c[2]); }, [&] { dma(3); },
-             [&] { bf_n[3] = P::decode(bw_c[3], 0, sc_c[3]); });
+             [&] { bf_n[3] = P::decode(bw_c[3], 0, sc_c[3]); }, nothing);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         af_c[q] = af_n[q];
@@ -637,7 +641,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           chunk4(q, std::true_type{}, [&] { af_n[q] = read_a1(base, j + 1, q); }, [&] { dma(4 + j * 4 + q); },
-                 [&] { bf_n[q] = P::decode(bw_c[q], j + 1, sc_c[q]); });
+                 [&] { bf_n[q] = P::decode(bw_c[q], j + 1, sc_c[q]); }, nothing);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           af_c[q] = af_n[q];
