@@ -117,15 +117,22 @@ def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev):
     return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "graph": graphed}
 
 
-def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev):
-    """BitLinear forward on quantised operands: int8 x 2-bit (offset-binary ternary), fused acc/s_a/s_w epilogue."""
+def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True):
+    """BitLinear forward on quantised operands: int8 x 2-bit (offset-binary ternary), fused acc/s_a/s_w epilogue.
+
+    ``interleaved``: the packed words went through ``interleave_weight(qw, 2, "int8")`` on the host, once, as in
+    the reference's kernel benchmarks (examples/bitnet-1.58b/kernel_benchmark/
+    tilelang_bitnet_158_int8xint2_prefill.py:372-373, ..._decode.py:249-250); False: the plain packing."""
     d = workloads.bitnet(M, N, K, seed=0)
     nbytes = workloads.bitnet_bytes(M, N, K)
     nc = _copies(nbytes, hi=40)
     A = torch.from_numpy(d["A"]).to(dev)
-    Bs = [torch.from_numpy(d["B"]).to(dev).view(torch.int8).clone() for _ in range(nc)]
+    B0 = torch.from_numpy(d["B"]).view(torch.int8)
+    if interleaved:
+        B0 = tl.quantize.interleave_weight(B0, 2, "int8")
+    Bs = [B0.to(dev).clone() for _ in range(nc)]
     s_a = torch.from_numpy(np.asarray(d["s_a"], dtype=np.float32)).to(dev)
-    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset")
+    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset", interleaved=interleaved)
     out = [None]
 
     def mk(i):
@@ -290,6 +297,8 @@ def main():
         for m in (1, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, k if m == 1 else kg, 2, dev)
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        r = bench_bitnet(torch, tl, workloads, 2048, 8192, 8192, kg, 2, dev, interleaved=False)
+        shapes.append(_row("bitnet_w2a8 M=2048 N=8192 K=8192 (plain packing, not interleaved)", r, "mfma", MFMA_I8_PEAK))
         r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, max(5, k // 4), 2, dev)
         shapes.append(_row("w4a16_zeros_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
         r = bench_mxfp4_quant(torch, tl, 8192, 8192, k, 2, dev)
