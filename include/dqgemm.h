@@ -136,6 +136,17 @@ int call_bitnet_activation_quant(const void* X, void* Q, void* S, int M, int K, 
  * scale_bias as in call_dequant_gemm_bf16_mxfp4 (127: E8M0).  Requires K % 32 == 0. */
 int call_quantize_bf16_mxfp4(const void* W, void* B, void* Scale, int N, int K, int scale_bias, dq_stream_t stream);
 
+/* Block-scaled MXFP4 x MXFP4: C[M,N] bf16 = (e2m1(A[M,K/2]) * 2^(ScaleA[M,K/32] - 127)) .
+ * (e2m1(B[N,K/2]) * 2^(ScaleB[N,K/32] - 127))^T (+ Bias[M,N] bf16), fp32 accumulation, on the gfx950 scaled matrix
+ * instruction: codes and E8M0 scale bytes go to the instruction as they lie in memory (the layout
+ * call_quantize_bf16_mxfp4 writes with scale_bias = 127, for either operand).  The arithmetic is that of
+ * blockscaled_gemm_ref, examples/blockscaled_gemm_sm100/gemm_mxfp8_blockscaled_1d1d.py:575-620; it stands where the
+ * reference's block-scaled kernels stand on NVIDIA parts (`C = kernel(A, B, SFA, SFB)` of :17-170 and of
+ * examples/gemm_sm120/sm120_nvfp4_blockscaled_gemm.py:58-148), with plain row-major scales.  A scale byte of 255 is
+ * NaN.  Requires K % 128 == 0, K >= 256. */
+int call_gemm_mxfp4_mxfp4(const void* A, const void* B, const void* ScaleA, const void* ScaleB, const void* Bias,
+                          void* C, int M, int N, int K, dq_stream_t stream);
+
 /* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T.
  * is_signed 1: two's-complement nibbles (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:10-21,
  * `call(A, B, Ct)` :109-147); 0: unsigned nibbles (example_dequant_gemm_fine_grained.py int8 path).

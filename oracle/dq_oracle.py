@@ -491,6 +491,27 @@ def ref_mxfp4(A_bf16_bits, packed, scale, bias_bf16_bits=None, fmt="e2m1", scale
     return f32_to_bf16_bits(C)
 
 
+def ref_mxfp4_mxfp4(A_packed, scale_a, B_packed, scale_b, bias_bf16_bits=None, scale_size=32):
+    """Block-scaled MXFP4 x MXFP4 GEMM: both operands e2m1 codes with one E8M0 byte per 32 k,
+    ``C = (decode(A) * 2**(SA-127)) @ (decode(B) * 2**(SB-127)).T (+ Bias) -> bf16 bits``, the sum in float64
+    (every product is exact there) rounded once to fp32 and once to bf16.
+
+    Follows blockscaled_gemm_ref of examples/blockscaled_gemm_sm100/gemm_mxfp8_blockscaled_1d1d.py:575-620
+    (``2 ** (sf - 127)`` per scale block, fp32 result) with the 4-bit element format of
+    examples/dequantize_gemm/quantize/nvfp4.py:17-34.  A scale byte of 255 is NaN (E8M0).
+    """
+    sa = np.asarray(scale_a); sb = np.asarray(scale_b)
+    A = mxfp4_dequant(A_packed, np.where(sa == 255, 127, sa), "e2m1", scale_size, 127).astype(np.float64)
+    W = mxfp4_dequant(B_packed, np.where(sb == 255, 127, sb), "e2m1", scale_size, 127).astype(np.float64)
+    K = A.shape[1]
+    A[(sa == 255)[:, np.arange(K) // scale_size]] = np.nan
+    W[(sb == 255)[:, np.arange(K) // scale_size]] = np.nan
+    C = np.matmul(A, W.T).astype(np.float32)
+    if bias_bf16_bits is not None:
+        C = C + bf16_bits_to_f32(np.asarray(bias_bf16_bits, dtype=np.uint16))
+    return f32_to_bf16_bits(C)
+
+
 def ref_fp16xfp4(A, packed):
     """``Ct[N, M] = (A.float() @ simple_fp16(B).float().T -> fp16).T``.
 

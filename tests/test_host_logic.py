@@ -70,6 +70,14 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     assert "multiple of 32" in lib.get_last_error().decode()
     assert lib.call_quantize_bf16_mxfp4(a, a, a, 4, 64, 300, vp(0)) == -1
     assert "scale_bias" in lib.get_last_error().decode()
+    assert lib.call_gemm_mxfp4_mxfp4(a, a, vp(0), a, vp(0), a, 64, 64, 256, vp(0)) == -1
+    assert "ScaleA is expected to have non-NULL" in lib.get_last_error().decode()
+    assert lib.call_gemm_mxfp4_mxfp4(a, a, a, a, vp(0), a, 64, 64, 320, vp(0)) == -1
+    assert "multiple of 128" in lib.get_last_error().decode()
+    assert lib.call_gemm_mxfp4_mxfp4(a, a, a, a, vp(0), a, 64, 64, 128, vp(0)) == -1
+    assert "at least 256" in lib.get_last_error().decode()
+    assert lib.call_gemm_mxfp4_mxfp4(a, a, a, vp(a.value + 2), vp(0), a, 64, 64, 256, vp(0)) == -1
+    assert "4-byte aligned" in lib.get_last_error().decode()
 
 
 def test_bitlinear_weight_packing_matches_oracle():

@@ -267,6 +267,42 @@ def test_ref_mxfp4_exact_scaling_and_identity():
     np.testing.assert_array_equal(W0, orc.decode_fp4_e2m1(B) * 4)
 
 
+def test_ref_mxfp4_mxfp4_brute_force_and_scale_linearity():
+    """Block-scaled product against a plain triple loop over the e2m1 table (nvfp4.py:17-34) and 2**(sf - 127)
+    (gemm_mxfp8_blockscaled_1d1d.py:602-603); with every scale at 127 it is the plain matmul of the decoded
+    codes; adding one to a scale byte of A doubles that block's contribution and nothing else."""
+    table = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6, -0.0, -0.5, -1, -1.5, -2, -3, -4, -6], dtype=np.float64)
+    rng = np.random.default_rng(11)
+    M, N, K = 3, 5, 64
+    ca = rng.integers(0, 16, size=(M, K), dtype=np.uint8)
+    cb = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    sa = rng.integers(120, 131, size=(M, K // 32)).astype(np.uint8)
+    sb = rng.integers(120, 131, size=(N, K // 32)).astype(np.uint8)
+    A, B = orc.pack_fp4_e2m1_codes(ca), orc.pack_fp4_e2m1_codes(cb)
+    want = np.zeros((M, N), dtype=np.float64)
+    for m in range(M):
+        for n in range(N):
+            for k in range(K):
+                want[m, n] += table[ca[m, k]] * 2.0 ** (int(sa[m, k // 32]) - 127) * table[cb[n, k]] * 2.0 ** (int(sb[n, k // 32]) - 127)
+    got = orc.bf16_bits_to_f32(orc.ref_mxfp4_mxfp4(A, sa, B, sb))
+    np.testing.assert_array_equal(got, orc.round_to_bf16(want.astype(np.float32)))
+    ones_a, ones_b = np.full_like(sa, 127), np.full_like(sb, 127)
+    plain = table[ca] @ table[cb].T
+    np.testing.assert_array_equal(orc.bf16_bits_to_f32(orc.ref_mxfp4_mxfp4(A, ones_a, B, ones_b)),
+                                  orc.round_to_bf16(plain.astype(np.float32)))
+    # linearity in one scale block: block 1 of A row 0 one exponent up
+    sa2 = sa.copy(); sa2[0, 1] += 1
+    blk = np.zeros((M, N)); 
+    for n in range(N):
+        blk[0, n] = sum(table[ca[0, k]] * 2.0 ** (int(sa[0, 1]) - 127) * table[cb[n, k]] * 2.0 ** (int(sb[n, 1]) - 127) for k in range(32, 64))
+    got2 = orc.bf16_bits_to_f32(orc.ref_mxfp4_mxfp4(A, sa2, B, sb))
+    np.testing.assert_array_equal(got2, orc.round_to_bf16((want + blk).astype(np.float32)))
+    # a scale byte of 255 is NaN for the whole output row
+    sa3 = sa.copy(); sa3[1, 0] = 255
+    got3 = orc.bf16_bits_to_f32(orc.ref_mxfp4_mxfp4(A, sa3, B, sb))
+    assert np.isnan(got3[1]).all() and np.isfinite(got3[[0, 2]]).all()
+
+
 def test_activation_quant_matches_torch_ops():
     """utils_quant.py:156-163 executed with torch's own CPU ops (the reference's statements verbatim in
     tilelang_amd.bitlinear.activation_quant_reference): scales bit-identical, codes identical, ties included."""

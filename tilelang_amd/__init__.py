@@ -15,6 +15,7 @@ from .kernels import (  # noqa: F401
     dequantize_gemv,
     dequantize_w4,
     matmul_bf16_mxfp4,
+    matmul_mxfp4_mxfp4,
     matmul_fp16_fp4,
     matmul_int8xint4,
     matmul_nt_int4,

@@ -36,6 +36,8 @@ int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int out_kind, hipStream_t stream);
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
 int mxfp4_quant(const void* W, void* B, void* S, int N, int K, int scale_bias, hipStream_t stream);
+int mxfp4_mxfp4_gemm(const void* A, const void* SA, const void* B, const void* SB, const void* Bias, void* C, int M,
+                     int N, int K, hipStream_t stream);
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
             hipStream_t stream);
 
@@ -213,6 +215,21 @@ extern "C" int call_quantize_bf16_mxfp4(const void* W, void* B, void* Scale, int
   if (scale_bias < 0 || scale_bias > 254) DQ_FAIL("%s: scale_bias=%d must be in 0..254", fn, scale_bias);
   if (!aligned16(W) || ((uintptr_t)B & 3) != 0) DQ_FAIL("%s: W must be 16-byte and B 4-byte aligned", fn);
   return mxfp4_quant(W, B, Scale, N, K, scale_bias, (hipStream_t)stream);
+}
+
+extern "C" int call_gemm_mxfp4_mxfp4(const void* A, const void* B, const void* ScaleA, const void* ScaleB,
+                                     const void* Bias, void* C, int M, int N, int K, dq_stream_t stream) {
+  const char* fn = "call_gemm_mxfp4_mxfp4";
+  if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
+  if (!ScaleA) DQ_FAIL("%s: ScaleA is expected to have non-NULL data pointer", fn);
+  if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
+  if (!ScaleB) DQ_FAIL("%s: ScaleB is expected to have non-NULL data pointer", fn);
+  if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
+  if (M <= 0 || N <= 0 || K <= 0) DQ_FAIL("%s: M, N, K must be positive (got %d %d %d)", fn, M, N, K);
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C) || (Bias && !aligned16(Bias)))
+    DQ_FAIL("%s: A, B, Bias and C must be 16-byte aligned", fn);
+  if (((uintptr_t)ScaleA & 3) != 0 || ((uintptr_t)ScaleB & 3) != 0) DQ_FAIL("%s: ScaleA and ScaleB must be 4-byte aligned", fn);
+  return mxfp4_mxfp4_gemm(A, ScaleA, B, ScaleB, Bias, C, M, N, K, (hipStream_t)stream);
 }
 
 extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed,

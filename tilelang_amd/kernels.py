@@ -235,6 +235,37 @@ def matmul_bf16_mxfp4(
     return KernelAdapter("matmul_bf16_mxfp4", params, [-1], launch, _lib.last_error)
 
 
+def matmul_mxfp4_mxfp4(M: int, N: int, K: int, out_dtype="bfloat16", accum_dtype="float32", with_bias: bool = False) -> KernelAdapter:
+    """Block-scaled MXFP4 x MXFP4 GEMM on the gfx950 scaled matrix instruction:
+    ``C[M,N] = (e2m1(A[M,K/2]) * 2**(SFA[M,K/32] - 127)) @ (e2m1(B[N,K/2]) * 2**(SFB[N,K/32] - 127)).T (+ Bias)``.
+
+    ``C = kernel(A, B, SFA, SFB, Bias)``: the argument order of ``mxfp8_blockscaled_gemm`` of
+    examples/blockscaled_gemm_sm100/gemm_mxfp8_blockscaled_1d1d.py:17-60 (A, B ``[N, K]`` as with its
+    ``transpose_B=True``, then the two scale tensors), with plain row-major E8M0 bytes instead of its packed
+    group-major words, 32 k per scale, and the 4-bit element format of ``matmul_bf16_mxfp4``.  Both operands
+    are what ``quantize_bf16_mxfp4(rows, K, scale_bias=127)`` writes.  ``Bias`` is read only when ``with_bias``.
+    """
+    if _dtype(out_dtype) != torch.bfloat16 or _dtype(accum_dtype) != torch.float32:
+        raise ValueError("matmul_mxfp4_mxfp4: out_dtype must be bfloat16 and accum_dtype float32")
+    if K % 128 != 0 or K < 256:
+        raise ValueError(f"matmul_mxfp4_mxfp4: K={K} must be a multiple of 128 and at least 256")
+    params = [
+        KernelParam("A", torch.uint8, (M, K // 2), packed=True),
+        KernelParam("B", torch.uint8, (N, K // 2), packed=True),
+        KernelParam("SFA", torch.uint8, (M, K // 32), packed=True),
+        KernelParam("SFB", torch.uint8, (N, K // 32), packed=True),
+        KernelParam("Bias", torch.bfloat16, (M, N)),
+        KernelParam("C", torch.bfloat16, (M, N)),
+    ]
+
+    def launch(ptrs, stream):
+        lib = _lib.get_library()
+        bias = ptrs[4] if with_bias else None
+        return lib.call_gemm_mxfp4_mxfp4(ptrs[0], ptrs[1], ptrs[2], ptrs[3], bias, ptrs[5], M, N, K, stream)
+
+    return KernelAdapter("matmul_mxfp4_mxfp4", params, [-1], launch, _lib.last_error)
+
+
 def matmul_fp16_fp4(
     M: int,
     N: int,

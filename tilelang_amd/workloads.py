@@ -54,6 +54,17 @@ def mxfp4(M: int, N: int, K: int, seed: int = 0, scale_exp_range=(-8, 0), scale_
     return {"A": A, "B": B, "Scale": S}
 
 
+def mxfp4_mxfp4(M: int, N: int, K: int, seed: int = 0, scale_exp_range=(-8, 0), scale_size: int = 32):
+    """Both operands block-scaled fp4: e2m1 codes uniform over 16 values packed [M,K/2] and [N,K/2];
+    E8M0 scales uint8 [M,K/scale_size], [N,K/scale_size] = 127 + e, e uniform in ``scale_exp_range`` (inclusive)."""
+    rng = np.random.default_rng(seed)
+    A = pack_nibbles(rng.integers(0, 16, size=(M, K), dtype=np.uint8))
+    B = pack_nibbles(rng.integers(0, 16, size=(N, K), dtype=np.uint8))
+    SA = (rng.integers(scale_exp_range[0], scale_exp_range[1] + 1, size=(M, K // scale_size)) + 127).astype(np.uint8)
+    SB = (rng.integers(scale_exp_range[0], scale_exp_range[1] + 1, size=(N, K // scale_size)) + 127).astype(np.uint8)
+    return {"A": A, "B": B, "SFA": SA, "SFB": SB}
+
+
 def bitnet(M: int, N: int, K: int, seed: int = 0, zero_point: int = 2):
     """A int8 [M,K] uniform -127..127 with fp32 per-row scale s_a [M]; ternary W in {-1,0,1} (p = 1/3 each),
     stored as 2-bit codes ``w + zero_point`` four per byte [N,K/4]; fp32 per-tensor weight scale s_w."""
@@ -92,6 +103,10 @@ def w4a16_bytes(M: int, N: int, K: int, group: int = 128, zeros: bool = False) -
 
 def mxfp4_bytes(M: int, N: int, K: int, scale_size: int = 32) -> int:
     return 2 * M * K + N * K // 2 + N * (K // scale_size) + 2 * M * N
+
+
+def mxfp4_mxfp4_bytes(M: int, N: int, K: int, scale_size: int = 32) -> int:
+    return (M + N) * (K // 2 + K // scale_size) + 2 * M * N
 
 
 def bitnet_bytes(M: int, N: int, K: int) -> int:
