@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12        # B/s
 MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense
 MFMA_I8_PEAK = 5.0e15    # OP/s dense
+MFMA_FP4_PEAK = 10.1e15  # FLOP/s dense, block-scaled fp4
 # HBM bytes per launch of the headline GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
 # same counters read for a plain 128 MiB copy kernel (59240.5 x 2 KiB read + 56 KiB written)
 GEMV_HBM_TRAFFIC = 121381888
@@ -115,6 +116,28 @@ def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev):
 
     ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
     return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "graph": graphed}
+
+
+def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev):
+    """Both operands MXFP4 (e2m1 codes + one E8M0 byte per 32 k), block-scaled matrix instruction."""
+    d = workloads.mxfp4_mxfp4(M, N, K, seed=0)
+    nbytes = workloads.mxfp4_mxfp4_bytes(M, N, K)
+    nc = _copies(nbytes, hi=12)
+    A = torch.from_numpy(d["A"]).to(dev)
+    SA = torch.from_numpy(d["SFA"]).to(dev)
+    Bs = [torch.from_numpy(d["B"]).to(dev).clone() for _ in range(nc)]
+    SBs = [torch.from_numpy(d["SFB"]).to(dev).clone() for _ in range(nc)]
+    bias = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    kern = tl.matmul_mxfp4_mxfp4(M, N, K)
+    out = [None]
+
+    def mk(i):
+        def f():
+            out[0] = kern(A, Bs[i], SA, SBs[i], bias, skip_tensor_validation=True)
+        return f
+
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
 
 
 def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True):
@@ -309,6 +332,8 @@ def main():
         shapes.append(_row("w4a8_gemm M=4096 N=4096 K=4096 (Ct int32)", r, "mfma", MFMA_I8_PEAK))
         r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, True, kg, 2, dev)
         shapes.append(_row("int4xint4_gemm M=4096 N=4096 K=4096", r, "mfma", MFMA_I8_PEAK))
+        r = bench_mxfp4_blockscaled(torch, tl, workloads, 4096, 8192, 8192, kg, 2, dev)
+        shapes.append(_row("mxfp4_x_mxfp4_blockscaled_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_FP4_PEAK))
 
     cpu = None
     if not args.no_cpu:

@@ -83,6 +83,20 @@ def test_ragged_shapes(cuda, M, N, K):
     np.testing.assert_array_equal(got, ref)
 
 
+def test_scale_byte_255_is_nan(cuda):
+    """E8M0 has no infinity: byte 255 is NaN, and the instruction propagates it to every output of that row."""
+    M = N = K = 256
+    d = workloads.mxfp4_mxfp4(M, N, K, seed=6)
+    d["SFA"][3, 1] = 255
+    d["SFB"][200, 7] = 255
+    got = orc.bf16_bits_to_f32(_run(cuda, d, M, N, K))
+    ref = orc.bf16_bits_to_f32(orc.ref_mxfp4_mxfp4(d["A"], d["SFA"], d["B"], d["SFB"]))
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
+    assert np.isnan(got[3]).all() and np.isnan(got[:, 200]).all() and np.isnan(got).sum() == M + N - 1
+    ok = ~np.isnan(ref)
+    np.testing.assert_allclose(got[ok], ref[ok], rtol=RTOL, atol=ATOL)
+
+
 def test_bias(cuda):
     M, N, K = 300, 512, 512
     d = workloads.mxfp4_mxfp4(M, N, K, seed=3, scale_exp_range=(-4, 0))
