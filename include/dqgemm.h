@@ -97,6 +97,15 @@ int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale
 int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int N, int K, int transposed,
                                dq_stream_t stream);
 
+/* The same product with K cut into `split` slices: slice z is multiplied by its own workgroups into
+ * SplitC[z] (M x N, or N x M when transposed, fp16) and a second kernel adds the slices in fp16, slice 0 first.
+ * Replaces `call(A, B, Ct, stream)` of the kernel built from `main_split`,
+ * examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:136-175, whose SplitC is an internal buffer: here the
+ * caller passes it (split * M * N fp16; NULL allowed when split == 1), since no entry point allocates.
+ * Requires K % (64 * split) == 0, split in 1..64, M * N % 8 == 0 when split > 1. */
+int call_dequant_gemm_fp16_fp4_splitk(const void* A, const void* B, void* SplitC, void* C, int M, int N, int K,
+                                      int split, int transposed, dq_stream_t stream);
+
 /* fp16 x uint4 with the integer decoders: C[M,N] fp16 = A[M,K] fp16 . dequant(B, Scale, Zeros)^T with
  * the dequantised tile rounded to fp16 exactly as call_dequantize_w4 does.  Replaces `call(A, B, C)` of
  * examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:45-88 (mode DQ_W4_UNSIGNED) and serves

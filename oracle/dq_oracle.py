@@ -521,6 +521,24 @@ def ref_fp16xfp4(A, packed):
     return np.ascontiguousarray(C.T)
 
 
+def ref_fp16xfp4_splitk(A, packed, split: int):
+    """The split-K form of the fp16 x fp4 GEMM: each K slice gives an fp32 product rounded to fp16
+    (``T.copy(Ct_local, SplitC[bz, ...])``, SplitC in ``out_dtype``), and the slices are added in fp16, slice 0 first
+    (``acc`` of ``out_dtype``, ``acc += SplitC[k]``): examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:136-175.
+    Returns ``C[M,N]`` fp16 (the example stores its transpose).
+    """
+    A = np.asarray(A, dtype=np.float16)
+    W = decode_fp4_simple_f16(packed)
+    K = A.shape[1]
+    assert K % split == 0
+    kk = K // split
+    acc = None
+    for z in range(split):
+        part = _matmul_f32(A[:, z * kk:(z + 1) * kk], W[:, z * kk:(z + 1) * kk]).astype(np.float16)
+        acc = part if acc is None else (acc.astype(np.float32) + part.astype(np.float32)).astype(np.float16)
+    return acc
+
+
 def ref_w4a8(A_i8, packed):
     """``Ct[N, M] int32 = (A @ sext4(B).T).T``.  Follows example_dequant_gemm_w4a8.py:68-82."""
     C = _matmul_int(np.asarray(A_i8, dtype=np.int8), decode_i4_signed(packed)).astype(np.int32)

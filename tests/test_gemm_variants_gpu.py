@@ -88,6 +88,54 @@ def test_fp16_fp4(cuda, transposed, M, N, K):
     np.testing.assert_allclose(out.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("transposed", [True, False])
+@pytest.mark.parametrize("M,N,K,split", [(256, 256, 1024, 4), (128, 192, 2048, 8), (100, 72, 512, 2), (300, 520, 768, 3),
+                                         (2048, 2048, 1024, 4)])  # last: direct-to-LDS kernel (256 tiles of 256 x 256 x 256)
+def test_fp16_fp4_split_k(cuda, transposed, M, N, K, split):
+    """main_split of examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:136-175: fp16 partial results per K
+    slice, added in fp16 in slice order.  The same call twice gives the same bits (fixed order, no atomics)."""
+    print(f"split-K M={M} N={N} K={K} split={split} transposed={transposed}", flush=True)
+    rng = np.random.default_rng(2)
+    A = (rng.standard_normal((M, K), dtype=np.float32) * 0.5).astype(np.float16)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    kern = tl.matmul_fp16_fp4(M, N, K, split=split, transposed_output=transposed)
+    Ad, Bd = _dev(A, cuda), _dev(B, cuda)
+    out = kern(Ad, Bd)
+    again = kern(Ad, Bd)
+    torch.cuda.synchronize()
+    assert out.shape == ((N, M) if transposed else (M, N))
+    assert torch.equal(out, again)
+    ref = orc.ref_fp16xfp4_splitk(A, B, split).astype(np.float32)
+    # Every slice result and every running sum is rounded to fp16.  The kernel's fp32 slice sums differ from the
+    # oracle's in the last bits (summation order), so each of those 2 * split roundings may land one fp16 ulp away:
+    # where large slices cancel, that ulp (of the largest intermediate) exceeds 1e-2 of the small final value, so
+    # it is added to the bar, element by element.
+    W = orc.decode_fp4_simple_f16(B).astype(np.float32)
+    kk = K // split
+    parts = np.stack([A[:, z * kk:(z + 1) * kk].astype(np.float32) @ W[:, z * kk:(z + 1) * kk].T for z in range(split)])
+    big = np.maximum(np.abs(parts).max(axis=0), np.abs(np.cumsum(parts, axis=0)).max(axis=0))
+    ulp = np.exp2(np.floor(np.log2(np.maximum(big, 2.0 ** -14))) - 10)
+    bound = RTOL * np.abs(ref) + ATOL + 2 * split * ulp
+    got = out.float().cpu().numpy()
+    if transposed:
+        got = got.T
+    assert (np.abs(got - ref) <= bound).all(), float((np.abs(got - ref) - bound).max())
+    # and almost everywhere the plain 1e-2 bar holds
+    assert np.isclose(got, ref, rtol=RTOL, atol=ATOL).mean() > 0.9999
+
+
+def test_fp16_fp4_split_k_exact_when_slices_are_exact(cuda):
+    """Small integers: every slice product is an exact fp16 value, so the split result must equal the oracle's bit
+    for bit (a slice read from the wrong columns or written to the wrong partial buffer cannot hide)."""
+    M, N, K, split = 64, 128, 512, 4
+    rng = np.random.default_rng(3)
+    A = rng.integers(-2, 3, size=(M, K)).astype(np.float16)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8) & 0x33  # codes 0..3 of both signs... magnitudes 0.5 .. 1.5
+    out = tl.matmul_fp16_fp4(M, N, K, split=split, transposed_output=False)(_dev(A, cuda), _dev(B, cuda))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), orc.ref_fp16xfp4_splitk(A, B, split))
+
+
 def test_fp16_fp4_weights_exact(cuda):
     K, N = 128, 256
     B = np.tile(np.arange(256, dtype=np.uint8), (N, 1))[:, : K // 2].copy()

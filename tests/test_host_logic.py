@@ -70,6 +70,12 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     assert "multiple of 32" in lib.get_last_error().decode()
     assert lib.call_quantize_bf16_mxfp4(a, a, a, 4, 64, 300, vp(0)) == -1
     assert "scale_bias" in lib.get_last_error().decode()
+    assert lib.call_dequant_gemm_fp16_fp4_splitk(a, a, vp(0), a, 64, 64, 256, 2, 1, vp(0)) == -1
+    assert "SplitC is expected to have non-NULL" in lib.get_last_error().decode()
+    assert lib.call_dequant_gemm_fp16_fp4_splitk(a, a, a, a, 64, 64, 256, 3, 1, vp(0)) == -1
+    assert "64 * split" in lib.get_last_error().decode()
+    assert lib.call_dequant_gemm_fp16_fp4_splitk(a, a, a, a, 3, 5, 256, 2, 1, vp(0)) == -1
+    assert "multiple of 8" in lib.get_last_error().decode()
     assert lib.call_gemm_mxfp4_mxfp4(a, a, vp(0), a, vp(0), a, 64, 64, 256, vp(0)) == -1
     assert "ScaleA is expected to have non-NULL" in lib.get_last_error().decode()
     assert lib.call_gemm_mxfp4_mxfp4(a, a, a, a, vp(0), a, 64, 64, 320, vp(0)) == -1

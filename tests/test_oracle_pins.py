@@ -267,6 +267,32 @@ def test_ref_mxfp4_exact_scaling_and_identity():
     np.testing.assert_array_equal(W0, orc.decode_fp4_e2m1(B) * 4)
 
 
+def test_ref_fp16xfp4_splitk_closed_forms():
+    """One slice is the plain reference program; with small integers every partial result is exact in fp16 and the
+    split form equals the unsplit one; in general it is the slice products rounded to fp16 and added in fp16 in order
+    (example_dequant_gemm_fp4_hopper.py:136-175), restated here with explicit loops."""
+    rng = np.random.default_rng(8)
+    M, N, K = 5, 7, 256
+    A = (rng.standard_normal((M, K), dtype=np.float32)).astype(np.float16)
+    B = rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)
+    np.testing.assert_array_equal(orc.ref_fp16xfp4_splitk(A, B, 1), orc.ref_fp16xfp4(A, B).T)
+    Ai = rng.integers(-2, 3, size=(M, K)).astype(np.float16)
+    Bi = B & 0x33
+    np.testing.assert_array_equal(orc.ref_fp16xfp4_splitk(Ai, Bi, 4), orc.ref_fp16xfp4(Ai, Bi).T)
+    W = orc.decode_fp4_simple_f16(B).astype(np.float64)
+    want = np.zeros((M, N), dtype=np.float16)
+    for m in range(M):
+        for n in range(N):
+            acc = np.float16(0)
+            for z in range(4):
+                part = np.float16(np.float32(np.dot(A[m, z * 64:(z + 1) * 64].astype(np.float64), W[n, z * 64:(z + 1) * 64])))
+                acc = np.float16(np.float32(acc) + np.float32(part))
+            want[m, n] = acc
+    got = orc.ref_fp16xfp4_splitk(A, B, 4)
+    # the fp32 matmul of a slice may differ from the float64 dot in the last fp32 bit, i.e. by at most one fp16 ulp
+    np.testing.assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
 def test_ref_mxfp4_mxfp4_brute_force_and_scale_linearity():
     """Block-scaled product against a plain triple loop over the e2m1 table (nvfp4.py:17-34) and 2**(sf - 127)
     (gemm_mxfp8_blockscaled_1d1d.py:602-603); with every scale at 127 it is the plain matmul of the decoded

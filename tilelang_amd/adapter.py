@@ -51,11 +51,16 @@ class KernelAdapter:
         launch: Callable[[list, int], int],
         get_last_error: Callable[[], str],
         device_type: str = "cuda",
+        workspace_idx: Sequence[int] = (),
     ):
         self.name = name
         self.params = list(params)
         n = len(self.params)
         self.result_idx = [i if i >= 0 else n + i for i in result_idx]
+        # parameters the kernel uses as scratch (the reference's T.alloc_buffer globals): allocated here, once per
+        # device, passed to the library, never returned
+        self.workspace_idx = [i if i >= 0 else n + i for i in workspace_idx]
+        self._workspaces = {}
         self._launch = launch
         self._get_last_error = get_last_error
         self.device_type = device_type
@@ -102,7 +107,7 @@ class KernelAdapter:
                 raise ValueError(f"Expected parameter {p.name} to be a contiguous tensor")
 
     def __call__(self, *inputs, stream: int = -1, skip_tensor_validation: bool = False):
-        n_params, n_in, n_out = len(self.params), len(inputs), len(self.result_idx)
+        n_params, n_in, n_out = len(self.params) - len(self.workspace_idx), len(inputs), len(self.result_idx)
         if n_params != n_in + n_out:
             raise ValueError(
                 f"Expected {n_params} inputs, got {n_in + n_out} with {n_in} inputs and {n_out} outputs"
@@ -117,7 +122,14 @@ class KernelAdapter:
                 break
         tensors, it = [], iter(inputs)
         for i, p in enumerate(self.params):
-            if i in self.result_idx:
+            if i in self.workspace_idx:
+                if device is None:
+                    device = torch.device(self.device_type)
+                key = (i, str(device))
+                if key not in self._workspaces:
+                    self._workspaces[key] = torch.empty(*p.shape, dtype=p.dtype, device=device)
+                tensors.append(self._workspaces[key])
+            elif i in self.result_idx:
                 if device is None:
                     device = torch.device(self.device_type)
                 tensors.append(torch.empty(*p.shape, dtype=p.dtype, device=device))

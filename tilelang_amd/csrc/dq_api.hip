@@ -36,6 +36,8 @@ int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int out_kind, hipStream_t stream);
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
 int mxfp4_quant(const void* W, void* B, void* S, int N, int K, int scale_bias, hipStream_t stream);
+int fp16_fp4_gemm_splitk(const void* A, const void* B, void* parts, void* C, int M, int N, int K, int split,
+                         int transposed, hipStream_t stream);
 int mxfp4_mxfp4_gemm(const void* A, const void* SA, const void* B, const void* SB, const void* Bias, void* C, int M,
                      int N, int K, hipStream_t stream);
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
@@ -167,6 +169,19 @@ extern "C" int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C,
                                           dq_stream_t stream) {
   if (check_gemm_args("call_dequant_gemm_fp16_fp4", A, B, C, M, N, K, 64)) return -1;
   return fp16_fp4_gemm(A, B, C, M, N, K, transposed, (hipStream_t)stream);
+}
+
+extern "C" int call_dequant_gemm_fp16_fp4_splitk(const void* A, const void* B, void* SplitC, void* C, int M, int N, int K,
+                                                 int split, int transposed, dq_stream_t stream) {
+  const char* fn = "call_dequant_gemm_fp16_fp4_splitk";
+  if (check_gemm_args(fn, A, B, C, M, N, K, 64)) return -1;
+  if (split < 1 || split > 64) DQ_FAIL("%s: split=%d must be in 1..64", fn, split);
+  if (K % (64 * split) != 0) DQ_FAIL("%s: K=%d must be a multiple of 64 * split (split=%d)", fn, K, split);
+  if (split == 1) return fp16_fp4_gemm(A, B, C, M, N, K, transposed, (hipStream_t)stream);
+  if (!SplitC) DQ_FAIL("%s: SplitC is expected to have non-NULL data pointer", fn);
+  if (!aligned16(SplitC)) DQ_FAIL("%s: SplitC must be 16-byte aligned", fn);
+  if (((size_t)M * N) % 8 != 0) DQ_FAIL("%s: M * N must be a multiple of 8 when split > 1 (got %d x %d)", fn, M, N);
+  return fp16_fp4_gemm_splitk(A, B, SplitC, C, M, N, K, split, transposed, (hipStream_t)stream);
 }
 
 extern "C" int call_dequant_gemm_w4_fp16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,

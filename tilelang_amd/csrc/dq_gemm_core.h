@@ -59,7 +59,9 @@ struct Params {
   const void* Z;     // zeros / second scale (policy specific) or nullptr
   const void* Bias;  // optional
   void* C;
-  int M, N, K;
+  int M, N, K;       // K: contraction length of this launch (of one K slice when split > 1)
+  int ldk;           // k elements per stored row of A and B (= K unless the launch covers K slices)
+  int split;         // K slices, each its own set of workgroups and its own M x N output behind C
   int tiles_m, tiles_n;
   int p0, p1;        // policy specific integers (e.g. scale exponent offset, group shift)
   float f0;          // policy specific float (e.g. 1 / weight scale)
@@ -79,6 +81,21 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   const int in_band = pid - (pid / band) * band;
   tm = first_m + in_band % gm;
   tn = in_band / gm;
+}
+
+// Split-K (examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:136-167): workgroup ids beyond the first
+// tiles_m x tiles_n belong to further K slices.  Slice z reads columns [z K, (z + 1) K) of A and B and writes the
+// z-th M x N (or N x M) partial result behind C; a second kernel sums the partial results.  Plain (unpacked) A only.
+template <class P>
+__device__ __forceinline__ void take_k_slice(Params& p, int& bid) {
+  if (p.split > 1) {
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int z = bid / tiles;
+    bid -= z * tiles;
+    p.A = (const unsigned char*)p.A + (size_t)z * p.K * (kARowBytes / P::kKPerBlock);
+    p.B = (const unsigned char*)p.B + (size_t)z * p.K * P::kBRowBytes / P::kKPerBlock;
+    p.C = (unsigned char*)p.C + (size_t)z * p.M * p.N * sizeof(typename P::out_t);
+  }
 }
 
 // Epilogue shared by both kernel variants (a macro: it uses the kernel's locals).
@@ -180,7 +197,10 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 //       the lane's kBRowBytes/2 packed bytes as dwords
 //   Epilogue: out_t, kTransposed, finish(acc value, p, m, n) -> value stored
 template <class P, int kMBW, int kNBW>
-__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
+__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
+  Params p = p_in;
+  int bid = blockIdx.x;
+  take_k_slice<P>(p, bid);
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int BM = 64 * kMBW, BN = 64 * kNBW;  // 2 x 2 waves of kMBW x kNBW blocks of 32 x 32 (shadow the 256 x 256 default)
   constexpr int kAStage = BM * kARowBytes;
@@ -200,11 +220,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p) {
   const int M = p.M, N = p.N, K = p.K;
 
   int tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  tile_of_block(bid, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int KB = K / P::kKPerBlock;
-  const size_t a_row_bytes = P::kAPacked ? (size_t)(K >> 1) : (size_t)K * (kARowBytes / P::kKPerBlock == 2 ? 2 : 1);
-  const size_t b_row_bytes = (size_t)K * P::kBRowBytes / P::kKPerBlock;
+  const size_t a_row_bytes = P::kAPacked ? (size_t)(p.ldk >> 1) : (size_t)p.ldk * (kARowBytes / P::kKPerBlock == 2 ? 2 : 1);
+  const size_t b_row_bytes = (size_t)p.ldk * P::kBRowBytes / P::kKPerBlock;
 
   // ---- global -> register staging ---------------------------------------------------------
   // A piece q = tid + 256 i: row q / 8, 16-byte piece q % 8 of the 128-byte row.  A packed A row
@@ -425,7 +445,10 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
 // (four along the rows, which keeps the LDS traffic of the four-wave form) measured the same 410 us: a
 // second wave per SIMD does not buy MFMA issue slots here.
 template <class P, int kMBW, int kNBW>
-__global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p) {
+__global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p_in) {
+  Params p = p_in;
+  int bid = blockIdx.x;
+  take_k_slice<P>(p, bid);
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(P::kBRowBytes == 32 || P::kBRowBytes == 64, "direct-to-LDS variant: 32 or 64 packed bytes per weight row per tile");
   static_assert(kMBW == 2 || kMBW == 4, "wave tile of 64 or 128 rows");
@@ -456,7 +479,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   const int M = p.M, N = p.N, K = p.K;
 
   int tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  tile_of_block(bid, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int KB = K / P::kKPerBlock;
   const unsigned lds0 = (unsigned)(size_t)smem;  // LDS byte address of the dynamic segment
@@ -467,14 +490,14 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   for (int i = 0; i < kAOps; ++i) {
     const int c = (wave * kAOps + i) * 64 + lane;  // A chunk: row c / 8, physical piece c % 8
     const int row = c >> 3, pp = c & 7;
-    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(K * (kARowBytes / P::kKPerBlock)) + (unsigned)((pp ^ a_swz(row)) << 4);
+    a_voff[i] = (unsigned)min(m0 + row, M - 1) * (unsigned)(p.ldk * (kARowBytes / P::kKPerBlock)) + (unsigned)((pp ^ a_swz(row)) << 4);
   }
 #pragma unroll
   for (int i = 0; i < kBOps; ++i) {
     const int c = (wave * kBOps + i) * 64 + lane;  // B chunk: row c / pieces per row, physical piece c % pieces per row
     const int row = c / kBPiecesPerRow, pp = c % kBPiecesPerRow;
     // LDS position (piece + rotation) % pieces holds source piece `piece`
-    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(K * P::kBRowBytes / P::kKPerBlock) +
+    b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(p.ldk * P::kBRowBytes / P::kKPerBlock) +
                 (unsigned)(((pp - (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);
   }
   const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(P::kScaleDma == 1 ? (K >> 5) : (K >> 6));  // waves 4..7 repeat 0..3
@@ -761,7 +784,7 @@ int launch(Params p, hipStream_t stream) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
     lds_limit_raised = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(kThreads), kLds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(kThreads), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }
@@ -771,7 +794,7 @@ int launch(Params p, hipStream_t stream) {
 // narrower M tile would).
 template <class P>
 int launch_auto(const Params& p, hipStream_t stream) {
-  auto tiles = [&](int bm, int bn) { return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+  auto tiles = [&](int bm, int bn) { return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.split; };
   if (tiles(256, 256) >= 192) return launch<P, 4, 4>(p, stream);
   if (tiles(128, 128) >= 192) return launch<P, 2, 2>(p, stream);
   return launch<P, 2, 1>(p, stream);
@@ -780,10 +803,10 @@ int launch_auto(const Params& p, hipStream_t stream) {
 template <class P>
 bool dma_eligible(const Params& p) {
   // the direct-to-LDS kernel has one tile shape (256 x 256): small problems go to the tile-size choice above
-  const long tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  const long tiles = (long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN) * p.split;
   // 32-bit lane offsets: A rows are 128 bytes per K block, packed B rows kBRowBytes
-  const size_t a_bytes = (size_t)p.M * (p.K / P::kKPerBlock) * kARowBytes;
-  const size_t b_bytes = (size_t)p.N * (p.K / P::kKPerBlock) * P::kBRowBytes;
+  const size_t a_bytes = (size_t)p.M * (p.ldk / P::kKPerBlock) * kARowBytes;
+  const size_t b_bytes = (size_t)p.N * (p.ldk / P::kKPerBlock) * P::kBRowBytes;
   return P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
 }
 
@@ -801,7 +824,7 @@ int launch_dma_tile(Params p, hipStream_t stream) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
     lds_limit_raised = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(64 * kWaves), kLds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(64 * kWaves), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }
@@ -816,6 +839,8 @@ inline Params make_params(const void* A, const void* B, const void* S, const voi
   Params p{};
   p.A = A; p.B = B; p.S = S; p.Z = Z; p.Bias = Bias; p.C = C;
   p.M = M; p.N = N; p.K = K;
+  p.ldk = K;
+  p.split = 1;
   p.tiles_m = (M + BM - 1) / BM;
   p.tiles_n = (N + BN - 1) / BN;
   return p;

@@ -211,6 +211,51 @@ int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, in
   return gemm::launch_auto<Fp16Fp4Policy<false>>(p, stream);
 }
 
+namespace {
+
+// Second kernel of the split-K form (examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:168-175): the
+// partial results are fp16 and are added in fp16, slice 0 first, as the reference's `acc += SplitC[k]` does.
+__global__ __launch_bounds__(256) void splitk_sum_f16_kernel(const half_t* __restrict__ parts, half_t* __restrict__ out,
+                                                             size_t count, int split) {
+  const size_t i8 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i8 + 8 <= count) {
+    half8_t acc = *reinterpret_cast<const half8_t*>(parts + i8);
+    for (int z = 1; z < split; ++z) acc = acc + *reinterpret_cast<const half8_t*>(parts + (size_t)z * count + i8);
+    *reinterpret_cast<half8_t*>(out + i8) = acc;
+  } else {
+    for (size_t i = i8; i < count; ++i) {
+      half_t acc = parts[i];
+      for (int z = 1; z < split; ++z) acc = acc + parts[(size_t)z * count + i];
+      out[i] = acc;
+    }
+  }
+}
+
+}  // namespace
+
+// K cut into `split` slices, each multiplied by its own workgroups into parts[z] (M x N, or N x M when transposed,
+// fp16), then summed.  Worth it when M x N alone gives the 256 CUs too few tiles.
+int fp16_fp4_gemm_splitk(const void* A, const void* B, void* parts, void* C, int M, int N, int K, int split,
+                         int transposed, hipStream_t stream) {
+  Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, parts, M, N, K / split);
+  p.ldk = K;
+  p.split = split;
+  int rc;
+  if (gemm::dma_eligible<Fp16Fp4Policy<true>>(p)) {
+    rc = transposed ? gemm::launch_dma<Fp16Fp4Policy<true>>(p, stream) : gemm::launch_dma<Fp16Fp4Policy<false>>(p, stream);
+  } else {
+    rc = transposed ? gemm::launch_auto<Fp16Fp4Policy<true>>(p, stream) : gemm::launch_auto<Fp16Fp4Policy<false>>(p, stream);
+  }
+  if (rc) return rc;
+  const size_t count = (size_t)M * N;
+  // the partial results are 16-byte aligned slice by slice only when M x N is a multiple of 8
+  if (count % 8 != 0) DQ_FAIL("fp16 x fp4 split-K gemm: M * N = %zu must be a multiple of 8", count);
+  const unsigned blocks = (unsigned)((count + 2047) / 2048);
+  hipLaunchKernelGGL(splitk_sum_f16_kernel, dim3(blocks), dim3(256), 0, stream, (const half_t*)parts, (half_t*)C, count, split);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                 int mode, int layout, hipStream_t stream) {
   Params p = gemm::make_params(A, B, S, Z, nullptr, C, M, N, K);

@@ -285,9 +285,10 @@ def matmul_fp16_fp4(
     """fp16 x "simple" fp4 GEMM: ``Ct[N,M] = (A[M,K] @ fp4_to_f16(B[N,K/2]).T).T``.
 
     Same arguments as ``matmul`` of examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:110-125;
-    ``Ct = kernel(A, B)`` (``out_idx=[2]``).  ``split`` is accepted: the K reduction stays inside one
-    workgroup in fp32 (the example's split variant sums ``split`` partial tiles in a second kernel), so the
-    result does not depend on it.  ``transposed_output=False`` gives ``C[M,N]``.
+    ``Ct = kernel(A, B)`` (``out_idx=[2]``).  ``split > 1`` is the example's ``main_split`` (:136-175): K is cut
+    into ``split`` slices that run on their own workgroups, their fp16 partial results are added in fp16 by a
+    second kernel; the partial-result buffer (the example's ``SplitC``) is allocated here once per device.
+    ``transposed_output=False`` gives ``C[M,N]``.
     """
     if num_bits != 4:
         raise ValueError("matmul_fp16_fp4: num_bits must be 4")
@@ -295,17 +296,29 @@ def matmul_fp16_fp4(
         raise ValueError("matmul_fp16_fp4: in_dtype and out_dtype must be float16")
     if K % 64 != 0:
         raise ValueError(f"matmul_fp16_fp4: K={K} must be a multiple of 64")
+    if split < 1 or K % (64 * split) != 0:
+        raise ValueError(f"matmul_fp16_fp4: K={K} must be a multiple of 64 * split (split={split})")
     out_shape = (N, M) if transposed_output else (M, N)
     params = [
         KernelParam("A", torch.float16, (M, K)),
         KernelParam("B", torch.uint8, (N, K // 2), packed=True),
         KernelParam("Ct" if transposed_output else "C", torch.float16, out_shape),
     ]
+    if split == 1:
+        def launch(ptrs, stream):
+            return _lib.get_library().call_dequant_gemm_fp16_fp4(ptrs[0], ptrs[1], ptrs[2], M, N, K, int(transposed_output), stream)
 
-    def launch(ptrs, stream):
-        return _lib.get_library().call_dequant_gemm_fp16_fp4(ptrs[0], ptrs[1], ptrs[2], M, N, K, int(transposed_output), stream)
+        return KernelAdapter("matmul_fp16_fp4", params, [2], launch, _lib.last_error)
 
-    return KernelAdapter("matmul_fp16_fp4", params, [2], launch, _lib.last_error)
+    if (M * N) % 8 != 0:
+        raise ValueError(f"matmul_fp16_fp4: M * N must be a multiple of 8 when split > 1 (got {M} x {N})")
+    params.append(KernelParam("SplitC", torch.float16, (split,) + out_shape))
+
+    def launch_split(ptrs, stream):
+        return _lib.get_library().call_dequant_gemm_fp16_fp4_splitk(ptrs[0], ptrs[1], ptrs[3], ptrs[2], M, N, K, split,
+                                                                    int(transposed_output), stream)
+
+    return KernelAdapter("matmul_fp16_fp4_splitk", params, [2], launch_split, _lib.last_error, workspace_idx=[3])
 
 
 def matmul_w4_fine_grained(
