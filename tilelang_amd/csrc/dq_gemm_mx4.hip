@@ -116,8 +116,8 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
   auto read_frag = [&](const unsigned char* base, int off, int blk) -> uint4_t {
     return *reinterpret_cast<const uint4_t*>(base + off + blk * (32 * kRowBytes));
   };
-  auto read_scale = [&](int stage, int off, int blk) -> int {
-    return (int)(*reinterpret_cast<const uint32_t*>(smem + off + stage * kScaleStage + blk * 128) >> shift);
+  auto read_scale = [&](int stage, int off, int blk) -> uint32_t {  // the row's four scale bytes, unshifted
+    return *reinterpret_cast<const uint32_t*>(smem + off + stage * kScaleStage + blk * 128);
   };
 
   float16_t acc[kMBW][kNBW];
@@ -138,6 +138,7 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
 
   uint4_t af_c[4], bf_c[4], af_n[4], bf_n[4];
   int sa_c[4], sb_c[4], sa_n[4], sb_n[4];
+  uint32_t sa_r[4], sb_r[4];
 
   // A chunk = one A fragment against the four B fragments; the side work sits behind the MFMAs it hides under.
   auto chunk = [&](int q, int step, auto do_mfma_tag, auto&& side_a, auto&& side_b, auto&& side_c, auto&& side_d) {
@@ -158,8 +159,10 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
 
   // One iteration = tile kb out of `stage`:
   //   chunks 0..3  MFMAs of step 1 of tile kb-1 (operands and scales already in registers); side work: read the
-  //                scale dwords and the step-0 fragments of tile kb
-  //   chunks 4..7  MFMAs of step 0 of tile kb; side work: read its step-1 fragments
+  //                scale dwords and the step-0 fragments of tile kb, B side first (every chunk needs all four B
+  //                fragments, chunk q only A fragment q), shift the scale dwords two chunks after their reads
+  //   chunks 4..7  MFMAs of step 0 of tile kb; side work: read its step-1 fragments, B side first again
+  // so that no LDS read is consumed sooner than four MFMAs after it was issued,
   // and the ten DMA instructions of tile kb+2 go into stage (kb+2) % 3, free since the barrier that ended
   // iteration kb-1.
   auto iteration = [&](int kb, int stage, auto first_tag, auto next2_tag) {
@@ -171,13 +174,22 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
     auto dma = [&](int op) {
       if (has_next2) issue_op(op, kb + 2, stage2);
     };
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      chunk(q, 1, DoMfma{},
-            [&] { sa_n[q] = read_scale(stage, sa_off, q); af_n[q] = read_frag(base, a_off[0], q); },
-            [&] { dma(q); },
-            [&] { sb_n[q] = read_scale(stage, sb_off, q); bf_n[q] = read_frag(base, b_off[0], q); },
-            [&] { if (q < 2) dma(8 + q); });
+    chunk(0, 1, DoMfma{},
+          [&] { for (int i = 0; i < 4; ++i) sb_r[i] = read_scale(stage, sb_off, i); },
+          [&] { dma(0); },
+          [&] { bf_n[0] = read_frag(base, b_off[0], 0); bf_n[1] = read_frag(base, b_off[0], 1); },
+          [&] { bf_n[2] = read_frag(base, b_off[0], 2); bf_n[3] = read_frag(base, b_off[0], 3); });
+    chunk(1, 1, DoMfma{},
+          [&] { for (int i = 0; i < 4; ++i) sa_r[i] = read_scale(stage, sa_off, i); },
+          [&] { dma(1); },
+          [&] { af_n[0] = read_frag(base, a_off[0], 0); af_n[1] = read_frag(base, a_off[0], 1); },
+          [&] { af_n[2] = read_frag(base, a_off[0], 2); af_n[3] = read_frag(base, a_off[0], 3); });
+    chunk(2, 1, DoMfma{},
+          [&] { for (int i = 0; i < 4; ++i) sb_n[i] = (int)(sb_r[i] >> shift); },
+          [&] { dma(2); },
+          [&] { for (int i = 0; i < 4; ++i) sa_n[i] = (int)(sa_r[i] >> shift); },
+          [&] { dma(8); });
+    chunk(3, 1, DoMfma{}, [] {}, [&] { dma(3); }, [] {}, [&] { dma(9); });
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       af_c[q] = af_n[q]; bf_c[q] = bf_n[q];
@@ -186,9 +198,9 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       chunk(q, 0, std::true_type{},
-            [&] { af_n[q] = read_frag(base, a_off[1], q); },
+            [&] { if (q < 2) bf_n[2 * q] = read_frag(base, b_off[1], 2 * q); else af_n[2 * (q - 2)] = read_frag(base, a_off[1], 2 * (q - 2)); },
             [&] { dma(4 + q); },
-            [&] { bf_n[q] = read_frag(base, b_off[1], q); },
+            [&] { if (q < 2) bf_n[2 * q + 1] = read_frag(base, b_off[1], 2 * q + 1); else af_n[2 * (q - 2) + 1] = read_frag(base, a_off[1], 2 * (q - 2) + 1); },
             [] {});
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
