@@ -10,7 +10,8 @@
 //
 //   * block tile 256 x 256 x 128 k, 4 waves as 2 x 2, 128 x 128 per wave = 4 x 4 accumulators of 32 x 32;
 //   * both operand tiles are 256 rows x 64 bytes; they and the scale dwords (4 bytes = the 4 scale blocks of a
-//     row and tile) travel global -> LDS by global_load_lds into a ring of three stages, two tiles ahead;
+//     row and tile) travel global -> LDS by global_load_lds into a ring of four stages, two or three tiles ahead,
+//     the loads of two consecutive tiles issued as pairs (together they cover whole 128-byte lines);
 //   * lane (r, g) of a wave feeds row r with the 32 codes (16 bytes) of scale block 2 s + g in MFMA step s; the
 //     16-byte pieces of a row are XOR-swizzled with (row >> 2) & 3 (on the source side of the DMA) so that a
 //     ds_read_b128 phase of 16 lanes covers all banks;
@@ -33,9 +34,10 @@ constexpr int kKTile = 128;                // k per tile
 constexpr int kRowBytes = kKTile / 2;      // 64 packed bytes per row and tile
 constexpr int kOpStage = 256 * kRowBytes;  // 16 KiB per operand
 constexpr int kStage = 2 * kOpStage;       // A then B
-constexpr int kRing = 3 * kStage;          // scale ring behind the three stages
+constexpr int kStages = 4;                 // tile t lives in stage t % 4
+constexpr int kRing = kStages * kStage;    // scale ring behind the operand stages
 constexpr int kScaleStage = 2 * 1024;      // 256 dwords of A scales, 256 of B scales
-constexpr int kPipe = kRing + 3 * kScaleStage;
+constexpr int kPipe = kRing + kStages * kScaleStage;
 constexpr int kTileOps = 10;               // DMA instructions per thread and tile: 4 A, 4 B, 2 scale
 
 template <bool HAS_BIAS>
@@ -128,12 +130,13 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
 
-  // ---- prologue: tiles 0 and 1 in flight, tile 0 landed
+  // ---- prologue: tiles 0 and 1 (KB >= 2 is checked by the launcher), instruction by instruction as a pair
 #pragma unroll
-  for (int op = 0; op < kTileOps; ++op) issue_op(op, 0, 0);
-#pragma unroll
-  for (int op = 0; op < kTileOps; ++op) issue_op(op, 1, 1);  // KB >= 2 is checked by the launcher
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kTileOps) : "memory");
+  for (int op = 0; op < kTileOps; ++op) {
+    issue_op(op, 0, 0);
+    issue_op(op, 1, 1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   uint4_t af_c[4], bf_c[4], af_n[4], bf_n[4];
@@ -163,33 +166,37 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
   //                fragments, chunk q only A fragment q), shift the scale dwords two chunks after their reads
   //   chunks 4..7  MFMAs of step 0 of tile kb; side work: read its step-1 fragments, B side first again
   // so that no LDS read is consumed sooner than four MFMAs after it was issued,
-  // and the ten DMA instructions of tile kb+2 go into stage (kb+2) % 3, free since the barrier that ended
-  // iteration kb-1.
-  auto iteration = [&](int kb, int stage, auto first_tag, auto next2_tag) {
+  // A tile's rows are 64 bytes, half a cache line, and the other half is the next tile's: the loads of tiles
+  // t and t + 1 (t even) are therefore issued as pairs, the same instruction for t and then for t + 1, so that
+  // the second finds its lines already on their way.  An even iteration kb issues the pairs of tiles kb + 2
+  // and kb + 3 (kIssue of them: 2, or 1 / 0 at the end of K) into stages (kb + 2) % 4 and (kb + 3) % 4, both
+  // free since the barrier that ended iteration kb - 1; an odd iteration issues nothing.
+  auto iteration = [&](int kb, auto first_tag, auto issue_tag) {
     constexpr bool first = decltype(first_tag)::value;
-    constexpr bool has_next2 = decltype(next2_tag)::value;
+    constexpr int kIssue = decltype(issue_tag)::value;
     using DoMfma = std::integral_constant<bool, !first>;
-    const int stage2 = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3
+    const int stage = kb & 3;
     const unsigned char* base = smem + stage * kStage;
     auto dma = [&](int op) {
-      if (has_next2) issue_op(op, kb + 2, stage2);
+      if constexpr (kIssue >= 1) issue_op(op, kb + 2, (kb + 2) & 3);
+      if constexpr (kIssue >= 2) issue_op(op, kb + 3, (kb + 3) & 3);
     };
     chunk(0, 1, DoMfma{},
           [&] { for (int i = 0; i < 4; ++i) sb_r[i] = read_scale(stage, sb_off, i); },
           [&] { dma(0); },
           [&] { bf_n[0] = read_frag(base, b_off[0], 0); bf_n[1] = read_frag(base, b_off[0], 1); },
-          [&] { bf_n[2] = read_frag(base, b_off[0], 2); bf_n[3] = read_frag(base, b_off[0], 3); });
+          [&] { bf_n[2] = read_frag(base, b_off[0], 2); bf_n[3] = read_frag(base, b_off[0], 3); dma(1); });
     chunk(1, 1, DoMfma{},
           [&] { for (int i = 0; i < 4; ++i) sa_r[i] = read_scale(stage, sa_off, i); },
-          [&] { dma(1); },
+          [&] { dma(2); },
           [&] { af_n[0] = read_frag(base, a_off[0], 0); af_n[1] = read_frag(base, a_off[0], 1); },
-          [&] { af_n[2] = read_frag(base, a_off[0], 2); af_n[3] = read_frag(base, a_off[0], 3); });
+          [&] { af_n[2] = read_frag(base, a_off[0], 2); af_n[3] = read_frag(base, a_off[0], 3); dma(3); });
     chunk(2, 1, DoMfma{},
           [&] { for (int i = 0; i < 4; ++i) sb_n[i] = (int)(sb_r[i] >> shift); },
-          [&] { dma(2); },
+          [&] { dma(4); },
           [&] { for (int i = 0; i < 4; ++i) sa_n[i] = (int)(sa_r[i] >> shift); },
-          [&] { dma(8); });
-    chunk(3, 1, DoMfma{}, [] {}, [&] { dma(3); }, [] {}, [&] { dma(9); });
+          [&] { dma(5); });
+    chunk(3, 1, DoMfma{}, [] {}, [&] { dma(6); }, [] {}, [&] { dma(7); });
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       af_c[q] = af_n[q]; bf_c[q] = bf_n[q];
@@ -199,34 +206,37 @@ __global__ __launch_bounds__(256, 1) void mx4_gemm_kernel(Params p) {
     for (int q = 0; q < 4; ++q)
       chunk(q, 0, std::true_type{},
             [&] { if (q < 2) bf_n[2 * q] = read_frag(base, b_off[1], 2 * q); else af_n[2 * (q - 2)] = read_frag(base, a_off[1], 2 * (q - 2)); },
-            [&] { dma(4 + q); },
+            [&] { if (q < 2) dma(8 + q); },
             [&] { if (q < 2) bf_n[2 * q + 1] = read_frag(base, b_off[1], 2 * q + 1); else af_n[2 * (q - 2) + 1] = read_frag(base, a_off[1], 2 * (q - 2) + 1); },
             [] {});
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       af_c[q] = af_n[q]; bf_c[q] = bf_n[q];
     }
-    if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kTileOps) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // tile kb + 1 must have landed.  After an even iteration it was issued two iterations ago and only this
+    // iteration's own loads may still be in flight; after an odd one it was issued in the iteration before, paired
+    // with tile kb + 2, so everything has to land.
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kIssue * kTileOps) : "memory");
     __syncthreads();
   };
 
-  int stage = 0;
-  int kb = 0;
-  if (KB > 2) {
-    iteration(0, 0, std::true_type{}, std::true_type{});
-    stage = 1;
-    for (kb = 1; kb + 2 < KB; ++kb) {
-      iteration(kb, stage, std::false_type{}, std::true_type{});
-      stage = stage == 2 ? 0 : stage + 1;
-    }
-    iteration(kb, stage, std::false_type{}, std::false_type{});
-    stage = stage == 2 ? 0 : stage + 1;
-    iteration(kb + 1, stage, std::false_type{}, std::false_type{});
-  } else {  // KB == 2
-    iteration(0, 0, std::true_type{}, std::false_type{});
-    iteration(1, 1, std::false_type{}, std::false_type{});
+  using Zero = std::integral_constant<int, 0>;
+  using One = std::integral_constant<int, 1>;
+  using Two = std::integral_constant<int, 2>;
+  if (KB > 3) iteration(0, std::true_type{}, Two{});
+  else if (KB == 3) iteration(0, std::true_type{}, One{});
+  else iteration(0, std::true_type{}, Zero{});
+  iteration(1, std::false_type{}, Zero{});
+  int kb = 2;
+  for (; kb + 3 < KB; kb += 2) {  // steady state: an issuing iteration and a quiet one
+    iteration(kb, std::false_type{}, Two{});
+    iteration(kb + 1, std::false_type{}, Zero{});
   }
+  if (kb + 2 < KB) {  // three tiles left: the last one still has to be fetched
+    iteration(kb, std::false_type{}, One{});
+    ++kb;
+  }
+  for (; kb < KB; ++kb) iteration(kb, std::false_type{}, Zero{});
   // step 1 of the last tile
 #pragma unroll
   for (int q = 0; q < 4; ++q)
