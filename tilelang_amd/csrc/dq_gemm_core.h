@@ -464,10 +464,19 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   constexpr int kBStage = BN * P::kBRowBytes;  // 8 KiB
   constexpr int kStage = kAStage + kBStage;    // 40 or 24 KiB
   constexpr int kStages = 3;
+  // A packed-B row of one tile is 32 bytes, a quarter of a cache line, and the next tile's row is the next 32:
+  // the B loads of tiles t and t + 1 (t even) are issued as pairs, the same instruction for t and then for t + 1,
+  // which halves the lines the B stream asks the L2 for.  Tile t + 1 then lands three iterations before it is
+  // read, which takes a fourth B slot, so B gets a ring of its own behind the three A stages: kPairB.  Policies
+  // with 64-byte rows keep A and B side by side in three stages (a fourth 16 KiB slot would not fit).
+  constexpr bool kPairB = P::kBRowBytes == 32 && kMBW == 4 && kNBW == 4;
+  constexpr int kBRing = kPairB ? kStages * kAStage : kAStage;       // where B of slot 0 starts
+  constexpr int kBSlot = kPairB ? kBStage : kStage;                  // distance between B slots
+  constexpr int kAStride = kPairB ? kAStage : kStage;                // distance between A stages
   // Scales that travel by DMA (P::kScaleDma): 1 = one byte per 32 k (a dword per row covers a pair of tiles),
   // 2 = one fp16 per 128 k (a dword per row covers four tiles), 3 = the same for scales and for zeros.
   // Ring: 4 slots x 1 KiB (256 rows x one dword), a second ring for the zeros.
-  constexpr int kRing = kStages * kStage;
+  constexpr int kRing = kPairB ? kStages * kAStage + 4 * kBStage : kStages * kStage;
   constexpr int kSOps = P::kScaleDma == 0 ? 0 : (P::kScaleDma == 3 ? 2 : 1);  // scale DMA instructions per wave per tile
   constexpr int kBWords = P::kBRowBytes / 8;   // dwords per lane and 32-row block: 4 or 8
 
@@ -507,7 +516,8 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   // chunks, then the packed-B chunks.
   constexpr int kTileOps = kSOps + kAOps + kBOps;
   auto issue_op = [&](int op, int kb, int stage) {
-    const unsigned sbase = lds0 + stage * kStage;
+    const unsigned sbase = lds0 + stage * kAStride;
+    const unsigned bbase = lds0 + kBRing + (kPairB ? (kb & 3) : stage) * kBSlot;
     if (op < kSOps) {
       if constexpr (P::kScaleDma == 1) {
         const int pair = kb >> 1;
@@ -522,7 +532,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
       dma16(sbase + (wave * kAOps + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
     } else {
       const int i = op - kSOps - kAOps;
-      dma16(sbase + kAStage + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * P::kBRowBytes);
+      dma16(bbase + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * P::kBRowBytes);
     }
   };
   constexpr int kWaitOps = kTileOps;  // outstanding DMA instructions of one tile
@@ -541,7 +551,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
 #pragma unroll
     for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
       const int piece = g * (kBPiecesPerRow / 2) + h;
-      b_off[nb][h] = kAStage + row * P::kBRowBytes + (((piece + (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);
+      b_off[nb][h] = row * P::kBRowBytes + (((piece + (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);  // in its B slot
     }
     s_off[nb] = kRing + row * 4 + (P::kScaleDma == 1 ? g : 0);
   }
@@ -584,11 +594,24 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
   // ---- prologue: tiles 0 and 1 (and their scales) in flight; only tile 0 has to have landed -------
+  if constexpr (kPairB) {  // scales, A of tile 0, the B pairs of tiles 0 and 1, then A of tile 1
 #pragma unroll
-  for (int op = 0; op < kTileOps; ++op) issue_op(op, 0, 0);
+    for (int op = 0; op < kSOps + kAOps; ++op) issue_op(op, 0, 0);
 #pragma unroll
-  for (int op = 0; op < kTileOps; ++op) issue_op(op, 1, 1);  // KB >= 2 because K % 128 == 0
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
+    for (int i = 0; i < kBOps; ++i) {
+      issue_op(kSOps + kAOps + i, 0, 0);
+      issue_op(kSOps + kAOps + i, 1, 1);
+    }
+#pragma unroll
+    for (int op = kSOps; op < kSOps + kAOps; ++op) issue_op(op, 1, 1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAOps) : "memory");
+  } else {
+#pragma unroll
+    for (int op = 0; op < kTileOps; ++op) issue_op(op, 0, 0);
+#pragma unroll
+    for (int op = 0; op < kTileOps; ++op) issue_op(op, 1, 1);  // KB >= 2 because K % 128 == 0
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
+  }
   __syncthreads();
 
   typename P::Scale sc_c[kNBW];
@@ -626,19 +649,34 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  auto iteration = [&](int kb, int stage, auto first_tag, auto next2_tag) {
+  // odd_tag: tile kb is odd (only looked at with kPairB, where even iterations issue the B pairs of tiles
+  // kb + 2 and kb + 3, the scales and A of tile kb + 2, and odd iterations A of tile kb + 2 only)
+  auto iteration = [&](int kb, int stage, auto first_tag, auto next2_tag, auto odd_tag) {
     constexpr bool first = decltype(first_tag)::value;
     constexpr bool has_next2 = decltype(next2_tag)::value;
+    constexpr bool odd = decltype(odd_tag)::value;
     const int stage2 = stage == 0 ? 2 : stage - 1;  // (stage + 2) % 3
-    const unsigned char* base = smem + stage * kStage;
+    const unsigned char* base = smem + stage * kAStride;
+    const unsigned char* bbase = smem + kBRing + (kPairB ? (kb & 3) : stage) * kBSlot;
+    constexpr int kIterOps = !kPairB ? kTileOps : (odd ? kAOps : kSOps + kAOps + 2 * kBOps);  // issued per iteration
     if constexpr (kMBW == 4 && kNBW == 4) {
       using DoMfma = std::integral_constant<bool, !first>;
       auto dma = [&](int chunk) {
-        if (has_next2 && chunk < kTileOps) issue_op(chunk, kb + 2, stage2);
+        if constexpr (!kPairB) {
+          if (has_next2 && chunk < kTileOps) issue_op(chunk, kb + 2, stage2);
+        } else if constexpr (odd) {
+          if (has_next2 && chunk < kAOps) issue_op(kSOps + chunk, kb + 2, stage2);
+        } else {
+          if (has_next2 && chunk < kSOps + kAOps) issue_op(chunk, kb + 2, stage2);
+          else if (has_next2 && chunk < kIterOps) {
+            const int j = chunk - kSOps - kAOps;  // B instruction j / 2 of tile kb + 2 + j % 2
+            issue_op(kSOps + kAOps + (j >> 1), kb + 2 + (j & 1), stage2);
+          }
+        }
       };
       int sc_byte[4];  // scale bytes are read in chunk 0 and turned into multipliers in chunk 1
       auto fetch_b = [&](int nb) {
-        read_b1(base, nb, bw_c[nb]);
+        read_b1(bbase, nb, bw_c[nb]);
         if constexpr (P::kScaleDma >= 2) sc_c[nb] = read_scale1(kb, nb);
         else sc_byte[nb] = read_scale_byte(kb, nb);
       };
@@ -678,7 +716,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
         if (q == 0) {
 #pragma unroll
           for (int nb = 0; nb < kNBW; ++nb) {
-            read_b1(base, nb, bw_c[nb]);
+            read_b1(bbase, nb, bw_c[nb]);
             sc_c[nb] = read_scale1(kb, nb);
           }
         } else if (q == 1) {
@@ -697,7 +735,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
         if (q == 0) {
 #pragma unroll
           for (int nb = 0; nb < kNBW; ++nb) {
-            read_b1(base, nb, bw_c[nb]);
+            read_b1(bbase, nb, bw_c[nb]);
             sc_c[nb] = read_scale1(kb, nb);
           }
           af_n[0] = read_a1(base, 0, 0);
@@ -740,26 +778,34 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     }
     // tile kb+1 must have landed before the next iteration reads it; tile kb+2 (issued during this
     // iteration) may still be in flight
-    if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
+    if (has_next2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kIterOps) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
 
+  // KB is even (K % (2 kKPerBlock) == 0): tiles come in (even, odd) pairs
+  using T = std::true_type;
+  using F = std::false_type;
   int stage = 0;
   int kb = 0;
+  auto next_stage = [&] { stage = stage == 2 ? 0 : stage + 1; };
   if (KB > 2) {
-    iteration(0, 0, std::true_type{}, std::true_type{});
+    iteration(0, 0, T{}, T{}, F{});
     stage = 1;
-    for (kb = 1; kb + 2 < KB; ++kb) {
-      iteration(kb, stage, std::false_type{}, std::true_type{});
-      stage = stage == 2 ? 0 : stage + 1;
+    for (kb = 1; kb + 3 < KB; kb += 2) {
+      iteration(kb, stage, F{}, T{}, T{});
+      next_stage();
+      iteration(kb + 1, stage, F{}, T{}, F{});
+      next_stage();
     }
-    iteration(kb, stage, std::false_type{}, std::false_type{});
-    stage = stage == 2 ? 0 : stage + 1;
-    iteration(kb + 1, stage, std::false_type{}, std::false_type{});
+    iteration(kb, stage, F{}, T{}, T{});  // kb = KB - 3
+    next_stage();
+    iteration(kb + 1, stage, F{}, F{}, F{});
+    next_stage();
+    iteration(kb + 2, stage, F{}, F{}, T{});
   } else {  // KB == 2
-    iteration(0, 0, std::true_type{}, std::false_type{});
-    iteration(1, 1, std::false_type{}, std::false_type{});
+    iteration(0, 0, T{}, F{}, F{});
+    iteration(1, 1, F{}, F{}, T{});
   }
   // step 3 of the last tile
 #pragma unroll
@@ -813,7 +859,8 @@ bool dma_eligible(const Params& p) {
 template <class P, int kMBW, int kNBW>
 int launch_dma_tile(Params p, hipStream_t stream) {
   constexpr int kWaves = 16 / kNBW;
-  constexpr int kPipe = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + 8 * 1024;
+  constexpr bool kPairB = P::kBRowBytes == 32 && kMBW == 4 && kNBW == 4;  // as in the kernel: a fourth B slot
+  constexpr int kPipe = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + (kPairB ? BN * P::kBRowBytes : 0) + 8 * 1024;
   constexpr int kSlabs = kWaves * 32 * (32 * kNBW + 4) * 4;  // epilogue staging
   constexpr int kLds = kPipe > kSlabs ? kPipe : kSlabs;
   p.tiles_m = (p.M + 64 * kMBW - 1) / (64 * kMBW);
