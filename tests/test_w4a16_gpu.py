@@ -151,11 +151,15 @@ def test_kernel_variants(cuda, variant):
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
 def test_streaming_small_batch_kernel(cuda, variant, mode):
     """The direct-to-LDS kernel: ragged M and N, a single K step, fewer steps than ring stages, many steps,
-    both layouts."""
-    _run_gemv(cuda, 37, 16 * 13 + 3, 256 * 3, 128, mode, variant=variant)
-    _run_gemv(cuda, 64, 130, 256, 128, mode, variant=variant)
+    both layouts.  With scales the kernel wants K >= 1024 (a row's scales travel 16 bytes = 1024 k at a time):
+    K = 1024 is one scale group, K = 1280 and 2304 end in a partial group whose load is shifted to the row's last
+    16 bytes."""
+    scaled = mode in ("scale", "uscale", "original", "rescale")
+    _run_gemv(cuda, 37, 16 * 13 + 3, 256 * 5 if scaled else 256 * 3, 128, mode, variant=variant)
+    _run_gemv(cuda, 64, 130, 1024 if scaled else 256, 128, mode, variant=variant)
     _run_gemv(cuda, 5, 64, 256 * 9, 128, mode, variant=variant, interleaved=True)
     _run_gemv(cuda, 16, 256, 4096, 128, mode, variant=variant)
+    _run_gemv(cuda, 20, 300, 11008, 128, mode, variant=variant)
 
 
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])

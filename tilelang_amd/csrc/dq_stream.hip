@@ -7,10 +7,10 @@
 // likes, at no register cost:
 //
 //   * a workgroup owns 64 or 128 weight rows (4 waves x 1 or 2 blocks of 16 rows) and walks K in
-//     steps of 256; the packed weights (rows x 128 B), the activations (16 MB rows x 512 B) and the
-//     group scales / zeros of a step (4 B per row) travel global -> LDS with
-//     global_load_lds_dwordx4 / _dword into a ring of NST stages, NST - 1 steps ahead of the
-//     arithmetic; every weight DMA instruction reads 8 rows x 128 contiguous bytes;
+//     steps of 256; the packed weights (rows x 128 B) and the activations (16 MB rows x 512 B) travel
+//     global -> LDS with global_load_lds_dwordx4 into a ring of NST stages, NST - 1 steps ahead of the
+//     arithmetic; every weight DMA instruction reads 8 rows x 128 contiguous bytes; the group scales / zeros
+//     travel the same way, 16 bytes (four steps) per row at a time, into a small ring of their own;
 //   * a lane's bytes land at LDS base + lane * 16 whatever its source address, so the
 //     bank-conflict swizzles are applied by permuting the SOURCE addresses: 16-byte piece p of
 //     weight row n sits at position p ^ ((n >> 1) & 7), piece p of activation row m at
@@ -50,8 +50,10 @@ struct StreamGeom {
   static constexpr int kRowsPerWg = 64 * RBW;
   static constexpr int kWBytes = kRowsPerWg * (kStepK / 2);  // packed weights of a stage
   static constexpr int kABytes = MB * 16 * (kStepK * 2);     // activations of a stage
-  static constexpr int kSOff = kWBytes + kABytes;            // scales: 128 rows x 4 B, then zeros
-  static constexpr int kStage = kSOff + 1024;
+  static constexpr int kStage = kWBytes + kABytes;
+  // Scales and zeros live in a ring of their own behind the stages: one slot = the 16 bytes (8 groups of 128 k =
+  // 4 steps) of 128 rows of scales, then the same of zeros.
+  static constexpr int kScaleSlot = 2 * 128 * 16;
 };
 
 // KSPLIT = 2: eight waves, two per SIMD; waves 4..7 own the same rows as waves 0..3 and take the second
@@ -74,7 +76,11 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   constexpr bool kScale = MODE >= W4_SCALE;
   constexpr bool kZeros = MODE >= W4_ZEROS_ORIGINAL;
   constexpr int kAOps = 2 * MB / KSPLIT;                // activation DMA instructions per wave per stage
-  constexpr int kOps = kWOps + kAOps + (kScale ? 1 : 0);    // DMA instructions per wave per stage
+  // DMA instructions per wave per stage; every fourth stage carries one more, the scales / zeros of four steps,
+  // which the waits below do not count (they then wait for one instruction more than they must)
+  constexpr int kOps = kWOps + kAOps;
+  constexpr int kScaleSlots = NST <= 4 ? 2 : 3;         // groups of four steps alive at a time, plus the one landing
+  constexpr int kRing = NST * G::kStage;
   constexpr int kWaitOps = (NST - 2) * kOps;            // younger instructions when the next stage must have landed
   static_assert((NST - 1) * kOps <= 63, "vmcnt is a 6-bit counter");
   constexpr int kU = 2 / KSPLIT;                        // 128-k halves of a step per wave
@@ -111,8 +117,18 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   // waves 0, 1: scales of rows 0..63 / 64..127 from the workgroup's first row; waves 2, 3: zeros (or,
   // without zeros, the scales again); waves 4..7 repeat 0..3.  Every wave issues the same number of
   // DMA instructions; with 64 rows per workgroup the second half is simply not read.
-  const unsigned s_voff = (unsigned)min(n0 + (wn & 1) * 64 + lane, N - 1) * (unsigned)(groups_per_row * 2);
+  // A dword of scales per row and step would ask for 64 different cache lines per instruction, and for the same
+  // line 32 steps in a row: instead a row's 16 bytes (four steps) travel at once, every fourth step.
+  const int row_bytes = groups_per_row * 2;  // >= 16: K >= 1024 is checked by the launcher
+  const unsigned s_voff = (unsigned)min(n0 + (wn & 1) * 64 + lane, N - 1) * (unsigned)row_bytes;
   const unsigned char* s_src = reinterpret_cast<const unsigned char*>((wn >= 2 && kZeros) ? Z : S);
+  // the last group of a row whose K is not a multiple of 1024 reads the row's last 16 bytes instead of running
+  // past its end, and the readers shift their offset by the same amount
+  auto scale_src_off = [&](int g4) { return min(g4 * 16, row_bytes - 16); };
+  auto scale_base = [&](int step) -> const unsigned char* {
+    const int g4 = step >> 2;
+    return smem + kRing + (g4 % kScaleSlots) * G::kScaleSlot + (step * 4 - scale_src_off(g4));
+  };
 
   auto issue_stage = [&](int step, int slot) {
     const unsigned sb = lds0 + slot * G::kStage;
@@ -122,7 +138,13 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
     for (int i = 0; i < kAOps; ++i)
       dma16(sb + kWBytes + (wave * kAOps + i) * 1024, a_voff[i],
             reinterpret_cast<const unsigned char*>(A) + (size_t)step * (kStepK * 2));
-    if constexpr (kScale) dma4(sb + G::kSOff + wn * 256, s_voff, s_src + (size_t)step * 4);
+    if constexpr (kScale) {
+      if ((step & 3) == 0) {
+        const int g4 = step >> 2;
+        dma16(lds0 + kRing + (g4 % kScaleSlots) * G::kScaleSlot + (wn >= 2 ? 2048 : 0) + (wn & 1) * 1024, s_voff,
+              s_src + scale_src_off(g4));
+      }
+    }
   };
 
   // ---- fragment read offsets inside a stage (ui: the wave's ui-th half of a step) -----------------
@@ -133,7 +155,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
 #pragma unroll
     for (int rb = 0; rb < RBW; ++rb) {
       const int row = wn * (16 * RBW) + rb * 16 + r;
-      sc_off[rb][ui] = G::kSOff + row * 4 + u * 2;
+      sc_off[rb][ui] = row * 16 + u * 2;  // from scale_base(step)
       w_off[rb][ui] = row * 128 + ((((u << 2) + g) ^ ((row >> 1) & 7)) << 4);
     }
 #pragma unroll
@@ -160,14 +182,15 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   uint4_t w_c[kU][RBW], w_n[kU][RBW], yraw[2][MB];
   half_t sc_c[kU][RBW], zp_c[kU][RBW], sc_n[kU][RBW], zp_n[kU][RBW];
   half8_t x_m[RBW], y_m[MB], x_d[RBW], y_d[MB];
+  const unsigned char* sc_nxt = scale_base(0);  // scales of the step whose weights read_weights fetches next
   auto read_weights = [&](const unsigned char* sb) {
 #pragma unroll
     for (int ui = 0; ui < kU; ++ui)
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb) {
         w_n[ui][rb] = *reinterpret_cast<const uint4_t*>(sb + w_off[rb][ui]);
-        sc_n[ui][rb] = kScale ? *reinterpret_cast<const half_t*>(sb + sc_off[rb][ui]) : (half_t)1.f;
-        zp_n[ui][rb] = kZeros ? *reinterpret_cast<const half_t*>(sb + sc_off[rb][ui] + 512) : (half_t)0.f;
+        sc_n[ui][rb] = kScale ? *reinterpret_cast<const half_t*>(sc_nxt + sc_off[rb][ui]) : (half_t)1.f;
+        zp_n[ui][rb] = kZeros ? *reinterpret_cast<const half_t*>(sc_nxt + sc_off[rb][ui] + 2048) : (half_t)0.f;
       }
   };
   auto decode = [&](uint32_t w, half_t sc, half_t zp) -> half8_t {
@@ -266,6 +289,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (step + NST < KS) issue_stage(step + NST, slot);
+    sc_nxt = scale_base(step + 1);
     run_slots(SlotNext{}, SlotEnd{}, sb_cur, smem + slot1 * G::kStage, std::true_type{}, std::true_type{});
     next_weights_become_current();
     slot = slot1;
@@ -318,7 +342,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
 template <int MB, int RBW, int NST, int KSPLIT>
 int launch_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int mode,
                   int layout, hipStream_t stream) {
-  constexpr int kLds = NST * StreamGeom<MB, RBW>::kStage;
+  constexpr int kLds = NST * StreamGeom<MB, RBW>::kStage + (NST <= 4 ? 2 : 3) * StreamGeom<MB, RBW>::kScaleSlot;
   constexpr int kRowsPerWg = StreamGeom<MB, RBW>::kRowsPerWg;
   static_assert(kLds <= 160 * 1024, "LDS budget");
   const dim3 grid((N + kRowsPerWg - 1) / kRowsPerWg, (M + 16 * MB - 1) / (16 * MB));
@@ -368,7 +392,7 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, hipStream_t stream) {
   if (K % kStepK != 0 || N < 1 || M < 1) return 1;
-  if (mode >= W4_SCALE && group != 128) return 1;
+  if (mode >= W4_SCALE && (group != 128 || K < 1024)) return 1;  // scales travel 16 bytes (1024 k) per row at a time
   if ((size_t)N * K / 2 >= (1ull << 32) || (size_t)M * K * 2 >= (1ull << 32)) return 1;
   switch (config) {
     case 0: return launch_stream<1, 2, 6, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
