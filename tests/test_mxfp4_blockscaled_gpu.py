@@ -97,6 +97,25 @@ def test_scale_byte_255_is_nan(cuda):
     np.testing.assert_allclose(got[ok], ref[ok], rtol=RTOL, atol=ATOL)
 
 
+def test_full_size_properties(cuda):
+    """M=4096, N=K=8192 (512 tiles, 64 K tiles each): a band of rows against the oracle, and two properties that
+    hold bit for bit at any size: raising every scale byte of A by one doubles every output (a power of two moves no
+    rounding), and swapping the operands transposes the result (the fp32 sums run in the same k order)."""
+    M, N, K = 4096, 8192, 8192
+    d = workloads.mxfp4_mxfp4(M, N, K, seed=9, scale_exp_range=(-6, 0))
+    got = _run(cuda, d, M, N, K)
+    rows = np.r_[0:8, 2040:2056, 4088:4096]
+    ref = orc.ref_mxfp4_mxfp4(d["A"][rows], d["SFA"][rows], d["B"], d["SFB"])
+    np.testing.assert_allclose(orc.bf16_bits_to_f32(got[rows]), orc.bf16_bits_to_f32(ref), rtol=RTOL, atol=ATOL)
+    d2 = dict(d)
+    d2["SFA"] = (d["SFA"] + 1).astype(np.uint8)
+    doubled = _run(cuda, d2, M, N, K)
+    np.testing.assert_array_equal(orc.bf16_bits_to_f32(doubled), 2.0 * orc.bf16_bits_to_f32(got))
+    d3 = {"A": d["B"][:M], "SFA": d["SFB"][:M], "B": d["A"], "SFB": d["SFA"]}  # (B[:M] . A^T) = (A . B[:M]^T)^T
+    swapped = _run(cuda, d3, M, M, K)
+    np.testing.assert_array_equal(swapped, got[:, :M].T)
+
+
 def test_bias(cuda):
     M, N, K = 300, 512, 512
     d = workloads.mxfp4_mxfp4(M, N, K, seed=3, scale_exp_range=(-4, 0))
