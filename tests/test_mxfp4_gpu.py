@@ -66,6 +66,9 @@ def test_many_tiles(cuda, fmt, with_bias):
     _check(cuda, 3581, 3589, 128, fmt, scale_bias=127, with_bias=with_bias)
     _check(cuda, 3584, 3584, 320, fmt, scale_bias=0, with_bias=with_bias, exp_range=(0, 4))
     _check(cuda, 1500, 2000, 192, fmt, scale_bias=127, with_bias=with_bias)
+    if not with_bias:  # direct-to-LDS kernel with 4, 6 and 10 K tiles: prologue pair, steady pairs, tail
+        for K in (256, 384, 640):
+            _check(cuda, 3584, 3600, K, fmt, scale_bias=127)
 
 
 @pytest.mark.parametrize("fmt", ["e2m1", "simple"])
