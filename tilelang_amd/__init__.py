@@ -24,6 +24,7 @@ from .kernels import (  # noqa: F401
     quantize_bf16_mxfp4,
 )
 from .bitlinear import BitLinear  # noqa: F401
+from .w4linear import W4A16Linear  # noqa: F401
 from .profiler import Profiler, TensorSupplyType, do_bench  # noqa: F401
 
 __version__ = "0.1.0"
