@@ -245,6 +245,53 @@ def fast_decode_i2_to_i8(words: np.ndarray, signed: bool) -> np.ndarray:
     return out
 
 
+def fast_decode_i2_to_f16(halfwords: np.ndarray, signed: bool, scale=None) -> np.ndarray:
+    """Semantics of decode_i2{u,s}_to_f16[_scale] on one 16-bit word -> 8 fp16, in output order.
+
+    Follows examples/dequantize_gemm/quantize/lop3.py:424-463 (and :465-500 with a scale):
+    ``i2s = (x & 0x00ff) | ((x & 0xff00) << 8)``; for i in 0..3
+    ``h[i] = ((i2s >> 2i) & 0x00030003) | 0x64006400`` as two fp16 (1024 + c), minus 1026 (signed) or
+    1024 (unsigned), then ``fma.rn.f16x2(h, s, 0)`` when scaled.  Output element ``2i`` is the low half.
+    """
+    x = np.asarray(halfwords).astype(np.uint32) & np.uint32(0xFFFF)
+    i2s = (x & np.uint32(0x00FF)) | ((x & np.uint32(0xFF00)) << np.uint32(8))
+    out = np.empty(x.shape + (8,), dtype=np.float16)
+    med = np.float16(1026.0 if signed else 1024.0)
+    for i in range(4):
+        h = ((i2s >> np.uint32(2 * i)) & np.uint32(0x00030003)) | np.uint32(0x64006400)
+        lo = (h & 0xFFFF).astype(np.uint16).view(np.float16)
+        hi = (h >> 16).astype(np.uint16).view(np.float16)
+        out[..., 2 * i] = lo - med
+        out[..., 2 * i + 1] = hi - med
+    if scale is not None:
+        out = ((out.astype(np.float32) * np.float32(np.float16(scale))) + np.float32(0.0)).astype(np.float16)
+    return out
+
+
+def dequant_u2(packed: np.ndarray, convention: str = "twos", scale: np.ndarray | None = None, group: int = -1) -> np.ndarray:
+    """2-bit codes -> fp16 weights ``w = decode_i2(c)`` (exact), times ``s[n, k // group]`` with one fp16 rounding.
+
+    ``"twos"`` is the GEMV example's slow path (``_tir_packed_int_to_int_convert`` with ``num_bits = 2``,
+    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124 and quantize/quantization.py:333-343);
+    ``"unsigned"`` / ``"offset"`` are decode_i2u_to_f16 / decode_i2s_to_f16 (quantize/lop3.py:424-463), the scaled
+    forms lop3.py:465-500: exact ``c - zp`` then ``fma.rn.f16x2(x, s, 0)``.
+    PARITY UNPINNED by reference tests for the scaled form (no caller in the reference).
+    """
+    w = decode_i2(packed, convention).astype(np.float32)
+    if scale is None:
+        return w.astype(np.float16)
+    K = w.shape[-1]
+    s = _expand_groups(np.asarray(scale, dtype=np.float16), K, K if group == -1 else group).astype(np.float32)
+    return ((w * s) + np.float32(0.0)).astype(np.float16)
+
+
+def ref_w2a16(A, packed, convention: str = "twos", scale=None, group: int = -1) -> np.ndarray:
+    """``ref_program`` of the 2-bit GEMV: dequantise, fp32 matmul, fp16 out (the pattern of
+    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:207-217 with the 2-bit unpack)."""
+    W = dequant_u2(packed, convention, scale, group)
+    return _matmul_f32(np.asarray(A, dtype=np.float16), W).astype(np.float16)
+
+
 # --------------------------------------------------------------------------------------
 # W4A16 dequantised weight tiles (fp16), exact rounding order of the device snippets
 # --------------------------------------------------------------------------------------

@@ -478,3 +478,55 @@ def test_gen_quant4_quantize_properties():
     ref, s, q = orc.gen_quant4_quantize(w, -1)
     assert s.shape == (1, N) and np.abs(q).max() == 8
 
+
+
+def test_i2_to_f16_fast_decode_all_halfwords_and_interleave():
+    """decode_i2{u,s}_to_f16 (lop3.py:424-463) over all 65536 inputs against the closed form (outputs 2i, 2i+1 are
+    the fields at bit 2i of byte 0 and byte 1), and fast_decode(interleave_weight(p, 2, "float16")) == plain decode."""
+    x = np.arange(65536, dtype=np.uint32)
+    for signed in (False, True):
+        out = orc.fast_decode_i2_to_f16(x, signed)
+        for i in range(4):
+            lo = ((x >> (2 * i)) & 3).astype(np.float32) - (2 if signed else 0)
+            hi = ((x >> (8 + 2 * i)) & 3).astype(np.float32) - (2 if signed else 0)
+            np.testing.assert_array_equal(out[:, 2 * i].astype(np.float32), lo)
+            np.testing.assert_array_equal(out[:, 2 * i + 1].astype(np.float32), hi)
+    rng = np.random.default_rng(5)
+    raw = rng.integers(0, 256, size=(8, 64), dtype=np.uint8)
+    il = orc.interleave_weight(raw.view(np.int8), 2, "float16")
+    fast = orc.fast_decode_i2_to_f16(il.view(np.uint16).reshape(8, -1), signed=True).reshape(8, -1)
+    np.testing.assert_array_equal(fast.astype(np.float32), orc.decode_i2(raw, "offset").astype(np.float32))
+    fastu = orc.fast_decode_i2_to_f16(il.view(np.uint16).reshape(8, -1), signed=False).reshape(8, -1)
+    np.testing.assert_array_equal(fastu, orc.dequant_u2(raw, "unsigned"))
+    # the scaled decoder rounds the product once; with signed codes the product is exact
+    s = np.float16(0.0137)
+    sc = orc.fast_decode_i2_to_f16(x[:4096], True, scale=s).astype(np.float64)
+    exact = orc.fast_decode_i2_to_f16(x[:4096], True).astype(np.float64) * float(s)
+    np.testing.assert_array_equal(sc, exact)
+    scu = orc.fast_decode_i2_to_f16(x[:4096], False, scale=s)
+    np.testing.assert_array_equal(scu, (orc.fast_decode_i2_to_f16(x[:4096], False).astype(np.float64) * float(s)).astype(np.float16))
+
+
+def test_ref_w2a16_brute_force():
+    """dequant_u2 / ref_w2a16 against a triple loop in float64 on a tiny case, every convention, with and without scales."""
+    rng = np.random.default_rng(11)
+    M, N, K, g = 2, 5, 128, 64
+    A = rng.standard_normal((M, K)).astype(np.float16)
+    packed = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    S = rng.uniform(0.01, 0.05, size=(N, K // g)).astype(np.float16)
+    table = {"unsigned": [0, 1, 2, 3], "offset": [-2, -1, 0, 1], "twos": [0, 1, -2, -1]}
+    for conv, tab in table.items():
+        for scale in (None, S):
+            want = np.zeros((M, N))
+            for n in range(N):
+                for k in range(K):
+                    c = (int(packed[n, k // 4]) >> (2 * (k % 4))) & 3
+                    w = float(tab[c])
+                    if scale is not None:
+                        w = float(np.float16(w * float(scale[n, k // g])))
+                    for m in range(M):
+                        want[m, n] += float(A[m, k]) * w
+            got = orc.ref_w2a16(A, packed, conv, scale, g if scale is not None else -1).astype(np.float64)
+            np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)
+    # sign extension of the reference's own known answer (test_tilelang_u32_signed_decode.py:26-30): codes 2,3,0,1 -> -2..1
+    np.testing.assert_array_equal(orc.dequant_u2(np.array([[0b01001110]], dtype=np.uint8), "twos")[0], np.array([-2, -1, 0, 1], dtype=np.float16))

@@ -1,0 +1,85 @@
+"""GPU parity of the 2-bit case of dequantize_gemv (fp16 activations, B[N, K/4]) through the C-ABI."""
+
+import numpy as np
+import pytest
+import torch
+
+import tilelang_amd as tl
+from oracle import dq_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(M, N, K, seed, integer_a=False):
+    rng = np.random.default_rng(seed)
+    if integer_a:
+        A = rng.integers(-4, 5, size=(M, K)).astype(np.float16)
+    else:
+        A = rng.standard_normal((M, K)).astype(np.float16)
+    packed = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    return A, packed
+
+
+def _run(kernel, cuda, A, B, S=None):
+    M, N = A.shape[0], B.shape[0]
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    args = [torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda)]
+    if S is not None:
+        args.append(torch.from_numpy(S).to(cuda))
+    kernel(*args, C)
+    torch.cuda.synchronize()
+    return C.cpu().numpy()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (1, 256, 128), (2, 1000, 4096), (1, 4096, 11008), (3, 517, 8192),
+                                   (1, 64, 16384), (1, 96, 20480), (5, 33, 2048), (1, 7, 32768)])
+@pytest.mark.parametrize("fast,fmt", [(False, "uint"), (True, "uint"), (True, "int")])
+def test_w2a16_exact_integers(cuda, M, N, K, fast, fmt):
+    """Small-integer activations: every product and partial sum is exact in fp32, so the result must be too
+    (slow path = two's complement; fast paths = interleaved words, unsigned / minus two)."""
+    A, packed = _inputs(M, N, K, seed=M * 7 + N + K + int(fast), integer_a=True)
+    conv = "twos" if not fast else ("offset" if fmt == "int" else "unsigned")
+    B = orc.interleave_weight(packed.view(np.int8), 2, "float16").view(np.uint8) if fast else packed
+    kernel = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", num_bits=2, source_format=fmt, fast_decoding=fast)
+    got = _run(kernel, cuda, A, B)
+    acc = A.astype(np.int64) @ orc.decode_i2(packed, conv).astype(np.int64).T
+    np.testing.assert_array_equal(got.astype(np.float64), acc.astype(np.float16).astype(np.float64))
+
+
+@pytest.mark.parametrize("M,N,K,group", [(1, 1024, 1024, 128), (1, 28672, 8192, 128), (2, 300, 4096, 64), (4, 1024, 8192, 8192),
+                                         (1, 512, 11008, 64)])
+@pytest.mark.parametrize("fast,fmt", [(False, "int"), (True, "int"), (True, "uint")])
+def test_w2a16_scaled(cuda, M, N, K, group, fast, fmt):
+    """Gaussian activations and group scales against dequantise + fp32 matmul, rtol = atol = 1e-2, no mismatches."""
+    A, packed = _inputs(M, N, K, seed=N + K + group)
+    S = np.random.default_rng(3).uniform(0.005, 0.02, size=(N, K // group)).astype(np.float16)
+    conv = "twos" if not fast else ("offset" if fmt == "int" else "unsigned")
+    B = orc.interleave_weight(packed.view(np.int8), 2, "float16").view(np.uint8) if fast else packed
+    kernel = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", num_bits=2, source_format=fmt, fast_decoding=fast,
+                                group_size=group, with_scaling=True)
+    got = _run(kernel, cuda, A, B, S)
+    ref = orc.ref_w2a16(A, packed, conv, S, group)
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=1e-2, atol=1e-2)
+
+
+def test_w2a16_unscaled_gaussian_and_repeatable(cuda):
+    """Unscaled, Gaussian activations; two launches give bit-identical results (fixed reduction order)."""
+    M, N, K = 2, 4096, 8192
+    A, packed = _inputs(M, N, K, seed=9)
+    kernel = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", num_bits=2)
+    got = _run(kernel, cuda, A, packed)
+    again = _run(kernel, cuda, A, packed)
+    np.testing.assert_array_equal(got.view(np.uint16), again.view(np.uint16))
+    ref = orc.ref_w2a16(A, packed, "twos")
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=1e-2, atol=1e-2)
+
+
+def test_w2a16_rejections(cuda):
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, with_zeros=True, group_size=128)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, group_size=32)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(128, 64, 1024, "float16", "float16", "float32", num_bits=2)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=3)
