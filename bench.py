@@ -99,6 +99,27 @@ def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev):
             "inputs": d, "out": C}
 
 
+def bench_w2a16(torch, tl, M, N, K, steps, warmup, dev, fast=True):
+    """The 2-bit case of dequantize_gemv: codes uniform over 0..3 (interleaved words, w = (c - 2) * s), group 128."""
+    from tilelang_amd import quantize
+
+    group = 128
+    rng = np.random.default_rng(0)
+    A = torch.from_numpy(rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)).to(dev)
+    nbytes = N * K // 4 + 2 * N * K // group + 2 * M * K + 2 * M * N
+    nc = _copies(nbytes)
+    Bs = []
+    for _ in range(nc):
+        b = torch.from_numpy(rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)).view(torch.int8)
+        Bs.append((quantize.interleave_weight(b, 2, "float16") if fast else b).to(dev).contiguous())
+    Ss = [torch.from_numpy(rng.uniform(0.005, 0.02, size=(N, K // group)).astype(np.float16)).to(dev) for _ in range(nc)]
+    C = torch.empty((M, N), dtype=torch.float16, device=dev)
+    kern = tl.dequantize_gemv(M, N, K, num_bits=2, source_format="int", fast_decoding=fast, group_size=group, with_scaling=True)
+    fns = [(lambda i=i: kern(A, Bs[i], Ss[i], C, skip_tensor_validation=True)) for i in range(nc)]
+    ms, graphed = _time_launches(torch, fns, steps, warmup)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * M * N * K, "graph": graphed}
+
+
 def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev):
     d = workloads.mxfp4(M, N, K, seed=0, scale_bias=127)
     A = torch.from_numpy(d["A"]).to(dev).view(torch.bfloat16)
@@ -315,6 +336,8 @@ def main():
             shapes.append({"config": f"w4a16_zeros M={m} N=28672 K=8192", "us": r["us"], "GB/s": r["bytes"] / r["us"] / 1e3,
                            "TFLOP/s": r["flops"] / r["us"] / 1e6, "bound": "hbm", "frac": r["bytes"] / (r["us"] * 1e-6) / HBM_PEAK,
                            "frac_mfma": r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK})
+        r = bench_w2a16(torch, tl, 1, 28672, 8192, k, 4, dev)
+        shapes.append(_row("w2a16_gemv M=1 N=28672 K=8192 (num_bits=2, interleaved words, (c-2)*s)", r, "hbm", MFMA_BF16_PEAK))
         kg = max(6, args.steps // 10)
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, kg, 2, dev)
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))

@@ -9,20 +9,19 @@
 // of every weight row of its workgroup, the threads of a row read consecutive chunks, the loads of
 // a whole batch of rows are in flight before any of it is decoded.
 //
-//   * a packed dword holds 16 codes; (w & (3 << b, 3 << b)) | magic_b is the fp16 pair
-//     (2^(10-b) + c_lo, 2^(10-b) + c_hi) of the fields at bit b of the two halfwords, for
-//     b = 0,2,4,6,8 straight from w and for the fields at bits 10,12,14 from w >> 8.  One packed
-//     subtraction removes 2^(10-b) + zero point exactly, so the weights that reach v_dot2_f32_f16
-//     are the small integers themselves and the fp32 sum sees only exact products;
+//   * a packed dword holds 16 codes; w & 0x33333333 and (w >> 2) & 0x33333333 leave one code in every
+//     nibble, and a 2-bit code c read as an e2m1 nibble is c / 2, so v_cvt_scalef32_pk_f16_fp4 with the
+//     scale 2 turns each byte into the exact fp16 pair (c_lo, c_hi): eleven instructions decode a
+//     dword, eight v_dot2_f32_f16 consume it, and the fp32 sum sees only exact products;
 //   * the thread's 64 activations are arranged once, in registers, as the pairs that decode
-//     produces: (k, k + 8) of each 16 for the plain packing; for words passed through
-//     interleave_weight(qw, 2, "float16") (bytes e0 e2 e4 e6 | e1 e3 e5 e7 | e8.. | e9..) the pairs
-//     (2p, 2p + 8) and (2p - 7, 2p + 1);
-//   * two's-complement codes are (c ^ 2) - 2; a group scale multiplies the fp32 sum of the
-//     thread's chunk (a chunk of 64 k never straddles a group: group % 64 == 0).  With the signed
-//     codes (c - 2) * s is exact in fp16, so this equals the per-weight fp16 rounding of the
-//     reference's scaled decoder; with unsigned codes 3 * s is the one product that the reference
-//     rounds and this kernel does not;
+//     produces: (4j, 4j + 2) and (4j + 1, 4j + 3) for byte j of the plain packing; for words passed
+//     through interleave_weight(qw, 2, "float16") (bytes e0 e2 e4 e6 | e1 e3 e5 e7 | e8.. | e9..) the
+//     pairs (e, e + 4);
+//   * the zero point is applied per chunk as  sum a (c - 2) = sum a c - 2 sum a;  two's-complement
+//     codes are (c ^ 2) - 2; a group scale multiplies the fp32 sum of the thread's chunk (a chunk of
+//     64 k never straddles a group: group % 64 == 0).  With the signed codes (c - 2) * s is exact in
+//     fp16, so this equals the per-weight fp16 rounding of the reference's scaled decoder; with
+//     unsigned codes 3 * s is the one product that the reference rounds and this kernel does not;
 //   * K is reduced over the lanes with DPP row operations and over the waves of a row through LDS,
 //     in a fixed order: results are bit-identical from run to run.
 #include "dq_common.h"
@@ -49,25 +48,18 @@ __device__ __forceinline__ float wave_half_reduce_f32(float v) {
 
 constexpr int kMaxRowsPerWg = 128;
 
-// decode one packed dword into the eight fp16 pairs (c_lo - zp, c_hi - zp); pair p holds the
-// fields at bit 2p of the low and of the high halfword
-__device__ __forceinline__ void decode_w2_dword(uint32_t w, const half2_t (&sub)[5], half2_t (&out)[8]) {
-  uint32_t m0 = 0x00030003u, m2 = 0x000C000Cu, m4 = 0x00300030u, m6 = 0x00C000C0u, m8 = 0x03000300u;
-  // masks kept in registers so that every (w & mask) | magic is one v_and_or_b32
-  asm("" : "+v"(m0));
-  asm("" : "+v"(m2));
-  asm("" : "+v"(m4));
-  asm("" : "+v"(m6));
-  asm("" : "+v"(m8));
-  const uint32_t w8 = w >> 8;
-  out[0] = as_half2((w & m0) | 0x64006400u) - sub[0];   // 1024 + c
-  out[1] = as_half2((w & m2) | 0x5C005C00u) - sub[1];   // 256 + c
-  out[2] = as_half2((w & m4) | 0x54005400u) - sub[2];   // 64 + c
-  out[3] = as_half2((w & m6) | 0x4C004C00u) - sub[3];   // 16 + c
-  out[4] = as_half2((w & m8) | 0x44004400u) - sub[4];   // 4 + c
-  out[5] = as_half2((w8 & m2) | 0x5C005C00u) - sub[1];
-  out[6] = as_half2((w8 & m4) | 0x54005400u) - sub[2];
-  out[7] = as_half2((w8 & m6) | 0x4C004C00u) - sub[3];
+// decode one packed dword into eight fp16 pairs of codes: pair 2j + t holds fields t and t + 2 of byte j
+__device__ __forceinline__ void decode_w2_dword(uint32_t w, half2_t (&out)[8]) {
+  const uint32_t d0 = w & 0x33333333u;
+  const uint32_t d1 = (w >> 2) & 0x33333333u;
+  out[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, 2.0f, 0);
+  out[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d1, 2.0f, 0);
+  out[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, 2.0f, 1);
+  out[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d1, 2.0f, 1);
+  out[4] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, 2.0f, 2);
+  out[5] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d1, 2.0f, 2);
+  out[6] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, 2.0f, 3);
+  out[7] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d1, 2.0f, 3);
 }
 
 template <int MROWS, int NP, int R, bool IL, bool HAS_SCALE>
@@ -113,19 +105,10 @@ __global__ __launch_bounds__(256) void w2a16_gemv_kernel(const half_t* __restric
 #pragma unroll
   for (int u = 0; u < R; ++u) issue_row(u, 0);
 
-  // bias + zero point of the five field positions, as packed fp16 (exact: at most 1024 + 2)
-  half2_t sub[5];
-  {
-    const float bias[5] = {1024.f, 256.f, 64.f, 16.f, 4.f};
-#pragma unroll
-    for (int i = 0; i < 5; ++i) {
-      const half_t v = (half_t)(bias[i] + (float)zsub);
-      sub[i] = half2_t{v, v};
-    }
-  }
-
   // the thread's activations, paired as the decoder pairs the codes
   uint32_t a[NP][MROWS][32];
+  float zasum[NP][MROWS];  // zero point times the sum of the chunk's activations
+  const half2_t one2 = {(half_t)1.f, (half_t)1.f};
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
     const int chunk = p * tpr + ct;
@@ -133,6 +116,7 @@ __global__ __launch_bounds__(256) void w2a16_gemv_kernel(const half_t* __restric
 #pragma unroll
     for (int m = 0; m < MROWS; ++m) {
       const half_t* ap = A + (size_t)min(m, M - 1) * K + (size_t)min(chunk, c16 - 1) * 64;
+      float asum = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {  // packed dword j: k = 16 j .. 16 j + 15, natural registers n[0..7]
         uint4_t lo = *reinterpret_cast<const uint4_t*>(ap + j * 16);
@@ -144,18 +128,21 @@ __global__ __launch_bounds__(256) void w2a16_gemv_kernel(const half_t* __restric
         const uint32_t n[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
+          const int bj = q >> 1, t = q & 1;  // byte of the packed dword, first field of the pair
           uint32_t v;
           if constexpr (IL) {
-            // q < 4: (a[2q], a[2q + 8]); q >= 4: (a[2q - 7], a[2q + 1])
-            if (q < 4) v = __builtin_amdgcn_perm(n[(q + 4) & 7], n[q], 0x05040100u);
-            else v = __builtin_amdgcn_perm(n[q], n[(q - 4) & 7], 0x07060302u);
+            // byte bj holds e[8 (bj / 2) + (bj % 2) + 2 f] in field f: the pair is (e, e + 4)
+            const int i = 4 * (bj >> 1) + t;
+            v = __builtin_amdgcn_perm(n[i + 2], n[i], (bj & 1) ? 0x07060302u : 0x05040100u);
           } else {
-            // (a[q], a[q + 8])
-            v = __builtin_amdgcn_perm(n[q / 2 + 4], n[q / 2], (q & 1) ? 0x07060302u : 0x05040100u);
+            // byte bj holds e[4 bj + f] in field f: the pair is (4 bj + t, 4 bj + t + 2)
+            v = __builtin_amdgcn_perm(n[2 * bj + 1], n[2 * bj], t ? 0x07060302u : 0x05040100u);
           }
           a[p][m][j * 8 + q] = v;
+          asum = __builtin_amdgcn_fdot2(as_half2(v), one2, asum, false);
         }
       }
+      zasum[p][m] = (float)zsub * asum;
     }
   }
 
@@ -173,7 +160,7 @@ __global__ __launch_bounds__(256) void w2a16_gemv_kernel(const half_t* __restric
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           half2_t wv[8];
-          decode_w2_dword(bq[u][p][j] ^ flip_mask, sub, wv);
+          decode_w2_dword(bq[u][p][j] ^ flip_mask, wv);
 #pragma unroll
           for (int q = 0; q < 8; ++q) {
 #pragma unroll
@@ -183,8 +170,8 @@ __global__ __launch_bounds__(256) void w2a16_gemv_kernel(const half_t* __restric
         }
 #pragma unroll
         for (int m = 0; m < MROWS; ++m) {
-          if constexpr (HAS_SCALE) acc[u][m] = __builtin_fmaf((float)sq[u][p], part[m], acc[u][m]);
-          else acc[u][m] += part[m];
+          if constexpr (HAS_SCALE) acc[u][m] = __builtin_fmaf((float)sq[u][p], part[m] - zasum[p][m], acc[u][m]);
+          else acc[u][m] += part[m] - zasum[p][m];
         }
       }
     }
