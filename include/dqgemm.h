@@ -106,16 +106,19 @@ int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int
 int call_dequant_gemm_fp16_fp4_splitk(const void* A, const void* B, void* SplitC, void* C, int M, int N, int K,
                                       int split, int transposed, dq_stream_t stream);
 
-/* The 2-bit case of the same example (`num_bits = 2`: B[N, K/4], sixteen codes per 32-bit word):
- * C[M,N] fp16 = A[M,K] fp16 . decode(B)^T (. Scale[N, K/group]), fp32 accumulation.  `convention` is a
- * DQ_I2_* value: DQ_I2_TWOS is the example's slow path (`_tir_packed_int_to_int_convert`,
- * examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124), DQ_I2_UNSIGNED / DQ_I2_OFFSET are
- * decode_i2u_to_f16 / decode_i2s_to_f16 (examples/dequantize_gemm/quantize/lop3.py:424-463; with Scale :465-500).
- * DQ_LAYOUT_INTERLEAVED: words passed through interleave_weight(qw, 2, "float16")
- * (examples/dequantize_gemm/quantize/utils.py:71-114).  Scale may be NULL.  Decode batches only: M <= 64
- * (rows go through the kernel two at a time).  Requires K % 64 == 0, K <= 32768, group % 64 == 0. */
-int call_dequantize_gemv_w2a16(const void* A, const void* B, const void* Scale, void* C, int M, int N, int K, int group,
-                               int convention, int layout, dq_stream_t stream);
+/* The 2-bit and 1-bit cases of the same example (`num_bits`: B[N, K * bits / 8], 16 or 32 codes per 32-bit word):
+ * C[M,N] fp16 = A[M,K] fp16 . dequant(B, Scale[N, K/group], Zeros[N, K/group])^T, fp32 accumulation.
+ * `convention` is a DQ_I2_* value: DQ_I2_TWOS is the example's slow path (`_tir_packed_int_to_int_convert`,
+ * examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124); DQ_I2_UNSIGNED is decode_i2u_to_f16 /
+ * decode_i1u_to_f16 (w = c); DQ_I2_OFFSET is decode_i2s_to_f16 (w = c - 2) / decode_i1s_to_f16 (w = 2 c - 1)
+ * (examples/dequantize_gemm/quantize/lop3.py:424-463, 679-746).  With Scale: w * s (lop3.py:465-500, 748-810); with
+ * Zeros as well: (w - z) * s, or w * s - z when `zeros_rescale` is non-zero (lop3.py:564-636, 812-891).
+ * DQ_LAYOUT_INTERLEAVED: words passed through interleave_weight(qw, bits, "float16")
+ * (examples/dequantize_gemm/quantize/utils.py:71-123).  Scale and Zeros may be NULL.  Decode batches only: M <= 64
+ * (rows go through the kernel two at a time).  Requires K % (128 / bits) == 0, K <= 32768, group % (128 / bits) == 0. */
+int call_dequantize_gemv_lowbit(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M, int N,
+                                int K, int group, int bits, int convention, int layout, int zeros_rescale,
+                                dq_stream_t stream);
 
 /* fp16 x uint4 with the integer decoders: C[M,N] fp16 = A[M,K] fp16 . dequant(B, Scale, Zeros)^T with
  * the dequantised tile rounded to fp16 exactly as call_dequantize_w4 does.  Replaces `call(A, B, C)` of

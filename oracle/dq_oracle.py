@@ -268,28 +268,87 @@ def fast_decode_i2_to_f16(halfwords: np.ndarray, signed: bool, scale=None) -> np
     return out
 
 
-def dequant_u2(packed: np.ndarray, convention: str = "twos", scale: np.ndarray | None = None, group: int = -1) -> np.ndarray:
-    """2-bit codes -> fp16 weights ``w = decode_i2(c)`` (exact), times ``s[n, k // group]`` with one fp16 rounding.
+def fast_decode_i1_to_f16(bytes_: np.ndarray, signed: bool) -> np.ndarray:
+    """Semantics of decode_i1{u,s}_to_f16 on one byte -> 8 fp16, in output order.
 
-    ``"twos"`` is the GEMV example's slow path (``_tir_packed_int_to_int_convert`` with ``num_bits = 2``,
-    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124 and quantize/quantization.py:333-343);
-    ``"unsigned"`` / ``"offset"`` are decode_i2u_to_f16 / decode_i2s_to_f16 (quantize/lop3.py:424-463), the scaled
-    forms lop3.py:465-500: exact ``c - zp`` then ``fma.rn.f16x2(x, s, 0)``.
-    PARITY UNPINNED by reference tests for the scaled form (no caller in the reference).
+    Follows examples/dequantize_gemm/quantize/lop3.py:679-746: ``i1s = (x & 0x0f) | ((x & 0xf0) << 12)``; for i in
+    0..3 ``h[i] = ((i1s >> i) & 0x00010001) | 0x64006400`` as two fp16 (1024 + c) minus 1024; the signed form then
+    computes ``h + h - 1`` (``2 c - 1``).  Output element ``2i`` is the low half.
     """
-    w = decode_i2(packed, convention).astype(np.float32)
+    x = np.asarray(bytes_).astype(np.uint32) & np.uint32(0xFF)
+    i1s = (x & np.uint32(0x0F)) | ((x & np.uint32(0xF0)) << np.uint32(12))
+    out = np.empty(x.shape + (8,), dtype=np.float16)
+    for i in range(4):
+        h = ((i1s >> np.uint32(i)) & np.uint32(0x00010001)) | np.uint32(0x64006400)
+        lo = (h & 0xFFFF).astype(np.uint16).view(np.float16) - np.float16(1024.0)
+        hi = (h >> 16).astype(np.uint16).view(np.float16) - np.float16(1024.0)
+        if signed:
+            lo = lo + lo - np.float16(1.0)
+            hi = hi + hi - np.float16(1.0)
+        out[..., 2 * i] = lo
+        out[..., 2 * i + 1] = hi
+    return out
+
+
+def decode_lowbit(packed: np.ndarray, bits: int, convention: str = "twos") -> np.ndarray:
+    """1- or 2-bit codes -> integer weights (int8), element ``e`` of a byte at bit ``bits * e``.
+
+    ``"unsigned"``: ``c``; ``"twos"``: two's complement of the field
+    (examples/dequantize_gemm/quantize/quantization.py:333-343); ``"offset"``: the signed fast decoders,
+    ``c - 2`` for two bits (lop3.py:430,446) and ``2 c - 1`` for one bit (lop3.py:699,719-723).
+    """
+    c = general_decompress(np.asarray(packed).view(np.uint8), bits).astype(np.int16)
+    if convention == "unsigned":
+        return c.astype(np.int8)
+    if convention == "twos":
+        return sign_extend(c, bits).astype(np.int8)
+    if convention == "offset":
+        return ((c - 2) if bits == 2 else (2 * c - 1)).astype(np.int8)
+    raise ValueError(convention)
+
+
+def dequant_lowbit(packed, bits: int, convention: str = "twos", scale=None, zeros=None, group: int = -1,
+                   zeros_mode: str = "original") -> np.ndarray:
+    """1- or 2-bit codes -> fp16 weights with the rounding order of the device snippets.
+
+    No scale: ``w`` exact.  Scale: ``RNE16(w * s)`` (``fma.rn.f16x2(x, s, 0)``, lop3.py:465-500, 748-810).  Zeros
+    ``"original"``: ``RNE16(RNE16(w - z) * s)`` (sub, then fma: lop3.py:564-599, 812-851); ``"rescale"``:
+    ``RNE16(RNE16(w * s) - z)`` (fma with 0, then sub: lop3.py:601-636, 853-891; the one-bit form :719-735).
+    PARITY UNPINNED by reference tests for the scaled and zero-point forms (no caller in the reference).
+    """
+    w = decode_lowbit(packed, bits, convention).astype(np.float32)
     if scale is None:
         return w.astype(np.float16)
     K = w.shape[-1]
-    s = _expand_groups(np.asarray(scale, dtype=np.float16), K, K if group == -1 else group).astype(np.float32)
-    return ((w * s) + np.float32(0.0)).astype(np.float16)
+    g = K if group == -1 else group
+    s = _expand_groups(np.asarray(scale, dtype=np.float16), K, g).astype(np.float32)
+    if zeros is None:
+        return ((w * s) + np.float32(0.0)).astype(np.float16)
+    z = _expand_groups(np.asarray(zeros, dtype=np.float16), K, g).astype(np.float32)
+    if zeros_mode == "original":
+        d = (w - z).astype(np.float16).astype(np.float32)
+        return ((d * s) + np.float32(0.0)).astype(np.float16)
+    if zeros_mode == "rescale":
+        d = ((w * s) + np.float32(0.0)).astype(np.float16).astype(np.float32)
+        return (d - z).astype(np.float16)
+    raise ValueError(zeros_mode)
+
+
+def dequant_u2(packed: np.ndarray, convention: str = "twos", scale: np.ndarray | None = None, group: int = -1) -> np.ndarray:
+    """The two-bit case of :func:`dequant_lowbit` without zeros."""
+    return dequant_lowbit(packed, 2, convention, scale, None, group)
+
+
+def ref_lowbit(A, packed, bits: int, convention: str = "twos", scale=None, zeros=None, group: int = -1,
+               zeros_mode: str = "original") -> np.ndarray:
+    """``ref_program`` of the 1- / 2-bit GEMV: dequantise, fp32 matmul, fp16 out (the pattern of
+    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:207-217 with the narrower unpack)."""
+    W = dequant_lowbit(packed, bits, convention, scale, zeros, group, zeros_mode)
+    return _matmul_f32(np.asarray(A, dtype=np.float16), W).astype(np.float16)
 
 
 def ref_w2a16(A, packed, convention: str = "twos", scale=None, group: int = -1) -> np.ndarray:
-    """``ref_program`` of the 2-bit GEMV: dequantise, fp32 matmul, fp16 out (the pattern of
-    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:207-217 with the 2-bit unpack)."""
-    W = dequant_u2(packed, convention, scale, group)
-    return _matmul_f32(np.asarray(A, dtype=np.float16), W).astype(np.float16)
+    return ref_lowbit(A, packed, 2, convention, scale, None, group)
 
 
 # --------------------------------------------------------------------------------------

@@ -1,4 +1,4 @@
-"""GPU parity of the 2-bit case of dequantize_gemv (fp16 activations, B[N, K/4]) through the C-ABI."""
+"""GPU parity of the 2-bit and 1-bit cases of dequantize_gemv (fp16 activations, B[N, K * bits / 8]) through the C-ABI."""
 
 import numpy as np
 import pytest
@@ -76,10 +76,66 @@ def test_w2a16_unscaled_gaussian_and_repeatable(cuda):
 
 def test_w2a16_rejections(cuda):
     with pytest.raises(ValueError):
-        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, with_zeros=True, group_size=128)
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, with_zeros=True,
+                           zeros_mode="quantized", group_size=128)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=1, with_scaling=True, group_size=64)
     with pytest.raises(ValueError):
         tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, group_size=32)
     with pytest.raises(ValueError):
         tl.dequantize_gemv(128, 64, 1024, "float16", "float16", "float32", num_bits=2)
     with pytest.raises(ValueError):
         tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=3)
+
+
+# ---- one bit, and the zero-point forms of both widths ---------------------------------------------------------
+
+
+def _packed(N, K, bits, seed):
+    return np.random.default_rng(seed).integers(0, 256, size=(N, K * bits // 8), dtype=np.uint8)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (1, 256, 128), (2, 1000, 4096), (1, 512, 11008), (3, 517, 8192), (1, 40, 32768)])
+@pytest.mark.parametrize("fast,fmt", [(False, "uint"), (True, "uint"), (True, "int")])
+def test_w1a16_exact_integers(cuda, M, N, K, fast, fmt):
+    """One bit per weight, small-integer activations: exact (two's complement -c; fast decoders c and 2c - 1 on
+    words passed through the 1-bit interleave)."""
+    A = np.random.default_rng(M + N + K).integers(-4, 5, size=(M, K)).astype(np.float16)
+    packed = _packed(N, K, 1, seed=K + int(fast))
+    conv = "twos" if not fast else ("offset" if fmt == "int" else "unsigned")
+    B = orc.interleave_weight(packed.view(np.int8), 1, "float16").view(np.uint8) if fast else packed
+    kernel = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", num_bits=1, source_format=fmt, fast_decoding=fast)
+    got = _run(kernel, cuda, A, B)
+    acc = A.astype(np.int64) @ orc.decode_lowbit(packed, 1, conv).astype(np.int64).T
+    np.testing.assert_array_equal(got.astype(np.float64), acc.astype(np.float16).astype(np.float64))
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("M,N,K,group", [(1, 1024, 1024, 128), (1, 28672, 8192, 128), (2, 300, 4096, 256), (3, 64, 8192, 8192)])
+@pytest.mark.parametrize("fast,fmt,zeros_mode", [(True, "uint", "original"), (True, "uint", "rescale"), (True, "int", "original"),
+                                                 (False, "int", "rescale"), (True, "int", None)])
+def test_lowbit_scale_and_zeros(cuda, bits, M, N, K, group, fast, fmt, zeros_mode):
+    """Group scales and zero points (original: (w - z) s; rescale: w s - z) against dequantise + fp32 matmul."""
+    rng = np.random.default_rng(bits * 1000 + N + K + group)
+    A = rng.standard_normal((M, K)).astype(np.float16)
+    packed = _packed(N, K, bits, seed=N + bits)
+    S = rng.uniform(0.005, 0.02, size=(N, K // group)).astype(np.float16)
+    if zeros_mode == "original":
+        Z = rng.integers(0, 1 << bits, size=(N, K // group)).astype(np.float16)
+    elif zeros_mode == "rescale":
+        Z = (rng.uniform(0.0, 0.03, size=(N, K // group))).astype(np.float16)
+    else:
+        Z = None
+    conv = "twos" if not fast else ("offset" if fmt == "int" else "unsigned")
+    B = orc.interleave_weight(packed.view(np.int8), bits, "float16").view(np.uint8) if fast else packed
+    kernel = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", num_bits=bits, source_format=fmt, fast_decoding=fast,
+                                group_size=group, with_scaling=True, with_zeros=Z is not None,
+                                zeros_mode=zeros_mode or "original")
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    args = [torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda), torch.from_numpy(S).to(cuda)]
+    if Z is not None:
+        args.append(torch.from_numpy(Z).to(cuda))
+    kernel(*args, C)
+    torch.cuda.synchronize()
+    ref = orc.ref_lowbit(A, packed, bits, conv, S, Z, group, zeros_mode or "original")
+    np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=1e-2, atol=1e-2)

@@ -530,3 +530,41 @@ def test_ref_w2a16_brute_force():
             np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)
     # sign extension of the reference's own known answer (test_tilelang_u32_signed_decode.py:26-30): codes 2,3,0,1 -> -2..1
     np.testing.assert_array_equal(orc.dequant_u2(np.array([[0b01001110]], dtype=np.uint8), "twos")[0], np.array([-2, -1, 0, 1], dtype=np.float16))
+
+
+def test_i1_to_f16_fast_decode_all_bytes_and_interleave():
+    """decode_i1{u,s}_to_f16 (lop3.py:679-746) over all 256 inputs against the closed form (outputs 2i, 2i+1 are bits i
+    and 4 + i: c, or 2c - 1 signed), fast_decode(interleave_weight(p, 1, "float16")) == plain decode, and the known
+    answer of the reference's own sign-extension test for one bit (0 -> 0, 1 -> -1)."""
+    x = np.arange(256, dtype=np.uint32)
+    for signed in (False, True):
+        out = orc.fast_decode_i1_to_f16(x, signed).astype(np.float32)
+        for i in range(4):
+            lo = ((x >> i) & 1).astype(np.float32)
+            hi = ((x >> (4 + i)) & 1).astype(np.float32)
+            if signed:
+                lo, hi = 2 * lo - 1, 2 * hi - 1
+            np.testing.assert_array_equal(out[:, 2 * i], lo)
+            np.testing.assert_array_equal(out[:, 2 * i + 1], hi)
+    raw = np.random.default_rng(8).integers(0, 256, size=(8, 64), dtype=np.uint8)
+    il = orc.interleave_weight(raw.view(np.int8), 1, "float16").view(np.uint8)
+    fast = orc.fast_decode_i1_to_f16(il, signed=True).reshape(8, -1)
+    np.testing.assert_array_equal(fast.astype(np.float32), orc.decode_lowbit(raw, 1, "offset").astype(np.float32))
+    fastu = orc.fast_decode_i1_to_f16(il, signed=False).reshape(8, -1)
+    np.testing.assert_array_equal(fastu.astype(np.float32), orc.decode_lowbit(raw, 1, "unsigned").astype(np.float32))
+    np.testing.assert_array_equal(orc.decode_lowbit(np.array([[0b10110010]], dtype=np.uint8), 1, "twos")[0], [0, -1, 0, 0, -1, -1, 0, -1])
+
+
+def test_dequant_lowbit_rounding_order():
+    """Zero-point forms: original rounds (w - z) then the product; rescale rounds the product then the difference;
+    checked against float64 arithmetic with explicit roundings on values chosen so that the orders differ."""
+    packed = np.array([[0b11100100]], dtype=np.uint8)  # 2-bit codes 0, 1, 2, 3
+    s = np.array([[0.00949859619140625]], dtype=np.float16)
+    z = np.array([[0.26904296875]], dtype=np.float16)
+    c = np.array([0.0, 1.0, 2.0, 3.0])
+    f16 = lambda v: np.asarray(v, dtype=np.float64).astype(np.float16).astype(np.float64)
+    got_o = orc.dequant_lowbit(packed, 2, "unsigned", s, z, 4, "original").astype(np.float64)[0]
+    np.testing.assert_array_equal(got_o, f16(f16(c - float(z[0, 0])) * float(s[0, 0])))
+    got_r = orc.dequant_lowbit(packed, 2, "unsigned", s, z, 4, "rescale").astype(np.float64)[0]
+    np.testing.assert_array_equal(got_r, f16(f16(c * float(s[0, 0])) - float(z[0, 0])))
+    assert not np.array_equal(got_r, f16(c * float(s[0, 0]) - float(z[0, 0])))  # a single rounding would differ

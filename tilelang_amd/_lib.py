@@ -27,7 +27,7 @@ _vp, _i = ctypes.c_void_p, ctypes.c_int
 SIGNATURES = {
     "init": [],
     "call_dequantize_gemv_w4a16": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
-    "call_dequantize_gemv_w2a16": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "call_dequantize_gemv_lowbit": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequantize_w4": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_bf16_mxfp4": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],

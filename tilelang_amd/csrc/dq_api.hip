@@ -32,8 +32,8 @@ int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void
                 int mode, int layout, hipStream_t stream);
 int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int bitnet_epilogue, hipStream_t stream);
-int w2a16_gemv(const void* A, const void* B, const void* Scale, void* C, int M, int N, int K, int group, int convention,
-               int layout, hipStream_t stream);
+int wlow_gemv(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M, int N, int K, int group,
+              int bits, int convention, int layout, int zeros_rescale, hipStream_t stream);
 int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int out_kind, hipStream_t stream);
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
@@ -129,26 +129,30 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
 }
 
-extern "C" int call_dequantize_gemv_w2a16(const void* A, const void* B, const void* Scale, void* C, int M, int N, int K,
-                                          int group, int convention, int layout, dq_stream_t stream) {
-  const char* fn = "call_dequantize_gemv_w2a16";
+extern "C" int call_dequantize_gemv_lowbit(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
+                                           int M, int N, int K, int group, int bits, int convention, int layout,
+                                           int zeros_rescale, dq_stream_t stream) {
+  const char* fn = "call_dequantize_gemv_lowbit";
   if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
   if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
   if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
+  if (bits != 1 && bits != 2) DQ_FAIL("%s: bits must be 1 or 2 (got %d)", fn, bits);
   if (M <= 0 || N <= 0 || K <= 0) DQ_FAIL("%s: M, N, K must be positive (got %d %d %d)", fn, M, N, K);
   if (M > 64) DQ_FAIL("%s: M=%d is beyond the decode batch this kernel is built for (64)", fn, M);
-  if (K % 64 != 0) DQ_FAIL("%s: K=%d must be a multiple of 64", fn, K);
+  const int chunk = 128 / bits;  // codes in 16 bytes
+  if (K % chunk != 0) DQ_FAIL("%s: K=%d must be a multiple of %d", fn, K, chunk);
   if (K > 32768) DQ_FAIL("%s: K=%d is beyond the 32768 this kernel is built for", fn, K);
   if (convention < I2_UNSIGNED || convention > I2_TWOS) DQ_FAIL("%s: unknown code convention %d", fn, convention);
   if (layout != LAYOUT_PLAIN && layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
+  if (Zeros && !Scale) DQ_FAIL("%s: Zeros without Scale", fn);
   if (Scale) {
-    if (group <= 0 || group % 64 != 0 || K % group != 0)
-      DQ_FAIL("%s: group=%d must be a multiple of 64 that divides K=%d", fn, group, K);
+    if (group <= 0 || group % chunk != 0 || K % group != 0)
+      DQ_FAIL("%s: group=%d must be a multiple of %d that divides K=%d", fn, group, chunk, K);
   } else {
     group = K;
   }
   if (!aligned16(A) || !aligned16(B)) DQ_FAIL("%s: A and B must be 16-byte aligned", fn);
-  const int rc = w2a16_gemv(A, B, Scale, C, M, N, K, group, convention, layout, (hipStream_t)stream);
+  const int rc = wlow_gemv(A, B, Scale, Zeros, C, M, N, K, group, bits, convention, layout, zeros_rescale, (hipStream_t)stream);
   if (rc > 0) DQ_FAIL("%s: shape M=%d N=%d K=%d is not covered", fn, M, N, K);
   return rc;
 }

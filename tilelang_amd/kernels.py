@@ -94,15 +94,15 @@ def dequantize_gemv(
     """
     assert trans_A is False, "Dequantize only implement for trans_A=False currently"
     assert trans_B is True, "Dequantize only implement for trans_B=TRue currently"
-    if num_bits not in (2, 4):
-        raise ValueError("dequantize_gemv: num_bits must be 4 or 2")
+    if num_bits not in (1, 2, 4):
+        raise ValueError("dequantize_gemv: num_bits must be 4, 2 or 1")
     if _dtype(in_dtype) != torch.float16 or _dtype(out_dtype) != torch.float16:
         raise ValueError("dequantize_gemv: in_dtype and out_dtype must be float16 (int8 x int2: bitnet_158_int8xint2_decode)")
     if _dtype(storage_dtype) not in (torch.int8, torch.uint8):
         raise ValueError("dequantize_gemv: storage_dtype must be int8 or uint8")
-    if num_bits == 2:
-        return _dequantize_gemv_w2(M, N, K, storage_dtype, source_format, fast_decoding, group_size, with_scaling,
-                                   with_zeros, _formula_fast)
+    if num_bits < 4:
+        return _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fast_decoding, group_size,
+                                       with_scaling, with_zeros, zeros_mode, _formula_fast)
     if group_size == -1:
         group_size = K
     if K % 128 != 0:
@@ -136,42 +136,52 @@ def dequantize_gemv(
     return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
 
 
-def _dequantize_gemv_w2(M, N, K, storage_dtype, source_format, fast_decoding, group_size, with_scaling, with_zeros,
-                        _formula_fast) -> KernelAdapter:
-    """The ``num_bits=2`` case of :func:`dequantize_gemv`: ``B[N, K/4]``, sixteen codes per 32-bit word.
+def _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fast_decoding, group_size, with_scaling,
+                            with_zeros, zeros_mode, _formula_fast) -> KernelAdapter:
+    """The ``num_bits`` = 2 and 1 cases of :func:`dequantize_gemv`: ``B[N, K * num_bits / 8]``.
 
     Slow path: two's-complement codes whatever ``source_format`` says
     (examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124).  ``fast_decoding=True``: B went through
-    ``interleave_weight(B, 2, "float16")`` and decodes as ``c`` (``"uint"``, decode_i2u_to_f16) or ``c - 2``
-    (``"int"``, decode_i2s_to_f16; examples/dequantize_gemm/quantize/lop3.py:424-463), times ``Scale[N, K/group]``
-    with ``with_scaling`` (lop3.py:465-500).  Call surface ``kernel(A, B[, Scale], C)``.
+    ``interleave_weight(B, num_bits, "float16")`` and decodes as ``c`` (``"uint"``) or as ``c - 2`` / ``2 c - 1``
+    (``"int"``, two bits / one bit; examples/dequantize_gemm/quantize/lop3.py:424-463, 679-746), times
+    ``Scale[N, K/group]`` with ``with_scaling``, and with ``with_zeros`` ``(w - z) * s`` (``"original"``) or
+    ``w * s - z`` (``"rescale"``) (lop3.py:564-636, 812-891).  Call surface ``kernel(A, B[, Scale[, Zeros]], C)``.
     """
-    if with_zeros:
-        raise ValueError("dequantize_gemv: with_zeros is built for num_bits=4 only")
+    chunk = 128 // num_bits
     if group_size == -1:
         group_size = K
     if K % 128 != 0:
         raise ValueError(f"dequantize_gemv: K={K} must be a multiple of 128")
     if K > 32768:
-        raise ValueError(f"dequantize_gemv: num_bits=2 is built for K <= 32768 (got {K})")
+        raise ValueError(f"dequantize_gemv: num_bits={num_bits} is built for K <= 32768 (got {K})")
     if M > 64:
-        raise ValueError(f"dequantize_gemv: num_bits=2 is a decode kernel, M <= 64 (got {M})")
-    if with_scaling and (K % group_size != 0 or group_size % 64 != 0):
-        raise ValueError(f"dequantize_gemv: group_size={group_size} must divide K={K} and be a multiple of 64")
+        raise ValueError(f"dequantize_gemv: num_bits={num_bits} is a decode kernel, M <= 64 (got {M})")
+    if with_zeros and not with_scaling:
+        raise ValueError("with_zeros requires with_scaling")
+    if with_zeros and zeros_mode not in ("original", "rescale"):
+        raise ValueError(f"dequantize_gemv: zeros_mode {zeros_mode!r} is not built for num_bits={num_bits}")
+    if with_scaling and (K % group_size != 0 or group_size % chunk != 0):
+        raise ValueError(f"dequantize_gemv: group_size={group_size} must divide K={K} and be a multiple of {chunk}")
     formula_fast = fast_decoding if _formula_fast is None else _formula_fast
     if not formula_fast:
         conv = I2_TWOS
     else:
         conv = I2_OFFSET if source_format == "int" else I2_UNSIGNED
     layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
-    params = [KernelParam("A", torch.float16, (M, K)), KernelParam("B", _dtype(storage_dtype), (N, K // 4), packed=True)]
+    rescale = 1 if (with_zeros and zeros_mode == "rescale") else 0
+    params = [KernelParam("A", torch.float16, (M, K)),
+              KernelParam("B", _dtype(storage_dtype), (N, K * num_bits // 8), packed=True)]
     if with_scaling:
         params.append(KernelParam("Scale", torch.float16, (N, K // group_size)))
+    if with_zeros:
+        params.append(KernelParam("Zeros", torch.float16, (N, K // group_size)))
     params.append(KernelParam("C", torch.float16, (M, N)))
 
     def launch(ptrs, stream):
         s = ptrs[2] if with_scaling else None
-        return _lib.get_library().call_dequantize_gemv_w2a16(ptrs[0], ptrs[1], s, ptrs[-1], M, N, K, group_size, conv, layout, stream)
+        z = ptrs[3] if with_zeros else None
+        return _lib.get_library().call_dequantize_gemv_lowbit(ptrs[0], ptrs[1], s, z, ptrs[-1], M, N, K, group_size, num_bits,
+                                                              conv, layout, rescale, stream)
 
     return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
 
