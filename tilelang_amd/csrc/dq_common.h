@@ -10,6 +10,7 @@ namespace dq {
 
 typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));

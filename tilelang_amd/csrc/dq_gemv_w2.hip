@@ -13,8 +13,8 @@
 //
 //   * (w >> t) & 0x33333333 (t = 0, 2) or & 0x11111111 (t = 0..3) leaves one code in every nibble,
 //     and a code read as an e2m1 nibble is c / 2, so v_cvt_scalef32_pk_f16_fp4 with the scale 2
-//     turns each byte into the exact fp16 pair (c_lo, c_hi); v_dot2_f32_f16 consumes the pair, and
-//     the fp32 sum sees only exact products;
+//     turns each byte into the exact fp16 pair (c_lo, c_hi); the products with the activations are
+//     exact in fp32 and are summed on the matrix pipe (see the loop), so the VALU only decodes;
 //   * the thread's activations are arranged once, in registers, as the pairs that decode produces;
 //     which two elements meet in a byte follows from the packing (plain, or the words of
 //     interleave_weight(qw, bits, "float16"), examples/dequantize_gemm/quantize/utils.py:71-123) and
@@ -201,19 +201,34 @@ __global__ __launch_bounds__(256) void wlow_gemv_kernel(const half_t* __restrict
       for (int m = 0; m < MROWS; ++m) acc[u][m] = 0.f;
 #pragma unroll
       for (int p = 0; p < NP; ++p) {
-        float part[MROWS];
+        // Four k per lane and instruction on the matrix pipe: v_mfma_f32_4x4x4_16B_f16 multiplies, in each
+        // group of four lanes, the four weight vectors with the four activation vectors of those lanes; the
+        // diagonal (lane i: register i) is the lane's own dot product, the other twelve products are unused.
+        // The conversions above it stay on the VALU, so the two pipes overlap.
+        float4_t part4[MROWS];
 #pragma unroll
-        for (int m = 0; m < MROWS; ++m) part[m] = 0.f;
+        for (int m = 0; m < MROWS; ++m) part4[m] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           half2_t wv[PAIRS];
           decode_codes<BITS>(bq[u][p][j] ^ flip_mask, wv);
 #pragma unroll
-          for (int q = 0; q < PAIRS; ++q) {
+          for (int q = 0; q < PAIRS; q += 2) {
+            const half4_t w4 = {wv[q][0], wv[q][1], wv[q + 1][0], wv[q + 1][1]};
 #pragma unroll
-            for (int m = 0; m < MROWS; ++m)
-              part[m] = __builtin_amdgcn_fdot2(as_half2(a[p][m][j * PAIRS + q]), wv[q], part[m], false);
+            for (int m = 0; m < MROWS; ++m) {
+              const half2_t a0 = as_half2(a[p][m][j * PAIRS + q]), a1 = as_half2(a[p][m][j * PAIRS + q + 1]);
+              const half4_t a4 = {a0[0], a0[1], a1[0], a1[1]};
+              part4[m] = __builtin_amdgcn_mfma_f32_4x4x4f16(w4, a4, part4[m], 0, 0, 0);
+            }
           }
+        }
+        float part[MROWS];
+#pragma unroll
+        for (int m = 0; m < MROWS; ++m) {
+          const float p01 = (lane & 1) ? part4[m][1] : part4[m][0];
+          const float p23 = (lane & 1) ? part4[m][3] : part4[m][2];
+          part[m] = (lane & 2) ? p23 : p01;
         }
 #pragma unroll
         for (int m = 0; m < MROWS; ++m) {
@@ -233,11 +248,9 @@ __global__ __launch_bounds__(256) void wlow_gemv_kernel(const half_t* __restrict
           }
         }
       }
-    }
-    // every row of the batch is consumed: refill all of them (wave-uniform branch)
-    if (b + 1 < nb) {
-#pragma unroll
-      for (int u = 0; u < R; ++u) issue_row(u, b + 1);
+      // the row's registers are free: its place in the next batch is requested while the other rows are
+      // worked on (wave-uniform branch)
+      if (b + 1 < nb) issue_row(u, b + 1);
     }
 #pragma unroll
     for (int u = 0; u < R; ++u) {
@@ -277,10 +290,11 @@ struct LowArgs {
 
 template <int BITS, int MROWS, int NP, bool IL, int SZ>
 int launch_low(const LowArgs& g) {
-  constexpr int R = 4 / NP;
+  constexpr int R = 4 / NP;  // rows in flight per thread (eight measured slower)
   const int rpp = 256 >> g.tpr_shift;
   const long wgs1 = ((long)g.N + R * rpp - 1) / (R * rpp);
   // about two workgroups per CU, each walking several batches of rows
+  // (measured at N = 28672, K = 8192: 512 workgroups 15.8 us, 1024 17.5 us, one batch each 20.7 us)
   int nb = (int)((wgs1 + 511) / 512);
   while (nb > 1 && nb * R * rpp > kMaxRowsPerWg) --nb;
   if (nb < 1) nb = 1;
