@@ -256,3 +256,18 @@ def test_workload_generators_are_seeded_and_shaped():
     assert workloads.mxfp4_bytes(4096, 8192, 8192) == 169869312
     assert workloads.bitnet_bytes(2048, 8192, 8192) == 67117060
     assert workloads.flops(4096, 8192, 8192) == 549755813888
+
+
+def test_lowbit_gemv_factory_rejections():
+    """Shape and option checks of dequantize_gemv(num_bits=2 / 1) fire before any launch (no GPU needed)."""
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, with_zeros=True,
+                           zeros_mode="quantized", group_size=128)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=1, with_scaling=True, group_size=64)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, group_size=32)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(128, 64, 1024, "float16", "float16", "float32", num_bits=2)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=3)

@@ -74,20 +74,6 @@ def test_w2a16_unscaled_gaussian_and_repeatable(cuda):
     np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=1e-2, atol=1e-2)
 
 
-def test_w2a16_rejections(cuda):
-    with pytest.raises(ValueError):
-        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, with_zeros=True,
-                           zeros_mode="quantized", group_size=128)
-    with pytest.raises(ValueError):
-        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=1, with_scaling=True, group_size=64)
-    with pytest.raises(ValueError):
-        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=2, with_scaling=True, group_size=32)
-    with pytest.raises(ValueError):
-        tl.dequantize_gemv(128, 64, 1024, "float16", "float16", "float32", num_bits=2)
-    with pytest.raises(ValueError):
-        tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=3)
-
-
 # ---- one bit, and the zero-point forms of both widths ---------------------------------------------------------
 
 
