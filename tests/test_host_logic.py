@@ -271,3 +271,9 @@ def test_lowbit_gemv_factory_rejections():
         tl.dequantize_gemv(128, 64, 1024, "float16", "float16", "float32", num_bits=2)
     with pytest.raises(ValueError):
         tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=3)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "int8", "float16", "int32", num_bits=2)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "int8", "int32", "int32", num_bits=4, fast_decoding=True)
+    with pytest.raises(ValueError):
+        tl.dequantize_gemv(1, 64, 1024, "int8", "int32", "int32", num_bits=2, with_scaling=True, group_size=128)

@@ -125,3 +125,27 @@ def test_lowbit_scale_and_zeros(cuda, bits, M, N, K, group, fast, fmt, zeros_mod
     torch.cuda.synchronize()
     ref = orc.ref_lowbit(A, packed, bits, conv, S, Z, group, zeros_mode or "original")
     np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=1e-2, atol=1e-2)
+
+
+# ---- the integer branch of dequantize_gemv (int8 activations, int32 accumulation) --------------------------------
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (3, 520, 2048), (64, 256, 1024)])
+@pytest.mark.parametrize("bits,fast,fmt", [(2, False, "uint"), (2, True, "int"), (2, True, "uint"), (4, False, "int")])
+def test_dequantize_gemv_int8_exact(cuda, M, N, K, bits, fast, fmt):
+    """use_dp4a branch of the example (example_dequant_gemv_fp16xint4.py:47-48,126-133): exact int32."""
+    rng = np.random.default_rng(M + N + K + bits)
+    A = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    packed = _packed(N, K, bits, seed=bits + int(fast))
+    if bits == 2:
+        conv = "twos" if not fast else ("offset" if fmt == "int" else "unsigned")
+        W = orc.decode_i2(packed, conv).astype(np.int64)
+        B = orc.interleave_weight(packed.view(np.int8), 2, "int8").view(np.uint8) if fast else packed
+    else:
+        W = orc.decode_i4_signed(packed).astype(np.int64)
+        B = packed
+    kernel = tl.dequantize_gemv(M, N, K, "int8", "int32", "int32", num_bits=bits, source_format=fmt, fast_decoding=fast)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    kernel(torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda), C)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), A.astype(np.int64) @ W.T)

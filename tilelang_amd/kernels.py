@@ -87,6 +87,10 @@ def dequantize_gemv(
     ``with_zeros`` ``kernel(A, B, Scale, Zeros, C)``, ``Scale``/``Zeros`` fp16
     ``[N, K // group_size]``.
 
+    ``num_bits`` 2 and 1 (``B[N, K * num_bits / 8]``) and ``in_dtype="int8"`` with int32 accumulation and output
+    (the example's ``use_dp4a`` branch) are served by their own kernels, see ``_dequantize_gemv_lowbit`` and
+    ``_dequantize_gemv_int8``; what follows describes the fp16 x 4-bit case.
+
     ``fast_decoding=True`` means, as in the example, that B was passed through
     ``interleave_weight(B, 4, "float16")``; otherwise B is the plain low-nibble-first
     layout.  Accumulation is always fp32.  ``source_format="int"`` with scaling is the
@@ -96,8 +100,11 @@ def dequantize_gemv(
     assert trans_B is True, "Dequantize only implement for trans_B=TRue currently"
     if num_bits not in (1, 2, 4):
         raise ValueError("dequantize_gemv: num_bits must be 4, 2 or 1")
+    if _dtype(in_dtype) == torch.int8:
+        return _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dtype, source_format, fast_decoding,
+                                     with_scaling, with_zeros, _formula_fast)
     if _dtype(in_dtype) != torch.float16 or _dtype(out_dtype) != torch.float16:
-        raise ValueError("dequantize_gemv: in_dtype and out_dtype must be float16 (int8 x int2: bitnet_158_int8xint2_decode)")
+        raise ValueError("dequantize_gemv: in_dtype must be float16 (with float16 out) or int8 (with int32 out)")
     if _dtype(storage_dtype) not in (torch.int8, torch.uint8):
         raise ValueError("dequantize_gemv: storage_dtype must be int8 or uint8")
     if num_bits < 4:
@@ -133,6 +140,41 @@ def dequantize_gemv(
         c = ptrs[-1]
         return lib.call_dequantize_gemv_w4a16(a, b, s, z, c, M, N, K, group_size, mode, layout, variant, stream)
 
+    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
+
+
+def _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dtype, source_format, fast_decoding,
+                          with_scaling, with_zeros, _formula_fast) -> KernelAdapter:
+    """The integer branch of :func:`dequantize_gemv` (``use_dp4a``: int8 activations, int32 accumulation,
+    examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:47-48,126-133): ``C[M,N] int32 = A[M,K] int8 .
+    decode(B)^T``, exact.  Two bits: every decoder and the ``interleave_weight(B, 2, "int8")`` layout of the fast path
+    (the BitNet decode kernel is this case); four bits: the slow path (two's-complement nibbles)."""
+    if _dtype(accum_dtype) != torch.int32 or _dtype(out_dtype) != torch.int32:
+        raise ValueError("dequantize_gemv: int8 activations accumulate and return int32")
+    if with_scaling or with_zeros:
+        raise ValueError("dequantize_gemv: the integer branch has no scales or zeros")
+    if K % 128 != 0:
+        raise ValueError(f"dequantize_gemv: K={K} must be a multiple of 128")
+    params = [KernelParam("A", torch.int8, (M, K)),
+              KernelParam("B", _dtype(storage_dtype), (N, K * num_bits // 8), packed=True),
+              KernelParam("C", torch.int32, (M, N))]
+    formula_fast = fast_decoding if _formula_fast is None else _formula_fast
+    if num_bits == 2:
+        conv = I2_TWOS if not formula_fast else (I2_OFFSET if source_format == "int" else I2_UNSIGNED)
+        layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
+
+        def launch(ptrs, stream):
+            return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, layout, None, 1.0, 0, stream)
+
+    elif num_bits == 4:
+        if fast_decoding:
+            raise ValueError("dequantize_gemv: int8 x int4 is built for the slow path only (fast_decoding=False)")
+
+        def launch(ptrs, stream):
+            return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, 1, 0, 0, stream)
+
+    else:
+        raise ValueError("dequantize_gemv: int8 activations are built for num_bits 4 and 2")
     return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
 
 
