@@ -77,19 +77,25 @@ def _copies(nbytes, min_total=640 << 20, lo=2, hi=24):
     return int(min(hi, max(lo, -(-min_total // max(nbytes, 1)))))
 
 
-def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev):
+def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False):
     group = 128
     d = workloads.w4a16(M, N, K, group, seed=0, scale_range=(0.002, 0.01) if zeros else (0.005, 0.02),
                         zeros_range=(6, 10) if zeros else None)
     nbytes = workloads.w4a16_bytes(M, N, K, group, zeros=zeros)
     nc = _copies(nbytes)
     A = torch.from_numpy(d["A"]).to(dev)
-    Bs = [torch.from_numpy(d["B"]).to(dev).view(torch.int8).clone() for _ in range(nc)]
+    b0 = torch.from_numpy(d["B"]).view(torch.int8)
+    if interleaved:
+        # the word permutation the example applies before its fast decoder (example_dequant_gemv_fp16xint4.py:201-204)
+        from tilelang_amd import quantize
+
+        b0 = quantize.interleave_weight(b0, 4, "float16")
+    Bs = [b0.to(dev).clone() for _ in range(nc)]
     Ss = [torch.from_numpy(d["Scale"]).to(dev).clone() for _ in range(nc)]
     Zs = [torch.from_numpy(d["Zeros"]).to(dev).clone() for _ in range(nc)] if zeros else None
     C = torch.empty((M, N), dtype=torch.float16, device=dev)
     kern = tl.dequantize_gemv(M, N, K, group_size=group, source_format="uint" if zeros else "int",
-                              with_scaling=True, with_zeros=zeros)
+                              with_scaling=True, with_zeros=zeros, fast_decoding=interleaved)
     if zeros:
         fns = [(lambda i=i: kern(A, Bs[i], Ss[i], Zs[i], C, skip_tensor_validation=True)) for i in range(nc)]
     else:
@@ -348,6 +354,8 @@ def main():
         shapes.append(_row("bitnet_w2a8 M=2048 N=8192 K=8192 (plain packing, not interleaved)", r, "mfma", MFMA_I8_PEAK))
         r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, max(5, k // 4), 2, dev)
         shapes.append(_row("w4a16_zeros_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
+        r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, max(5, k // 4), 2, dev, interleaved=True)
+        shapes.append(_row("w4a16_zeros_gemm M=4096 N=8192 K=8192 (interleaved words, the example's fast-decode layout)", r, "mfma", MFMA_BF16_PEAK))
         r = bench_mxfp4_quant(torch, tl, 8192, 8192, k, 2, dev)
         shapes.append(_row("mxfp4_quantize N=8192 K=8192", r, "hbm", MFMA_BF16_PEAK))
         r = bench_activation_quant(torch, tl, 2048, 8192, k, 2, dev)
