@@ -367,6 +367,14 @@ def main():
         r = bench_mxfp4_blockscaled(torch, tl, workloads, 4096, 8192, 8192, kg, 2, dev)
         shapes.append(_row("mxfp4_x_mxfp4_blockscaled_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_FP4_PEAK))
 
+    # the metric's second half: the M=4096 MXFP4-weight GEMM against the dense bf16 MFMA peak
+    roof_gemm = None
+    for row in shapes:
+        if row["config"].startswith("mxfp4_gemm M=4096"):
+            roof_gemm = {"bound": "mfma", "achieved": row["TFLOP/s"], "peak": MFMA_BF16_PEAK / 1e12, "unit": "TFLOP/s",
+                         "frac": row["frac"], "us": row["us"], "kernel": "gemm_kernel_dma<MxPolicy<e2m1>,4,4>",
+                         "workload": "A bf16 [4096,8192] x e2m1 [8192,8192] with e8m0 scales per 32, bf16 out",
+                         "algorithmic_flops": 2 * 4096 * 8192 * 8192}
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline_w4a16(N, K, rows=N)
@@ -387,6 +395,7 @@ def main():
         "config": {"workload": "W4A16 decode GEMV M=1 N=28672 K=8192 group=128 w=(q-8)*s, fp32 accumulate, fp16 out",
                    "weights_rotated_over_copies": _copies(head["bytes"]), "timed_with": "hip graph replay" if head["graph"] else "direct launches"},
         "roofline": roof,
+        "roofline_gemm": roof_gemm,
         "cpu_baseline": cpu,
         "shapes": shapes,
     }
