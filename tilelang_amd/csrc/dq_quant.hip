@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void mxfp4_quant_kernel(const uint4_t* __restr
       const uint32_t nonzero = ((packed & 0x77777777u) + 0x77777777u) & 0x88888888u;
       packed &= nonzero | 0x77777777u;
       if (p < pieces) {
-        B[p] = packed;
+        __builtin_nontemporal_store(packed, &B[p]);  // written once, read by a later kernel: kept out of the L2
         if ((threadIdx.x & 3) == 0) S[p >> 2] = (uint8_t)byte;
       }
     }
