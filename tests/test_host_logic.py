@@ -84,6 +84,21 @@ def test_entry_points_reject_bad_arguments_before_any_launch():
     assert "at least 256" in lib.get_last_error().decode()
     assert lib.call_gemm_mxfp4_mxfp4(a, a, a, vp(a.value + 2), vp(0), a, 64, 64, 256, vp(0)) == -1
     assert "4-byte aligned" in lib.get_last_error().decode()
+    # low-bit GEMV: (A, B, Scale, Zeros, C, M, N, K, group, bits, convention, layout, zeros_rescale, stream)
+    assert lib.call_dequantize_gemv_lowbit(a, a, vp(0), vp(0), a, 1, 64, 256, 256, 3, 0, 0, 0, vp(0)) == -1
+    assert "bits must be 1 or 2" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_lowbit(a, vp(0), vp(0), vp(0), a, 1, 64, 256, 256, 2, 0, 0, 0, vp(0)) == -1
+    assert "B is expected to have non-NULL" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_lowbit(a, a, vp(0), vp(0), a, 65, 64, 256, 256, 2, 0, 0, 0, vp(0)) == -1
+    assert "decode batch" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_lowbit(a, a, vp(0), vp(0), a, 1, 64, 192, 192, 1, 0, 0, 0, vp(0)) == -1
+    assert "multiple of 128" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_lowbit(a, a, a, vp(0), a, 1, 64, 256, 32, 2, 0, 0, 0, vp(0)) == -1
+    assert "group" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_lowbit(a, a, vp(0), a, a, 1, 64, 256, 256, 2, 0, 0, 0, vp(0)) == -1
+    assert "Zeros without Scale" in lib.get_last_error().decode()
+    assert lib.call_dequantize_gemv_lowbit(a, a, vp(0), vp(0), a, 1, 64, 256, 256, 2, 4, 0, 0, vp(0)) == -1
+    assert "unknown code convention" in lib.get_last_error().decode()
 
 
 def test_bitlinear_weight_packing_matches_oracle():
