@@ -33,6 +33,12 @@ scale rule is the OCP Microscaling v1.0 conversion and only the element rule
 is pinned by closed forms instead (exact powers of two, round trip through ``mxfp4_dequant``,
 idempotence, the block maximum always landing in e2m1's top binade).  ``gen_quant4_quantize`` is
 pinned by its closed form (absmax scale, rint, clamp) against torch's own ops on the CPU.
+``dequant_lowbit`` (2-bit / 1-bit codes to fp16): the unscaled decoders are pinned over all 65536 / 256 inputs of
+``fast_decode_i2_to_f16`` / ``fast_decode_i1_to_f16`` (examples/dequantize_gemm/quantize/lop3.py:424-463, 679-746)
+against closed forms, through the interleave, and by the reference's sign-extension known answers; the rounding order
+of its scaled and zero-point forms (lop3.py:465-636, 748-891) has no caller, test or fixture in the reference: parity
+unpinned, contract = the operation order of the device snippets, checked against float64 arithmetic with explicit
+roundings on values where the orders differ.
 """
 
 from __future__ import annotations
