@@ -27,57 +27,79 @@ HBM_PEAK = 8.0e12        # B/s
 MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense
 MFMA_I8_PEAK = 5.0e15    # OP/s dense
 MFMA_FP4_PEAK = 10.1e15  # FLOP/s dense, block-scaled fp4
-# HBM bytes per launch of the headline GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
-# same counters read for a plain 128 MiB copy kernel (59240.5 x 2 KiB read + 56 KiB written)
-GEMV_HBM_TRAFFIC = 121381888
+# HBM bytes per launch of the headline GEMV: not measured by this script (counters need the profiler) but quoted
+# from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary, scaled there by what the same counters read
+# for a plain 128 MiB copy kernel.  Re-measure and update all three fields whenever the kernel changes.
+GEMV_HBM_TRAFFIC = {"bytes": 121381888, "kernel": "w4a16_gemv_kernel<1,1,4,scale,g128,wide>",
+                    "source": "profiles/bench_all_configs_hbm_traffic.md"}
 
 
-def _time_launches(torch, fns, steps, warmup):
-    """Average device time per call of fns[i % len(fns)] over `steps` calls.
+def _time_launches(torch, fns, steps, warmup, min_launches=120, max_launches=None, settle_ms=50.0, replays=30):
+    """Median device time per call of fns[i % len(fns)], independent of `steps`.
 
-    The launches are captured into one HIP graph (the kernels are microseconds long; replaying a
-    graph keeps the host out of the measurement) and the replay is bracketed by events on the
-    stream it runs on.  Falls back to plain back-to-back launches if capture is refused.
+    `steps` launches (repeated for whole rounds until the graph holds at least `min_launches`) are captured
+    into one HIP graph: the kernels are microseconds long and replaying a graph keeps the host out of the
+    measurement.  The graph is replayed untimed until `settle_ms` of device time have passed, so the clocks
+    have ramped, then `replays` times with an event pair of its own around every replay, all on the stream
+    the kernels run on (per-iteration events as in tilelang/profiler/bench.py:172-272).  Returns the median
+    over the replays of (replay time / launches in the graph), with the minimum and the mean beside it.
+    Falls back to plain back-to-back launches if capture is refused.
     """
     for i in range(max(warmup, len(fns))):
         fns[i % len(fns)]()
     torch.cuda.synchronize()
+    rounds = max(1, -(-min_launches // max(steps, 1)))
+    launches = steps * rounds
+    if max_launches is not None:
+        launches = min(launches, max_launches)
     stream = torch.cuda.Stream()
     graph = None
     try:
         with torch.cuda.stream(stream):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
-                for i in range(steps):
+                for i in range(launches):
                     fns[i % len(fns)]()
             graph = g
     except Exception as exc:  # pragma: no cover - depends on the runtime
         print(f"[bench] graph capture refused ({exc}); timing direct launches", file=sys.stderr)
         torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with torch.cuda.stream(stream):
+
+    def once():
         if graph is not None:
-            for _ in range(10):  # untimed replays: warm the instantiated graph and let the clocks settle
-                graph.replay()
-            stream.synchronize()
-            e0.record(stream)
             graph.replay()
-            e1.record(stream)
         else:
-            e0.record(stream)
-            for i in range(steps):
+            for i in range(launches):
                 fns[i % len(fns)]()
-            e1.record(stream)
-    e1.synchronize()
+
+    with torch.cuda.stream(stream):
+        settled, n_settle = 0.0, 0
+        while settled < settle_ms and n_settle < 10000:
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            once()
+            b.record(stream)
+            b.synchronize()
+            settled += a.elapsed_time(b)
+            n_settle += 1
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(replays)]
+        for a, b in pairs:
+            a.record(stream)
+            once()
+            b.record(stream)
+        stream.synchronize()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps, graph is not None
+    per = sorted(a.elapsed_time(b) / launches for a, b in pairs)
+    stats = {"graph": graph is not None, "launches_per_replay": launches, "replays": replays,
+             "us_min": per[0] * 1e3, "us_mean": sum(per) / len(per) * 1e3, "settle_replays": n_settle}
+    return float(np.median(per)), stats
 
 
 def _copies(nbytes, min_total=640 << 20, lo=2, hi=24):
     return int(min(hi, max(lo, -(-min_total // max(nbytes, 1)))))
 
 
-def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False):
+def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False, **tk):
     group = 128
     d = workloads.w4a16(M, N, K, group, seed=0, scale_range=(0.002, 0.01) if zeros else (0.005, 0.02),
                         zeros_range=(6, 10) if zeros else None)
@@ -100,12 +122,12 @@ def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interl
         fns = [(lambda i=i: kern(A, Bs[i], Ss[i], Zs[i], C, skip_tensor_validation=True)) for i in range(nc)]
     else:
         fns = [(lambda i=i: kern(A, Bs[i], Ss[i], C, skip_tensor_validation=True)) for i in range(nc)]
-    ms, graphed = _time_launches(torch, fns, steps, warmup)
-    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed,
+    ms, graphed = _time_launches(torch, fns, steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed,
             "inputs": d, "out": C}
 
 
-def bench_w2a16(torch, tl, M, N, K, steps, warmup, dev, fast=True):
+def bench_w2a16(torch, tl, M, N, K, steps, warmup, dev, fast=True, **tk):
     """The 2-bit case of dequantize_gemv: codes uniform over 0..3 (interleaved words, w = (c - 2) * s), group 128."""
     from tilelang_amd import quantize
 
@@ -122,11 +144,11 @@ def bench_w2a16(torch, tl, M, N, K, steps, warmup, dev, fast=True):
     C = torch.empty((M, N), dtype=torch.float16, device=dev)
     kern = tl.dequantize_gemv(M, N, K, num_bits=2, source_format="int", fast_decoding=fast, group_size=group, with_scaling=True)
     fns = [(lambda i=i: kern(A, Bs[i], Ss[i], C, skip_tensor_validation=True)) for i in range(nc)]
-    ms, graphed = _time_launches(torch, fns, steps, warmup)
-    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * M * N * K, "graph": graphed}
+    ms, graphed = _time_launches(torch, fns, steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * M * N * K, "timing": graphed}
 
 
-def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev):
+def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev, **tk):
     d = workloads.mxfp4(M, N, K, seed=0, scale_bias=127)
     A = torch.from_numpy(d["A"]).to(dev).view(torch.bfloat16)
     nc = 3
@@ -141,11 +163,11 @@ def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev):
             out[0] = kern(A, Bs[i], S, bias, skip_tensor_validation=True)
         return f
 
-    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
-    return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "graph": graphed}
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
-def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev):
+def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev, **tk):
     """Both operands MXFP4 (e2m1 codes + one E8M0 byte per 32 k), block-scaled matrix instruction."""
     d = workloads.mxfp4_mxfp4(M, N, K, seed=0)
     nbytes = workloads.mxfp4_mxfp4_bytes(M, N, K)
@@ -163,11 +185,11 @@ def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev):
             out[0] = kern(A, Bs[i], SA, SBs[i], bias, skip_tensor_validation=True)
         return f
 
-    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
-    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
-def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True):
+def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True, **tk):
     """BitLinear forward on quantised operands: int8 x 2-bit (offset-binary ternary), fused acc/s_a/s_w epilogue.
 
     ``interleaved``: the packed words went through ``interleave_weight(qw, 2, "int8")`` on the host, once, as in
@@ -190,11 +212,11 @@ def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=
             out[0] = kern(A, Bs[i], s_a, skip_tensor_validation=True)
         return f
 
-    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
-    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
-def bench_activation_quant(torch, tl, M, K, steps, warmup, dev):
+def bench_activation_quant(torch, tl, M, K, steps, warmup, dev, **tk):
     """BitLinear activation quantiser (fp16 rows -> int8 + fp32 scale), the step before the W2A8 GEMM."""
     nc = _copies(3 * M * K, hi=12)
     gen = torch.Generator(device="cpu").manual_seed(0)
@@ -207,11 +229,11 @@ def bench_activation_quant(torch, tl, M, K, steps, warmup, dev):
             out[0] = kern(xs[i], skip_tensor_validation=True)
         return f
 
-    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
-    return {"us": ms * 1e3, "bytes": 3 * M * K + 4 * M, "flops": 2 * M * K, "graph": graphed}
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": 3 * M * K + 4 * M, "flops": 2 * M * K, "timing": graphed}
 
 
-def bench_mxfp4_quant(torch, tl, N, K, steps, warmup, dev):
+def bench_mxfp4_quant(torch, tl, N, K, steps, warmup, dev, **tk):
     """MXFP4 weight quantiser (bf16 -> e2m1 codes + one scale byte per 32), the producer of the GEMM's B and Scale."""
     nbytes = 2 * N * K + N * K // 2 + N * K // 32
     nc = _copies(nbytes, hi=6)
@@ -225,11 +247,11 @@ def bench_mxfp4_quant(torch, tl, N, K, steps, warmup, dev):
             out[0] = kern(ws[i], skip_tensor_validation=True)
         return f
 
-    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup)
-    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * N * K, "graph": graphed}
+    ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * N * K, "timing": graphed}
 
 
-def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev):
+def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev, **tk):
     """W4A8 (int8 x int4, Ct[N,M] int32) or int4 x int4 (C[M,N] int32), exact."""
     if a_packed:
         from tilelang_amd import quantize
@@ -250,43 +272,95 @@ def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev):
     def f():
         out[0] = kern(A, B, skip_tensor_validation=True)
 
-    ms, graphed = _time_launches(torch, [f], steps, warmup)
-    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "graph": graphed}
+    ms, graphed = _time_launches(torch, [f], steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
 def _row(config, r, bound, peak):
     sec = r["us"] * 1e-6
-    row = {"config": config, "us": r["us"], "GB/s": r["bytes"] / sec / 1e9, "TFLOP/s": r["flops"] / sec / 1e12, "bound": bound}
+    row = {"config": config, "us": r["us"], "us_min": r["timing"]["us_min"], "GB/s": r["bytes"] / sec / 1e9, "TFLOP/s": r["flops"] / sec / 1e12, "bound": bound}
     row["frac"] = (r["bytes"] / sec / HBM_PEAK) if bound == "hbm" else (r["flops"] / sec / peak)
     return row
 
 
-def cpu_baseline_w4a16(N, K, rows, budget_s=12.0, max_runs=40):
-    """torch-CPU ref_program on the first `rows` weight rows of the headline shape (all of them by default),
-    repeated for about `budget_s` seconds; the median run, extrapolated to N rows when rows < N."""
+def _median_time(fn, budget_s, min_runs=3, max_runs=25):
+    fn()  # warm-up
+    times, t_start = [], time.perf_counter()
+    while len(times) < max_runs and (len(times) < min_runs or time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return float(np.median(times)), len(times)
+
+
+def cpu_baselines(budget_s=16.0):
+    """The reference's ``ref_program`` of every benchmark configuration restated in torch, on CPU tensors and all
+    host cores: dequantise and matmul timed separately (median of at least 3 runs each).  Configurations whose
+    CPU time is seconds are timed on the first rows of the weight matrix and scaled; `sample` says which.
+    Returns (headline entry, per-configuration list)."""
     import torch
 
     from oracle import ref_torch
     from tilelang_amd import workloads
 
     torch.set_num_threads(os.cpu_count() or 1)
-    d = workloads.w4a16(1, rows, K, 128, seed=0)
-    A, B, S = torch.from_numpy(d["A"]), torch.from_numpy(d["B"]), torch.from_numpy(d["Scale"])
-    ref_torch.ref_w4a16(A, B, S)  # warm-up
-    times, t_start = [], time.perf_counter()
-    while len(times) < max_runs and (len(times) < 5 or time.perf_counter() - t_start < budget_s):
-        t0 = time.perf_counter()
-        ref_torch.ref_w4a16(A, B, S)
-        times.append(time.perf_counter() - t0)
-    med = float(np.median(times))
-    return {
-        "value": med * (N / rows) * 1e6,
-        "unit": "us",
-        "cores": torch.get_num_threads(),
-        "kind": "port",
-        "sample": f"torch-CPU ref_program (unpack, (q-8)*s in fp16, fp32 matmul) on the first {rows} of {N} weight rows, "
-                  f"K={K}, median of {len(times)} runs x {N / rows:.0f}",
+    cores = torch.get_num_threads()
+    rows_out = []
+
+    def leg(name, n_full, n_rows, make, dequant, matmul, share):
+        d = make(n_rows)
+        t_deq, r1 = _median_time(lambda: dequant(d), share / 2)
+        W = dequant(d)
+        t_mm, r2 = _median_time(lambda: matmul(d, W), share / 2)
+        f = n_full / n_rows
+        rows_out.append({"config": name, "dequant_us": t_deq * f * 1e6, "matmul_us": t_mm * f * 1e6,
+                         "us": (t_deq + t_mm) * f * 1e6, "cores": cores,
+                         "sample": (f"all {n_full} weight rows" if n_rows == n_full else
+                                    f"first {n_rows} of {n_full} weight rows x {f:.0f}") + f", median of {r1}/{r2} runs"})
+        return rows_out[-1]
+
+    def w4(M, N, K, zeros, rows, share, tag):
+        def make(n):
+            d = workloads.w4a16(M, n, K, 128, seed=0, scale_range=(0.002, 0.01) if zeros else (0.005, 0.02),
+                                zeros_range=(6, 10) if zeros else None)
+            return {k: torch.from_numpy(v) for k, v in d.items()}
+        return leg(f"{tag} M={M} N={N} K={K}", N, rows, make,
+                   lambda d: ref_torch.dequant_w4a16(d["B"], d["Scale"], d.get("Zeros")),
+                   lambda d, W: ref_torch.matmul_f32(d["A"], W, torch.half), share)
+
+    unit = budget_s / 24.0
+    w4(1, 1024, 1024, False, 1024, 0.5 * unit, "w4a16_gemv (the CPU-path configuration)")
+    head = w4(1, 28672, 8192, False, 28672, 4 * unit, "w4a16_gemv")
+    for (n, k) in [(11008, 4096), (4096, 11008), (4096, 4096)]:
+        w4(1, n, k, False, n, 1 * unit, "w4a16_gemv")
+    for m in (4, 16, 64):
+        w4(m, 28672, 8192, True, 28672, 2 * unit, "w4a16_zeros")
+
+    def mx_make(n):
+        d = workloads.mxfp4(4096, n, 8192, seed=0, scale_bias=127)
+        return {"A": torch.from_numpy(d["A"]).view(torch.bfloat16), "B": torch.from_numpy(d["B"]), "Scale": torch.from_numpy(d["Scale"])}
+    leg("mxfp4_gemm M=4096 N=8192 K=8192", 8192, 1024, mx_make,
+        lambda d: ref_torch.dequant_mxfp4_e2m1(d["B"], d["Scale"], 127),
+        lambda d, W: ref_torch.matmul_f32(d["A"], W, torch.bfloat16), 3 * unit)
+
+    for m, rows in ((1, 8192), (256, 8192), (2048, 2048)):
+        def bn_make(n, m=m):
+            d = workloads.bitnet(m, n, 8192, seed=0)
+            return {"A": torch.from_numpy(d["A"]), "B": torch.from_numpy(d["B"]),
+                    "s_a": torch.from_numpy(np.asarray(d["s_a"], dtype=np.float32)), "s_w": float(d["s_w"])}
+        leg(f"bitnet_w2a8 M={m} N=8192 K=8192", 8192, rows, bn_make,
+            lambda d: ref_torch.dequant_bitnet(d["B"]),
+            lambda d, W: ref_torch.bitnet_epilogue(torch.matmul(d["A"].float(), W.T), d["s_a"], d["s_w"]), 2 * unit)
+
+    cpu = {
+        "value": head["us"], "unit": "us", "cores": cores, "kind": "port",
+        "dequant_us": head["dequant_us"], "matmul_us": head["matmul_us"],
+        "sample": "torch-CPU ref_program (unpack, (q-8)*s in fp16; fp32 matmul) of the headline GEMV, " + head["sample"],
+        "note": "the reference's other CPU path, TileLang's LLVM CPU backend, cannot be built here (it needs the TVM "
+                "submodule and LLVM, both absent), so the baseline is the torch restatement of ref_program only",
+        "configs": rows_out,
     }
+    return cpu
 
 
 def main():
@@ -316,11 +390,14 @@ def main():
 
     # ---- headline: M=1 W4A16 GEMV at N=28672, K=8192 ------------------------------------------
     M, N, K = 1, 28672, 8192
-    head = bench_w4a16(torch, tl, workloads, M, N, K, False, args.steps, args.warmup, dev)
+    S, W = args.steps, args.warmup
+    head = bench_w4a16(torch, tl, workloads, M, N, K, False, S, W, dev)
     us = head["us"]
     gbs = head["bytes"] / (us * 1e-6) / 1e9
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": gbs * 1e9 / HBM_PEAK,
-            "traffic": GEMV_HBM_TRAFFIC, "kernel": "w4a16_gemv_kernel<1,1,4,scale,g128,wide>", "algorithmic_bytes": head["bytes"]}
+            "traffic": GEMV_HBM_TRAFFIC["bytes"], "traffic_source": GEMV_HBM_TRAFFIC["source"],
+            "kernel": GEMV_HBM_TRAFFIC["kernel"], "algorithmic_bytes": head["bytes"],
+            "us_min": head["timing"]["us_min"], "us_mean": head["timing"]["us_mean"]}
 
     if args.copy_calibration:
         src = torch.full((128 << 20,), 3, dtype=torch.uint8, device=dev).view(torch.int32)
@@ -332,40 +409,42 @@ def main():
 
     shapes = []
     if not args.headline_only:
-        k = max(10, args.steps // 3)
+        gemm = {"min_launches": 24, "max_launches": 48}  # launches of hundreds of microseconds: a replay is milliseconds
         for (m, n, kk) in [(1, 1024, 1024), (1, 11008, 4096), (1, 4096, 11008), (1, 4096, 4096)]:
-            r = bench_w4a16(torch, tl, workloads, m, n, kk, False, k, 4, dev)
-            shapes.append({"config": f"w4a16_gemv M={m} N={n} K={kk}", "us": r["us"], "GB/s": r["bytes"] / r["us"] / 1e3,
-                           "TFLOP/s": r["flops"] / r["us"] / 1e6, "bound": "hbm", "frac": r["bytes"] / (r["us"] * 1e-6) / HBM_PEAK})
+            r = bench_w4a16(torch, tl, workloads, m, n, kk, False, S, W, dev)
+            shapes.append(_row(f"w4a16_gemv M={m} N={n} K={kk}", r, "hbm", MFMA_BF16_PEAK))
         for m in (4, 16, 64):
-            r = bench_w4a16(torch, tl, workloads, m, 28672, 8192, True, k, 4, dev)
-            shapes.append({"config": f"w4a16_zeros M={m} N=28672 K=8192", "us": r["us"], "GB/s": r["bytes"] / r["us"] / 1e3,
-                           "TFLOP/s": r["flops"] / r["us"] / 1e6, "bound": "hbm", "frac": r["bytes"] / (r["us"] * 1e-6) / HBM_PEAK,
-                           "frac_mfma": r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK})
-        r = bench_w2a16(torch, tl, 1, 28672, 8192, k, 4, dev)
+            r = bench_w4a16(torch, tl, workloads, m, 28672, 8192, True, S, W, dev)
+            row = _row(f"w4a16_zeros M={m} N=28672 K=8192", r, "hbm", MFMA_BF16_PEAK)
+            row["frac_mfma"] = r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK
+            shapes.append(row)
+        r = bench_w2a16(torch, tl, 1, 28672, 8192, S, W, dev)
         shapes.append(_row("w2a16_gemv M=1 N=28672 K=8192 (num_bits=2, interleaved words, (c-2)*s)", r, "hbm", MFMA_BF16_PEAK))
-        kg = max(6, args.steps // 10)
-        r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, kg, 2, dev)
+        r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
         for m in (1, 256, 2048):
-            r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, k if m == 1 else kg, 2, dev)
+            r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m == 1 else gemm))
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
-        r = bench_bitnet(torch, tl, workloads, 2048, 8192, 8192, kg, 2, dev, interleaved=False)
+        r = bench_bitnet(torch, tl, workloads, 2048, 8192, 8192, S, W, dev, interleaved=False, **gemm)
         shapes.append(_row("bitnet_w2a8 M=2048 N=8192 K=8192 (plain packing, not interleaved)", r, "mfma", MFMA_I8_PEAK))
-        r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, max(5, k // 4), 2, dev)
+        r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, S, W, dev, **gemm)
         shapes.append(_row("w4a16_zeros_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
-        r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, max(5, k // 4), 2, dev, interleaved=True)
+        r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, S, W, dev, interleaved=True, **gemm)
         shapes.append(_row("w4a16_zeros_gemm M=4096 N=8192 K=8192 (interleaved words, the example's fast-decode layout)", r, "mfma", MFMA_BF16_PEAK))
-        r = bench_mxfp4_quant(torch, tl, 8192, 8192, k, 2, dev)
+        r = bench_mxfp4_quant(torch, tl, 8192, 8192, S, W, dev, **gemm)
         shapes.append(_row("mxfp4_quantize N=8192 K=8192", r, "hbm", MFMA_BF16_PEAK))
-        r = bench_activation_quant(torch, tl, 2048, 8192, k, 2, dev)
+        r = bench_activation_quant(torch, tl, 2048, 8192, S, W, dev)
         shapes.append(_row("bitnet_activation_quant M=2048 K=8192", r, "hbm", MFMA_I8_PEAK))
-        r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, False, kg, 2, dev)
+        r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, False, S, W, dev, **gemm)
         shapes.append(_row("w4a8_gemm M=4096 N=4096 K=4096 (Ct int32)", r, "mfma", MFMA_I8_PEAK))
-        r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, True, kg, 2, dev)
+        r = bench_int4(torch, tl, workloads, 4096, 4096, 4096, True, S, W, dev, **gemm)
         shapes.append(_row("int4xint4_gemm M=4096 N=4096 K=4096", r, "mfma", MFMA_I8_PEAK))
-        r = bench_mxfp4_blockscaled(torch, tl, workloads, 4096, 8192, 8192, kg, 2, dev)
+        r = bench_mxfp4_blockscaled(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
         shapes.append(_row("mxfp4_x_mxfp4_blockscaled_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_FP4_PEAK))
+        # what a launch costs before any byte moves: the same timing of the smallest problem the library takes
+        r = bench_w4a16(torch, tl, workloads, 1, 16, 1024, False, S, W, dev)
+        shapes.append({"config": "launch floor: w4a16_gemv M=1 N=16 K=1024 (back-to-back launches in a graph, 10 KB of work)",
+                       "us": r["us"], "us_min": r["timing"]["us_min"], "bound": "launch"})
 
     # the metric's second half: the M=4096 MXFP4-weight GEMM against the dense bf16 MFMA peak
     roof_gemm = None
@@ -377,7 +456,7 @@ def main():
                          "algorithmic_flops": 2 * 4096 * 8192 * 8192}
     cpu = None
     if not args.no_cpu:
-        cpu = cpu_baseline_w4a16(N, K, rows=N)
+        cpu = cpu_baselines()
 
     line = {
         "metric": "M=1 W4A16 GEMV us + %HBM peak; M=4096 dequant GEMM TFLOP/s + %MFMA peak",
@@ -393,7 +472,9 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "W4A16 decode GEMV M=1 N=28672 K=8192 group=128 w=(q-8)*s, fp32 accumulate, fp16 out",
-                   "weights_rotated_over_copies": _copies(head["bytes"]), "timed_with": "hip graph replay" if head["graph"] else "direct launches"},
+                   "weights_rotated_over_copies": _copies(head["bytes"]), "timed_with": ("hip graph replay" if head["timing"]["graph"] else "direct launches")
+                   + f", median of {head['timing']['replays']} event-bracketed replays of {head['timing']['launches_per_replay']} launches"
+                     f" after {head['timing']['settle_replays']} untimed replays (at least 50 ms)"},
         "roofline": roof,
         "roofline_gemm": roof_gemm,
         "cpu_baseline": cpu,
