@@ -216,6 +216,39 @@ def test_full_size_linearity(cuda):
     np.testing.assert_allclose(outs[0][:, rows], ref.astype(np.float32), rtol=RTOL, atol=ATOL)
 
 
+@pytest.fixture(scope="module")
+def cfg3_full_size():
+    """Configuration 3 at its full size, N = 28672, K = 8192, with the oracle's tile over ALL weight rows."""
+    M, N, K, group = 64, 28672, 8192, 128
+    d = workloads.w4a16(M, N, K, group, seed=7, scale_range=(0.002, 0.01), zeros_range=(6, 10))
+    W = orc.dequant_u4_scale_zeros(d["B"], d["Scale"], d["Zeros"], group, "original").astype(np.float32)
+    return d, W
+
+
+@pytest.mark.parametrize("M", [4, 16, 64])
+def test_small_batch_full_size_default_dispatch(cuda, cfg3_full_size, M):
+    """Configuration 3 as the benchmark runs it: M in {4, 16, 64}, N = 28672, K = 8192, (q - z) * s with zeros 6..10,
+    the library's own choice of kernel (variant = -1), every output against the oracle; and the kernel is linear in A."""
+    d, W = cfg3_full_size
+    N, K, group = 28672, 8192, 128
+    print(f"cfg3 full size, default dispatch: M={M} N={N} K={K}", flush=True)
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, source_format="uint",
+                              with_scaling=True, with_zeros=True, zeros_mode="original")
+    Bd, Sd, Zd = _dev(d["B"], cuda).view(torch.int8), _dev(d["Scale"], cuda), _dev(d["Zeros"], cuda)
+    A1 = d["A"][:M]
+    A2 = np.random.default_rng(8).standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    outs = []
+    for a in (A1, A2, (A1.astype(np.float32) + A2.astype(np.float32)).astype(np.float16)):
+        C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+        kern(_dev(a, cuda), Bd, Sd, Zd, C)
+        torch.cuda.synchronize()
+        outs.append(C.float().cpu().numpy())
+    ref = (A1.astype(np.float32) @ W.T).astype(np.float16).astype(np.float32)
+    assert np.isfinite(outs[0]).all()
+    np.testing.assert_allclose(outs[0], ref, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(outs[2], outs[0] + outs[1], rtol=2e-2, atol=5e-2)
+
+
 def test_null_pointer_and_bad_args(cuda):
     kern = tl.dequantize_gemv(1, 64, 256, group_size=128, source_format="int", with_scaling=True)
     A = torch.zeros((1, 256), dtype=torch.float16, device=cuda)
