@@ -106,6 +106,18 @@ int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int
 int call_dequant_gemm_fp16_fp4_splitk(const void* A, const void* B, void* SplitC, void* C, int M, int N, int K,
                                       int split, int transposed, dq_stream_t stream);
 
+/* The same split-K product for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose SplitC is allocated
+ * inside the kernel function.  The partial results live in a buffer of DQ_STATIC_SCRATCH_BYTES that the library
+ * holds in device memory, one per GPU, from the moment it is loaded there until the process ends; the call
+ * allocates and frees nothing.  Fails with a message when split * M * N * 2 bytes exceed the buffer.  Every
+ * call on a GPU shares that GPU's buffer: calls that overlap in time on one GPU (two streams, two threads) race
+ * on it; calls in one stream's order do not.  The current device must be the one `stream` belongs to.
+ * Other requirements and results as call_dequant_gemm_fp16_fp4_splitk (bit-identical to it). */
+#define DQ_STATIC_SCRATCH_BYTES (16u << 20)
+int call_dequant_gemm_fp16_fp4_splitk_static(const void* A, const void* B, void* C, int M, int N, int K, int split,
+                                             int transposed, dq_stream_t stream);
+
 /* The 2-bit and 1-bit cases of the same example (`num_bits`: B[N, K * bits / 8], 16 or 32 codes per 32-bit word):
  * C[M,N] fp16 = A[M,K] fp16 . dequant(B, Scale[N, K/group], Zeros[N, K/group])^T, fp32 accumulation.
  * `convention` is a DQ_I2_* value: DQ_I2_TWOS is the example's slow path (`_tir_packed_int_to_int_convert`,

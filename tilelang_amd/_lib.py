@@ -32,6 +32,7 @@ SIGNATURES = {
     "call_dequant_gemm_bf16_mxfp4": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4_splitk": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "call_dequant_gemm_fp16_fp4_splitk_static": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_w4_fp16": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "call_gemm_int8xint2": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, ctypes.c_float, _i, _vp],
     "call_bitnet_activation_quant": [_vp, _vp, _vp, _i, _i, _vp],

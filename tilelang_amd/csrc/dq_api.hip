@@ -47,6 +47,29 @@ int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_s
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// ---- device-resident scratch of the entry point that allocates nothing ---------------------------------
+// One copy per GPU, held from the moment the library's code object is loaded on that GPU until the process
+// ends.  Host code never uses the array's name as an address: the name is a host-side stand-in, the device
+// address comes from hipGetSymbolAddress, once per device with that device current.
+constexpr size_t kStaticScratchBytes = DQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+
+static int scratch_of_current_device(const char* fn, void** out) {
+  int device = -1;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("%s: device index %d is beyond the %d this library tracks", fn, device, kMaxDevices);
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    DQ_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) DQ_FAIL("%s: the static scratch buffer has no address on device %d", fn, device);
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return 0;
+}
+
 static int check_w4_args(const char* fn, const void* B, const void* S, const void* Z, int N, int K, int group, int mode,
                          int layout) {
   if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
@@ -82,6 +105,8 @@ extern "C" int init(void) {
   const int kLargestLdsRequest = 160 * 1024;
   if (kLargestLdsRequest > max_lds)
     DQ_FAIL("Requested dynamic shared memory %d exceeds device limit %d", kLargestLdsRequest, max_lds);
+  void* scratch_ptr = nullptr;
+  if (scratch_of_current_device("init", &scratch_ptr)) return -1;
   return 0;
 }
 
@@ -212,6 +237,25 @@ extern "C" int call_dequant_gemm_fp16_fp4_splitk(const void* A, const void* B, v
   if (!aligned16(SplitC)) DQ_FAIL("%s: SplitC must be 16-byte aligned", fn);
   if (((size_t)M * N) % 8 != 0) DQ_FAIL("%s: M * N must be a multiple of 8 when split > 1 (got %d x %d)", fn, M, N);
   return fp16_fp4_gemm_splitk(A, B, SplitC, C, M, N, K, split, transposed, (hipStream_t)stream);
+}
+
+extern "C" int call_dequant_gemm_fp16_fp4_splitk_static(const void* A, const void* B, void* C, int M, int N, int K,
+                                                        int split, int transposed, dq_stream_t stream) {
+  const char* fn = "call_dequant_gemm_fp16_fp4_splitk_static";
+  if (check_gemm_args(fn, A, B, C, M, N, K, 64)) return -1;
+  if (split < 1 || split > 64) DQ_FAIL("%s: split=%d must be in 1..64", fn, split);
+  if (K % (64 * split) != 0) DQ_FAIL("%s: K=%d must be a multiple of 64 * split (split=%d)", fn, K, split);
+  if (split == 1) return fp16_fp4_gemm(A, B, C, M, N, K, transposed, (hipStream_t)stream);
+  if (((size_t)M * N) % 8 != 0) DQ_FAIL("%s: M * N must be a multiple of 8 when split > 1 (got %d x %d)", fn, M, N);
+  const size_t need = (size_t)split * (size_t)M * (size_t)N * sizeof(half_t);
+  if (need > kStaticScratchBytes)
+    DQ_FAIL("%s: split * M * N fp16 partial results need %zu bytes, the static scratch buffer holds %zu; use "
+            "call_dequant_gemm_fp16_fp4_splitk with a buffer of your own", fn, need, kStaticScratchBytes);
+  void* parts = nullptr;
+  if (scratch_of_current_device(fn, &parts)) return -1;
+  // every partial result the summing kernel reads is written by its slice's workgroups first, in stream order:
+  // nothing has to start at zero, whatever the last call left behind
+  return fp16_fp4_gemm_splitk(A, B, parts, C, M, N, K, split, transposed, (hipStream_t)stream);
 }
 
 extern "C" int call_dequant_gemm_w4_fp16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
