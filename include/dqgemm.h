@@ -70,6 +70,20 @@ int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, 
 int call_dequantize_w4(const void* B, const void* Scale, const void* Zeros, void* W, int N, int K, int group,
                        int mode, int layout, dq_stream_t stream);
 
+enum dq_qzeros_format {
+  DQ_QZEROS_INT16 = 0,  /* QZeros[N, groups] int16, one zero point per group: what decode_i4u_to_f16_scale_zeros_quantized
+                           reads (`int16_t zero_r`, examples/dequantize_gemm/quantize/lop3.py:339-341)                    */
+  DQ_QZEROS_PACKED4 = 1 /* QZeros[N, ceil(groups / 2)] bytes, 4-bit zero points, group g in bits 4 (g % 2) of byte g / 2:
+                           the `(qzeros >> (group_offset * 4)) & 0xf` of the _offset variant, lop3.py:381-385             */
+};
+
+/* Zeros[N, groups] fp16 = the integer zero points of the "quantized" zeros mode.  The reference's decoder computes
+ * (q - qz) exactly in fp16 by folding qz into its magic number and multiplies by the scale once
+ * (examples/dequantize_gemm/quantize/lop3.py:326-363, 367-420); DQ_W4_ZEROS_ORIGINAL fed with the fp16 copy of qz
+ * returns the same bits, because fp16(qz) and q - fp16(qz) are exact.  So a caller with integer zero points converts
+ * them with this call (once for static weights, or per call) and uses DQ_W4_ZEROS_ORIGINAL. */
+int call_unpack_qzeros(const void* QZeros, void* Zeros, int N, int groups, int format, dq_stream_t stream);
+
 /* ---- MXFP4 x bf16 ------------------------------------------------------------------------ */
 
 enum dq_fp4_format {
@@ -182,13 +196,38 @@ int call_quantize_bf16_mxfp4(const void* W, void* B, void* Scale, int N, int K, 
 int call_gemm_mxfp4_mxfp4(const void* A, const void* B, const void* ScaleA, const void* ScaleB, const void* Bias,
                           void* C, int M, int N, int K, dq_stream_t stream);
 
-/* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T.
- * is_signed 1: two's-complement nibbles (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:10-21,
- * `call(A, B, Ct)` :109-147); 0: unsigned nibbles (example_dequant_gemm_fine_grained.py int8 path).
- * a_packed 1: A is packed int4 too, A[M,K/2] (examples/gemm_int4/example_tilelang_gemm_int4.py:17-38).
- * Requires K % 128 == 0. */
-int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed,
+enum dq_i4_decode {
+  DQ_I4_UNSIGNED = 0,      /* w = q, plain nibbles (example_dequant_gemm_fine_grained.py int8 path)                     */
+  DQ_I4_TWOS = 1,          /* w = sext4(q), plain nibbles (example_dequant_gemm_w4a8.py:10-21)                          */
+  DQ_I4U_INTERLEAVED = 2,  /* w = q, words through interleave_weight(qB, 4, "int8"): decode_i4u_to_i8s,
+                              examples/dequantize_gemm/quantize/lop3.py:1027-1047                                      */
+  DQ_I4S_INTERLEAVED = 3   /* w = q - 7 (the decoder's MEDIAN_NUM is 0x07070707), same words: decode_i4s_to_i8s,
+                              lop3.py:999-1025                                                                         */
+};
+
+/* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T, `decode` a DQ_I4_* value.
+ * Replaces `call(A, B, Ct)` of examples/dequantize_gemm/example_dequant_gemm_w4a8.py:109-147 (DQ_I4_TWOS), the int8
+ * path of example_dequant_gemm_fine_grained.py (DQ_I4_UNSIGNED) and the int8 branch of
+ * example_dequant_gemv_fp16xint4.py:47-48,113-133 with fast_decoding (the two interleaved decoders).
+ * a_packed 1: A is packed int4 too, A[M,K/2] (examples/gemm_int4/example_tilelang_gemm_int4.py:17-38), DQ_I4_TWOS
+ * only, K < 131072 (both operands carry a factor 16 in the int32 accumulator).  Requires K % 128 == 0. */
+int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int decode, int a_packed,
                         int transposed, dq_stream_t stream);
+
+/* ---- plain GEMM on the same MFMA tile (no dequantise step) ----------------------------------------- */
+
+enum dq_dtype { DQ_DT_F16 = 0, DQ_DT_BF16 = 1, DQ_DT_I8 = 2, DQ_DT_F32 = 3, DQ_DT_I32 = 4 };
+
+/* C[M,N] = op(A) . op(B), both operands at the compute type, fp32 / int32 accumulation on the tile the dequantize
+ * GEMMs share.  Replaces `call(A, B, C, stream)` of the kernel built by `matmul(M, N, K, ..., trans_A, trans_B,
+ * in_dtype, out_dtype, accum_dtype)` of testing/python/kernel/test_tilelang_kernel_gemm.py:5-49 (and
+ * testing/python/amd/test_tilelang_test_amd.py:7-55): A is [M,K], or [K,M] when trans_A; B is [N,K] when trans_B
+ * (the layout of every dequantize kernel), else [K,N].  in_dtype DQ_DT_F16 / DQ_DT_BF16 with out_dtype the same or
+ * DQ_DT_F32; DQ_DT_I8 with DQ_DT_I32 (exact).  An operand stored the other way round is transposed first into
+ * Workspace, which the caller passes: (trans_A ? M*K : 0) + (trans_B ? 0 : N*K) elements of in_dtype, each part rounded
+ * up to 256 bytes; NULL allowed for trans_A = 0, trans_B = 1.  Requires K % 64 == 0 (K % 128 == 0 for int8). */
+int call_gemm_plain(const void* A, const void* B, void* C, void* Workspace, int M, int N, int K, int in_dtype,
+                    int out_dtype, int trans_A, int trans_B, dq_stream_t stream);
 
 #ifdef __cplusplus
 }

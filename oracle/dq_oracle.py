@@ -251,6 +251,62 @@ def fast_decode_i2_to_i8(words: np.ndarray, signed: bool) -> np.ndarray:
     return out
 
 
+def fast_decode_i4_to_i8(word_pairs: np.ndarray, signed: bool) -> np.ndarray:
+    """Semantics of decode_i4{u,s}_to_i8s on two uint32 (``[..., 2]``) -> 16 int8, in output order.
+
+    Follows examples/dequantize_gemm/quantize/lop3.py:999-1047: for i in 0..1,
+    ``i8s[i] = (i4b[0] >> 4i) & 0x0f0f0f0f`` and ``i8s[i + 2] = (i4b[1] >> 4i) & 0x0f0f0f0f``; the signed decoder
+    then subtracts 0x07070707 per byte with signed saturation (``__vsubss4``; its MEDIAN_NUM is 7, not 8).
+    """
+    w = np.asarray(word_pairs).astype(np.uint32)
+    assert w.shape[-1] == 2
+    out = np.empty(w.shape[:-1] + (16,), dtype=np.int8)
+    for i in range(2):
+        for src in range(2):
+            d = (w[..., src] >> np.uint32(4 * i)) & np.uint32(0x0F0F0F0F)
+            for b in range(4):
+                v = ((d >> np.uint32(8 * b)) & 0xFF).astype(np.int16)
+                if signed:
+                    v = np.clip(v - 7, -128, 127)
+                out[..., 4 * (i + 2 * src) + b] = v.astype(np.int8)
+    return out
+
+
+def decode_i4_fast_int8(packed_interleaved: np.ndarray, signed: bool) -> np.ndarray:
+    """[N, K/2] bytes whose 32-bit words went through ``interleave_weight(., 4, "int8")`` -> int8 [N, K] as
+    decode_i4{u,s}_to_i8s yields them, 16 values per pair of words (lop3.py:999-1047)."""
+    p = np.ascontiguousarray(packed_interleaved).view(np.uint8)
+    w = p.view(np.uint32).reshape(p.shape[0], -1, 2)
+    return fast_decode_i4_to_i8(w, signed).reshape(p.shape[0], -1)
+
+
+def fast_decode_i4u_to_f16_zeros_quantized(words: np.ndarray, scale, qzero) -> np.ndarray:
+    """Bit-level semantics of decode_i4u_to_f16_scale_zeros_quantized on one uint32 -> 8 fp16, in output order
+    (examples/dequantize_gemm/quantize/lop3.py:326-363): ``h = (w >> 4i) & 0x000f000f | 0x64006400`` as two fp16,
+    plus ``(0xe400 | zero)`` as fp16 (= -(1024 + zero)) in an fp16 add, then one fp16 fma with the scale and 0."""
+    w = np.asarray(words).astype(np.uint32)
+    s = np.asarray(scale, dtype=np.float16).astype(np.float32)
+    med = (np.uint16(0xE400) | np.asarray(qzero).astype(np.uint16)).view(np.float16).astype(np.float32)
+    out = np.empty(w.shape + (8,), dtype=np.float16)
+    for i in range(4):
+        h = ((w >> np.uint32(4 * i)) & np.uint32(0x000F000F)) | np.uint32(0x64006400)
+        for half, sh in ((0, 0), (1, 16)):
+            x = ((h >> np.uint32(sh)) & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float32)
+            d = (x + med).astype(np.float16).astype(np.float32)          # add.f16x2
+            out[..., 2 * i + half] = (d * s + np.float32(0)).astype(np.float16)  # fma.rn.f16x2 (product exact in fp32)
+    return out
+
+
+def unpack_qzeros(qzeros: np.ndarray, groups: int, fmt: str = "int16") -> np.ndarray:
+    """Integer zero points of the "quantized" zeros mode as int32 [N, groups].  ``"int16"``: one per group
+    (lop3.py:339-341).  ``"packed4"``: 4-bit, group g in bits 4 (g % 2) of byte g / 2 (lop3.py:381-385)."""
+    if fmt == "int16":
+        return np.asarray(qzeros).astype(np.int16).astype(np.int32)
+    b = np.ascontiguousarray(qzeros).view(np.uint8)
+    z = np.stack((b & 0xF, b >> 4), axis=-1).reshape(b.shape[0], -1)
+    return z[:, :groups].astype(np.int32)
+
+
 def fast_decode_i2_to_f16(halfwords: np.ndarray, signed: bool, scale=None) -> np.ndarray:
     """Semantics of decode_i2{u,s}_to_f16[_scale] on one 16-bit word -> 8 fp16, in output order.
 

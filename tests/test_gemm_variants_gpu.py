@@ -29,6 +29,29 @@ def test_w4a8_exact(cuda, M, N, K):
     np.testing.assert_array_equal(Ct.cpu().numpy(), orc.ref_w4a8(d["A"], d["B"]))
 
 
+@pytest.mark.parametrize("decode", [2, 3])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 256), (100, 130, 384), (1500, 2000, 256), (3581, 3589, 768)])  # last: direct-to-LDS kernel
+def test_int8xint4_fast_decode_exact(cuda, M, N, K, decode):
+    """The int8 branch of the GEMV example with fast_decoding, at GEMM sizes, through the C-ABI: words passed through
+    interleave_weight(., 4, "int8"), decode_i4u_to_i8s (w = q) / decode_i4s_to_i8s (w = q - 7),
+    examples/dequantize_gemm/quantize/lop3.py:999-1047; exact int32, all byte values."""
+    import ctypes
+
+    from tilelang_amd import _lib
+
+    d = workloads.int8_int4(M, N, K, seed=M + decode)
+    Bil = orc.interleave_weight(d["B"].view(np.int8), 4, "int8").view(np.uint8)
+    W = orc.decode_i4_fast_int8(Bil, signed=(decode == 3)).astype(np.int64)
+    A, B = _dev(d["A"], cuda), _dev(Bil, cuda)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    lib = _lib.get_library()
+    rc = lib.call_gemm_int8xint4(ctypes.c_void_p(A.data_ptr()), ctypes.c_void_p(B.data_ptr()), ctypes.c_void_p(C.data_ptr()),
+                                 M, N, K, decode, 0, 0, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, lib.get_last_error().decode()
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), d["A"].astype(np.int64) @ W.T)
+
+
 @pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (16, 16, 128), (300, 200, 256), (1500, 2000, 256), (3584, 3590, 128)])
 def test_int4xint4_exact(cuda, M, N, K):
     """examples/gemm_int4/example_tilelang_gemm_int4.py:70-103: rtol=0, atol=0."""

@@ -288,7 +288,14 @@ def test_lowbit_gemv_factory_rejections():
         tl.dequantize_gemv(1, 64, 1024, "float16", "float16", "float32", num_bits=3)
     with pytest.raises(ValueError):
         tl.dequantize_gemv(1, 64, 1024, "int8", "float16", "int32", num_bits=2)
-    with pytest.raises(ValueError):
-        tl.dequantize_gemv(1, 64, 1024, "int8", "int32", "int32", num_bits=4, fast_decoding=True)
+    # int8 x int4 with fast_decoding is built (decode_i4{u,s}_to_i8s over interleave_weight(., 4, "int8") words)
+    assert tl.dequantize_gemv(1, 64, 1024, "int8", "int32", "int32", num_bits=4, fast_decoding=True).name == "dequantize_gemv"
+    with pytest.raises(ValueError, match="qzeros_format"):
+        tl.dequantize_gemv(1, 64, 1024, with_scaling=True, with_zeros=True, zeros_mode="quantized", group_size=128,
+                           qzeros_format="int3")
+    k = tl.dequantize_gemv(1, 64, 1024, with_scaling=True, with_zeros=True, zeros_mode="quantized", group_size=128)
+    assert [p.dtype for p in k.params if p.name == "Zeros"] == [torch.int16] and k.workspace_idx == [len(k.params) - 1]
+    k = tl.dequantize_w4(64, 1024, 128, source_format="uint", with_zeros=True, zeros_mode="quantized", qzeros_format="packed4")
+    assert [p.shape for p in k.params if p.name == "Zeros"] == [(64, 4)]
     with pytest.raises(ValueError):
         tl.dequantize_gemv(1, 64, 1024, "int8", "int32", "int32", num_bits=2, with_scaling=True, group_size=128)

@@ -131,7 +131,8 @@ def test_lowbit_scale_and_zeros(cuda, bits, M, N, K, group, fast, fmt, zeros_mod
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (3, 520, 2048), (64, 256, 1024)])
-@pytest.mark.parametrize("bits,fast,fmt", [(2, False, "uint"), (2, True, "int"), (2, True, "uint"), (4, False, "int")])
+@pytest.mark.parametrize("bits,fast,fmt", [(2, False, "uint"), (2, True, "int"), (2, True, "uint"), (4, False, "int"),
+                                           (4, True, "uint"), (4, True, "int")])
 def test_dequantize_gemv_int8_exact(cuda, M, N, K, bits, fast, fmt):
     """use_dp4a branch of the example (example_dequant_gemv_fp16xint4.py:47-48,126-133): exact int32."""
     rng = np.random.default_rng(M + N + K + bits)
@@ -141,6 +142,11 @@ def test_dequantize_gemv_int8_exact(cuda, M, N, K, bits, fast, fmt):
         conv = "twos" if not fast else ("offset" if fmt == "int" else "unsigned")
         W = orc.decode_i2(packed, conv).astype(np.int64)
         B = orc.interleave_weight(packed.view(np.int8), 2, "int8").view(np.uint8) if fast else packed
+    elif fast:
+        # decode_i4{u,s}_to_i8s over interleave_weight(., 4, "int8") words (lop3.py:999-1047): w = q, or q - 7
+        B = orc.interleave_weight(packed.view(np.int8), 4, "int8").view(np.uint8)
+        W = orc.decode_i4_fast_int8(B, signed=(fmt == "int")).astype(np.int64)
+        assert np.array_equal(W, orc.unpack_u4(packed).astype(np.int64) - (7 if fmt == "int" else 0))
     else:
         W = orc.decode_i4_signed(packed).astype(np.int64)
         B = packed

@@ -5,6 +5,8 @@ import itertools
 import json
 import os
 
+from fractions import Fraction
+
 import numpy as np
 import pytest
 
@@ -142,6 +144,107 @@ def test_w4_zeros_modes_rounding_order():
     quant = orc.dequant_u4_scale_zeros(packed, s, np.array([[7]]), 4, "quantized")[0]
     want = [np.float16((x - 7) * float(s[0, 0])) for x in q]
     assert quant.tolist() == [float(v) for v in want]
+
+
+def _rne(x: Fraction, mant_bits: int, emin: int, emax: int) -> float:
+    """Round an exact rational to the nearest value of a binary floating-point format (ties to even), written out
+    with integers only: `mant_bits` stored mantissa bits, normal exponents emin..emax, subnormals below."""
+    if x == 0:
+        return 0.0
+    sign, a = (-1.0 if x < 0 else 1.0), abs(x)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1
+    assert Fraction(2) ** e <= a < Fraction(2) ** (e + 1)
+    e = max(e, emin)
+    quantum = Fraction(2) ** (e - mant_bits)
+    n = a / quantum
+    lo = n.numerator // n.denominator
+    rem = n - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+        lo += 1
+    val = lo * quantum
+    if val >= Fraction(2) ** (emax + 1):
+        return sign * float("inf")
+    return sign * float(val)
+
+
+def _rne16(x):
+    return _rne(Fraction(x), 10, -14, 15)
+
+
+def _rne32(x):
+    return _rne(Fraction(x), 23, -126, 127)
+
+
+def test_rne_helper_against_numpy_casts():
+    rng = np.random.default_rng(11)
+    xs = np.concatenate([rng.standard_normal(500) * 10.0 ** rng.integers(-8, 5, 500), [65504.0, 65519.9, 65520.0, 6e-8, 2.98e-8, 0.0]])
+    for x in xs:
+        assert _rne16(Fraction(float(x))) == float(np.float64(x).astype(np.float16))
+        assert _rne32(Fraction(float(x))) == float(np.float64(x).astype(np.float32))
+
+
+def test_w4_decoders_rounding_order_step_by_step():
+    """Every scaled / zero-point uint4 decoder against its operation order written out with exact rationals and an
+    explicit round-to-nearest-even per fp16 instruction (examples/dequantize_gemm/quantize/lop3.py:41-81, 136-176,
+    233-271, 326-363): sub.f16x2 rounds, fma.rn.f16x2 rounds once."""
+    rng = np.random.default_rng(12)
+    scales = np.concatenate([rng.uniform(1e-4, 2.0, 60), [6.1e-5, 1.0, 0.013, 655.0]]).astype(np.float16)
+    zeros = np.array([0.0, 7.0, 7.5, 8.0, 15.0, -3.25, 6.0, 10.0, 0.3335], dtype=np.float16)
+    qz_int = [0, 1, 7, 8, 15, 100, 1023]
+    for s in scales:
+        S = np.array([[s]], dtype=np.float16)
+        fs = Fraction(float(s))
+        packed = np.array([[(2 * i) | ((2 * i + 1) << 4) for i in range(8)]], dtype=np.uint8)  # q = 0..15
+        got = orc.dequant_u4_scale(packed, S, 16)[0]
+        assert got.tolist() == [_rne16((q - 8) * fs) for q in range(16)]
+        for z in zeros:
+            Z = np.array([[z]], dtype=np.float16)
+            fz = Fraction(float(z))
+            got = orc.dequant_u4_scale_zeros(packed, S, Z, 16, "original")[0]
+            assert got.tolist() == [_rne16(Fraction(_rne16(q - fz)) * fs) for q in range(16)]
+            got = orc.dequant_u4_scale_zeros(packed, S, Z, 16, "rescale")[0]
+            assert got.tolist() == [_rne16(q * fs - fz) for q in range(16)]
+        for qz in qz_int:
+            got = orc.dequant_u4_scale_zeros(packed, S, np.array([[qz]]), 16, "quantized")[0]
+            want = [_rne16((q - qz) * fs) for q in range(16)]
+            assert got.tolist() == want
+            # the device snippet's own route: magic-number add, then one fma (emits nibble pairs (i, i + 4))
+            w = np.array([0x76543210, 0xFEDCBA98], dtype=np.uint32)
+            bits = orc.fast_decode_i4u_to_f16_zeros_quantized(w, s, qz)
+            order = [0, 4, 1, 5, 2, 6, 3, 7]
+            assert bits[0].tolist() == [want[i] for i in order]
+            assert bits[1].tolist() == [want[8 + i] for i in order]
+            # and the "original" decoder fed with fp16(qz) gives the same bits (what the library relies on)
+            if qz <= 15:
+                same = orc.dequant_u4_scale_zeros(packed, S, np.array([[qz]], dtype=np.float16), 16, "original")[0]
+                np.testing.assert_array_equal(same.view(np.uint16), got.view(np.uint16))
+
+
+def test_unpack_qzeros_formats():
+    z = np.array([[3, 15, 0, 9, 7]], dtype=np.int16)
+    assert orc.unpack_qzeros(z, 5, "int16").tolist() == [[3, 15, 0, 9, 7]]
+    packed = np.array([[3 | (15 << 4), 0 | (9 << 4), 7]], dtype=np.uint8)
+    assert orc.unpack_qzeros(packed, 5, "packed4").tolist() == [[3, 15, 0, 9, 7]]
+
+
+def test_i4_to_i8_fast_decode_and_interleave():
+    """decode_i4{u,s}_to_i8s (lop3.py:999-1047) over interleave_weight(., 4, "int8") words: the unsigned decoder gives
+    back the plain nibbles in k order, the signed one q - 7 (its MEDIAN_NUM is 0x07070707), for every nibble value
+    at every position."""
+    one = orc.interleave_weight(np.array([0x76543210], dtype=np.uint32).view(np.int8), 4, "int8").view(np.uint32)[0]
+    assert one == 0x73625140  # element e at byte e % 4, nibble slot e / 4
+    got = orc.fast_decode_i4_to_i8(np.array([[0x73625140, 0xFBEAD9C8]], dtype=np.uint32), signed=False)[0]
+    assert got.tolist() == list(range(16))
+    got = orc.fast_decode_i4_to_i8(np.array([[0x73625140, 0xFBEAD9C8]], dtype=np.uint32), signed=True)[0]
+    assert got.tolist() == [q - 7 for q in range(16)]
+    rng = np.random.default_rng(13)
+    raw = rng.integers(0, 256, size=(16, 64), dtype=np.uint8)
+    raw[0, :16] = np.arange(16, dtype=np.uint8) * 17  # every nibble value in both halves
+    il = orc.interleave_weight(raw.view(np.int8), 4, "int8").view(np.uint8)
+    np.testing.assert_array_equal(orc.decode_i4_fast_int8(il, signed=False), orc.unpack_u4(raw).astype(np.int8))
+    np.testing.assert_array_equal(orc.decode_i4_fast_int8(il, signed=True), orc.unpack_u4(raw).astype(np.int8) - 7)
 
 
 def test_i2_conventions():
@@ -357,6 +460,16 @@ def test_bitlinear_quantisers_and_epilogue():
     acc = np.array([[100, -7]], dtype=np.int32)
     out = orc.post_quant_process(acc, np.array([[4.0]], np.float32), np.float32(2.0))
     assert out.dtype == np.float16 and out.tolist() == [[12.5, -0.875]]
+    # two fp32 divisions in that order, then one rounding to fp16 (utils_quant.py:165-170), with exact rationals and
+    # an explicit rounding per operation; (acc / (s_a * s_w)) would differ in the last bit for some of these
+    accs = rng.integers(-1040384, 1040385, size=200)
+    sas = rng.uniform(0.5, 50.0, size=200).astype(np.float32)
+    sws = rng.uniform(0.5, 4.0, size=200).astype(np.float32)
+    for a, sa, sw_ in zip(accs, sas, sws):
+        got = orc.post_quant_process(np.array([[a]], dtype=np.int32), np.array([[sa]], np.float32), np.float32(sw_))[0, 0]
+        step1 = _rne32(Fraction(int(a)) / Fraction(float(sa)))
+        step2 = _rne32(Fraction(step1) / Fraction(float(sw_)))
+        assert float(got) == _rne16(Fraction(step2))
 
 
 def test_torch_restatement_matches_numpy_oracle():

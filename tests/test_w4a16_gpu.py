@@ -81,6 +81,65 @@ def test_dequant_tile_bit_exact(cuda, mode, interleaved):
     np.testing.assert_array_equal(got.view(np.uint16), expected.view(np.uint16))
 
 
+@pytest.mark.parametrize("qfmt", ["int16", "packed4"])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_dequant_tile_quantized_zeros_bit_exact(cuda, qfmt, interleaved):
+    """zeros_mode="quantized": integer zero points (examples/dequantize_gemm/quantize/lop3.py:326-420), as one int16
+    per group or as packed 4-bit values; the tile equals the oracle's (q - qz) * s bit for bit."""
+    N, K, group = 96, 1280, 128  # ten groups per row: an odd byte count is not involved, five bytes per row when packed
+    rng = np.random.default_rng(5)
+    d = workloads.w4a16(1, N, K, group, seed=6, scale_range=(0.002, 0.02))
+    B, S = d["B"], d["Scale"]
+    B[0, :128] = np.arange(256, dtype=np.uint8)[::2]
+    S[2, :4] = np.array([6.1e-5, 1.0, -0.013, 655.0], dtype=np.float16)
+    groups = K // group
+    qz = rng.integers(0, 16, size=(N, groups)).astype(np.int16)
+    if qfmt == "int16":
+        qz[1, :4] = [0, 100, 1023, 15]  # beyond a nibble: the int16 form allows it (0xe400 | qz holds 10 bits)
+        Zdev = _dev(qz, cuda)
+    else:
+        packed = (qz[:, 0::2] | (qz[:, 1::2] << 4)).astype(np.uint8)
+        assert np.array_equal(orc.unpack_qzeros(packed, groups, "packed4"), qz)
+        Zdev = _dev(packed, cuda)
+    expected = orc.dequant_u4_scale_zeros(B, S, qz, group, "quantized")
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = tl.quantize.interleave_weight(Bdev, 4, "float16")
+    kern = tl.dequantize_w4(N, K, group, source_format="uint", fast_decoding=interleaved, with_scaling=True,
+                            with_zeros=True, zeros_mode="quantized", qzeros_format=qfmt)
+    W = kern(Bdev, _dev(S, cuda), Zdev)
+    torch.cuda.synchronize()
+    got = W.cpu().numpy()
+    assert got.shape == (N, K)
+    np.testing.assert_array_equal(got.view(np.uint16), expected.view(np.uint16))
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 64, 300])
+@pytest.mark.parametrize("qfmt", ["int16", "packed4"])
+def test_gemv_quantized_zeros(cuda, M, qfmt):
+    """kernel(A, B, Scale, QZeros, C) with integer zero points through every kernel the dispatch picks for these M
+    (dot2 GEMV, register-resident, streaming, tiled GEMM), against the oracle's quantized-mode tile."""
+    N, K, group = 1536, 2048, 128
+    rng = np.random.default_rng(M)
+    d = workloads.w4a16(M, N, K, group, seed=M, scale_range=(0.002, 0.01))
+    qz = rng.integers(6, 11, size=(N, K // group)).astype(np.int16)
+    Z = _dev(qz, cuda) if qfmt == "int16" else _dev((qz[:, 0::2] | (qz[:, 1::2] << 4)).astype(np.uint8), cuda)
+    kern = tl.dequantize_gemv(M, N, K, group_size=group, source_format="uint", with_scaling=True, with_zeros=True,
+                              zeros_mode="quantized", qzeros_format=qfmt)
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["Scale"], cuda), Z, C)
+    torch.cuda.synchronize()
+    W = orc.dequant_u4_scale_zeros(d["B"], d["Scale"], qz, group, "quantized")
+    ref = (d["A"].astype(np.float32) @ W.astype(np.float32).T).astype(np.float16)
+    np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+    # the GEMM factory takes the same operands
+    C2 = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    tl.matmul_w4a16(M, N, K, group, source_format="uint", with_scaling=True, with_zeros=True, zeros_mode="quantized",
+                    qzeros_format=qfmt)(_dev(d["A"], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["Scale"], cuda), Z, C2)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(C2.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+
+
 def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False, scale_range=(0.005, 0.02)):
     d = workloads.w4a16(M, N, K, group, seed=seed, scale_range=scale_range, zeros_range=(6, 10))
     kw = _mode_kwargs(mode)

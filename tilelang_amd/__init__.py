@@ -18,6 +18,7 @@ from .kernels import (  # noqa: F401
     matmul_mxfp4_mxfp4,
     matmul_fp16_fp4,
     matmul_int8xint4,
+    matmul,
     matmul_nt_int4,
     matmul_w4_fine_grained,
     matmul_w4a16,

@@ -28,6 +28,7 @@ SIGNATURES = {
     "init": [],
     "call_dequantize_gemv_w4a16": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequantize_gemv_lowbit": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "call_unpack_qzeros": [_vp, _vp, _i, _i, _i, _vp],
     "call_dequantize_w4": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_bf16_mxfp4": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
@@ -38,6 +39,7 @@ SIGNATURES = {
     "call_bitnet_activation_quant": [_vp, _vp, _vp, _i, _i, _vp],
     "call_quantize_bf16_mxfp4": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "call_gemm_int8xint4": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "call_gemm_plain": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_gemm_mxfp4_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
 }
 

@@ -57,10 +57,10 @@ class KernelAdapter:
         self.params = list(params)
         n = len(self.params)
         self.result_idx = [i if i >= 0 else n + i for i in result_idx]
-        # parameters the kernel uses as scratch (the reference's T.alloc_buffer globals): allocated here, once per
-        # device, passed to the library, never returned
+        # parameters the kernel uses as scratch (the reference's T.alloc_buffer globals): allocated here for every
+        # call, passed to the library, never returned.  torch's caching allocator hands a freed block back to the
+        # stream it was used on only, so calls on different streams never share a scratch buffer.
         self.workspace_idx = [i if i >= 0 else n + i for i in workspace_idx]
-        self._workspaces = {}
         self._launch = launch
         self._get_last_error = get_last_error
         self.device_type = device_type
@@ -125,10 +125,7 @@ class KernelAdapter:
             if i in self.workspace_idx:
                 if device is None:
                     device = torch.device(self.device_type)
-                key = (i, str(device))
-                if key not in self._workspaces:
-                    self._workspaces[key] = torch.empty(*p.shape, dtype=p.dtype, device=device)
-                tensors.append(self._workspaces[key])
+                tensors.append(torch.empty(*p.shape, dtype=p.dtype, device=device))
             elif i in self.result_idx:
                 if device is None:
                     device = torch.device(self.device_type)

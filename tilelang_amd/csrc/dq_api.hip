@@ -42,8 +42,12 @@ int fp16_fp4_gemm_splitk(const void* A, const void* B, void* parts, void* C, int
                          int transposed, hipStream_t stream);
 int mxfp4_mxfp4_gemm(const void* A, const void* SA, const void* B, const void* SB, const void* Bias, void* C, int M,
                      int N, int K, hipStream_t stream);
-int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
+int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int decode, int a_packed, int transposed,
             hipStream_t stream);
+
+int unpack_qzeros(const void* QZ, void* Z, int N, int groups, int packed, hipStream_t stream);
+int plain_gemm(const void* A, const void* B, void* C, void* workspace, int M, int N, int K, int in_dtype, int out_dtype,
+               int trans_A, int trans_B, hipStream_t stream);
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -192,6 +196,17 @@ extern "C" int call_dequantize_w4(const void* B, const void* Scale, const void* 
   return w4_dequant(B, Scale, Zeros, W, N, K, group, mode, layout, (hipStream_t)stream);
 }
 
+extern "C" int call_unpack_qzeros(const void* QZeros, void* Zeros, int N, int groups, int format, dq_stream_t stream) {
+  const char* fn = "call_unpack_qzeros";
+  if (!QZeros) DQ_FAIL("%s: QZeros is expected to have non-NULL data pointer", fn);
+  if (!Zeros) DQ_FAIL("%s: Zeros is expected to have non-NULL data pointer", fn);
+  if (N <= 0 || groups <= 0) DQ_FAIL("%s: N and groups must be positive (got %d, %d)", fn, N, groups);
+  if (format != DQ_QZEROS_INT16 && format != DQ_QZEROS_PACKED4) DQ_FAIL("%s: unknown qzeros format %d", fn, format);
+  if (format == DQ_QZEROS_INT16 && ((uintptr_t)QZeros & 1) != 0) DQ_FAIL("%s: int16 QZeros must be 2-byte aligned", fn);
+  if (((uintptr_t)Zeros & 1) != 0) DQ_FAIL("%s: Zeros must be 2-byte aligned", fn);
+  return unpack_qzeros(QZeros, Zeros, N, groups, format == DQ_QZEROS_PACKED4, (hipStream_t)stream);
+}
+
 extern "C" int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale, const void* Bias, void* C,
                                             int M, int N, int K, int scale_size, int fp4_format, int scale_bias,
                                             dq_stream_t stream) {
@@ -321,8 +336,24 @@ extern "C" int call_gemm_mxfp4_mxfp4(const void* A, const void* B, const void* S
   return mxfp4_mxfp4_gemm(A, ScaleA, B, ScaleB, Bias, C, M, N, K, (hipStream_t)stream);
 }
 
-extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int is_signed,
+extern "C" int call_gemm_plain(const void* A, const void* B, void* C, void* Workspace, int M, int N, int K, int in_dtype,
+                               int out_dtype, int trans_A, int trans_B, dq_stream_t stream) {
+  const char* fn = "call_gemm_plain";
+  if (in_dtype != DQ_DT_F16 && in_dtype != DQ_DT_BF16 && in_dtype != DQ_DT_I8)
+    DQ_FAIL("%s: in_dtype must be DQ_DT_F16, DQ_DT_BF16 or DQ_DT_I8 (got %d)", fn, in_dtype);
+  const bool ok_out = in_dtype == DQ_DT_I8 ? out_dtype == DQ_DT_I32 : (out_dtype == in_dtype || out_dtype == DQ_DT_F32);
+  if (!ok_out) DQ_FAIL("%s: out_dtype %d does not go with in_dtype %d (int8 -> int32; fp16 / bf16 -> the same or fp32)", fn, out_dtype, in_dtype);
+  if (check_gemm_args(fn, A, B, C, M, N, K, in_dtype == DQ_DT_I8 ? 128 : 64)) return -1;
+  if ((trans_A || !trans_B) && !Workspace) DQ_FAIL("%s: Workspace is expected to have non-NULL data pointer when trans_A or not trans_B", fn);
+  if (Workspace && !aligned16(Workspace)) DQ_FAIL("%s: Workspace must be 16-byte aligned", fn);
+  return plain_gemm(A, B, C, Workspace, M, N, K, in_dtype, out_dtype, trans_A != 0, trans_B != 0, (hipStream_t)stream);
+}
+
+extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int decode,
                                    int a_packed, int transposed, dq_stream_t stream) {
-  if (check_gemm_args("call_gemm_int8xint4", A, B, C, M, N, K, 128)) return -1;
-  return i4_gemm(A, B, C, M, N, K, is_signed, a_packed, transposed, (hipStream_t)stream);
+  const char* fn = "call_gemm_int8xint4";
+  if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
+  if (decode < DQ_I4_UNSIGNED || decode > DQ_I4S_INTERLEAVED) DQ_FAIL("%s: unknown decode %d", fn, decode);
+  if (a_packed && decode != DQ_I4_TWOS) DQ_FAIL("%s: a packed A goes with decode DQ_I4_TWOS only (got %d)", fn, decode);
+  return i4_gemm(A, B, C, M, N, K, decode, a_packed, transposed, (hipStream_t)stream);
 }

@@ -52,6 +52,15 @@ constexpr int kAStage = BM * kARowBytes;   // 32 KiB
 // XOR key of the 16-byte pieces of A row `row` in LDS (rows are 128 B).
 __host__ __device__ constexpr int a_swz(int row) { return (row >> DQ_SWZ_SHIFT) & 7; }
 
+// Where 16-byte piece `piece` of packed-B row `row` sits inside the row in LDS (register-staged kernel).  Rows of
+// 32 or 64 bytes: rotated by the row index so that the 16 rows of one ds_read_b128 phase cover all 64 banks.  Rows
+// of 128 bytes (an operand stored at the compute type, nothing to decode): the XOR swizzle of the A rows.
+template <int kPieces>
+__host__ __device__ constexpr int b_piece_pos(int row, int piece) {
+  if (kPieces == 8) return piece ^ a_swz(row);
+  return (piece + (row >> (kPieces == 2 ? 3 : 2))) % kPieces;
+}
+
 struct Params {
   const void* A;
   const void* B;
@@ -259,8 +268,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
     const int q = b_on[i] ? q0 : 0;
     const int row = q / kBPiecesPerRow, piece = q % kBPiecesPerRow;
     b_src[i] = (const unsigned char*)p.B + (size_t)min(n0 + row, N - 1) * b_row_bytes + piece * 16;
-    // rotate the pieces of a row so that the 16 rows of one ds_read_b128 phase cover all 64 banks
-    b_dst[i] = kAStage + row * P::kBRowBytes + (((piece + (row >> (kBPiecesPerRow == 2 ? 3 : 2))) % kBPiecesPerRow) << 4);
+    b_dst[i] = kAStage + row * P::kBRowBytes + (b_piece_pos<kBPiecesPerRow>(row, piece) << 4);
   }
 
   uint4_t a_reg[kALoads], b_reg[kBLoads];
@@ -309,7 +317,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
 #pragma unroll
     for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
       const int piece = g * (kBPiecesPerRow / 2) + h;
-      b_off[nb][h] = kAStage + row * P::kBRowBytes + (((piece + (row >> (kBPiecesPerRow == 2 ? 3 : 2))) % kBPiecesPerRow) << 4);
+      b_off[nb][h] = kAStage + row * P::kBRowBytes + (b_piece_pos<kBPiecesPerRow>(row, piece) << 4);
     }
   }
 

@@ -77,27 +77,43 @@ struct I2Policy : I8Mfma, gemm::NoScale, EPI {
 };
 
 // ---- int8 x 4-bit ---------------------------------------------------------------------------------
-// SIGNED: nibbles are two's complement; they are decoded as 16 x value (nibble in the top of the
+// DEC = I4_TWOS: nibbles are two's complement; they are decoded as 16 x value (nibble in the top of the
 // byte) and the accumulator is shifted back in the epilogue.  A_PACKED: A is packed int4 too and
 // is expanded the same way while it is staged, so both operands carry the factor 16.
-template <bool SIGNED, bool A_PACKED, class EPI>
+// DEC = I4U_INTERLEAVED / I4S_INTERLEAVED: the words went through interleave_weight(qB, 4, "int8")
+// (examples/dequantize_gemm/quantize/utils.py:71-125: element e of a word at byte e % 4, nibble slot e / 4), and
+// decode as decode_i4u_to_i8s (w = q) / decode_i4s_to_i8s (w = q - 7: its MEDIAN_NUM is 0x07070707)
+// (examples/dequantize_gemm/quantize/lop3.py:999-1047).  The same mask and shift then yield elements 0..3 and 4..7
+// in natural order, so A needs no shuffle.
+enum { I4_UNSIGNED = 0, I4_TWOS = 1, I4U_INTERLEAVED = 2, I4S_INTERLEAVED = 3 };
+
+template <int DEC, bool A_PACKED, class EPI>
 struct I4Policy : I8Mfma, gemm::NoScale, EPI {
   static constexpr int kBRowBytes = 64;
   static constexpr bool kAPacked = A_PACKED;
+  static constexpr bool kNatural = DEC >= I4U_INTERLEAVED;  // decoded elements come out in k order
+  __device__ static __forceinline__ uint32_t minus7(uint32_t x) {
+    // bytes 0..15 -> two's-complement bytes of x - 7: with bit 7 set no byte borrows from its neighbour
+    return ((x | 0x80808080u) - 0x07070707u) ^ 0x80808080u;
+  }
   __device__ static __forceinline__ uint32_t even(uint32_t w) {
-    return SIGNED ? ((w << 4) & 0xF0F0F0F0u) : (w & 0x0F0F0F0Fu);
+    if constexpr (DEC == I4_TWOS) return (w << 4) & 0xF0F0F0F0u;
+    else if constexpr (DEC == I4S_INTERLEAVED) return minus7(w & 0x0F0F0F0Fu);
+    else return w & 0x0F0F0F0Fu;
   }
   __device__ static __forceinline__ uint32_t odd(uint32_t w) {
-    return SIGNED ? (w & 0xF0F0F0F0u) : ((w >> 4) & 0x0F0F0F0Fu);
+    if constexpr (DEC == I4_TWOS) return w & 0xF0F0F0F0u;
+    else if constexpr (DEC == I4S_INTERLEAVED) return minus7((w >> 4) & 0x0F0F0F0Fu);
+    else return (w >> 4) & 0x0F0F0F0Fu;
   }
-  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return split_even_odd_bytes(v); }
+  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return kNatural ? v : split_even_odd_bytes(v); }
   // direct-to-LDS kernel (int8 A only: a packed A is expanded on its way to LDS): the byte shuffle moves behind
   // the LDS read, fragment by fragment
   static bool dma_ok(const Params&) { return !A_PACKED; }
   __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
   using gemm::NoScale::prep_scale;
   __device__ static __forceinline__ frag_t fix_a(frag_t f) {
-    return __builtin_bit_cast(frag_t, split_even_odd_bytes(__builtin_bit_cast(uint4_t, f)));
+    return kNatural ? f : __builtin_bit_cast(frag_t, split_even_odd_bytes(__builtin_bit_cast(uint4_t, f)));
   }
   __device__ static __forceinline__ void expand_a(uint4_t v, uint4_t& lo, uint4_t& hi) {
     lo = uint4_t{even(v[0]), odd(v[0]), even(v[1]), odd(v[1])};
@@ -139,26 +155,35 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
 #undef DQ_I2L
 }
 
-int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int is_signed, int a_packed, int transposed,
+int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int decode, int a_packed, int transposed,
             hipStream_t stream) {
   Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
   if (a_packed) {
-    if (!is_signed) DQ_FAIL("int4 gemm: packed A is built for signed int4 only");
-    if (transposed) return gemm::launch_auto<I4Policy<true, true, Int32Out<8, true>>>(p, stream);
-    return gemm::launch_auto<I4Policy<true, true, Int32Out<8, false>>>(p, stream);
+    if (decode != I4_TWOS) DQ_FAIL("int4 gemm: packed A is built for two's-complement int4 only");
+    // both operands carry a factor 16: |sum| <= 128 * 128 * K must stay below 2^31
+    if (K >= 131072) DQ_FAIL("int4 gemm: K=%d is beyond the 131071 that keep the int32 accumulation of packed operands exact", K);
+    if (transposed) return gemm::launch_auto<I4Policy<I4_TWOS, true, Int32Out<8, true>>>(p, stream);
+    return gemm::launch_auto<I4Policy<I4_TWOS, true, Int32Out<8, false>>>(p, stream);
   }
-#define DQ_I4(SIGNED_, SHIFT_, TRANS_)                                        \
+#define DQ_I4(DEC_, SHIFT_, TRANS_)                                           \
   do {                                                                        \
-    using Pol = I4Policy<SIGNED_, false, Int32Out<SHIFT_, TRANS_>>;           \
+    using Pol = I4Policy<DEC_, false, Int32Out<SHIFT_, TRANS_>>;              \
     if (gemm::dma_eligible<Pol>(p)) return gemm::launch_dma<Pol>(p, stream);  \
     return gemm::launch_auto<Pol>(p, stream);                                 \
   } while (0)
-  if (is_signed) {
-    if (transposed) DQ_I4(true, 4, true);
-    DQ_I4(true, 4, false);
+#define DQ_I4T(DEC_, SHIFT_)                  \
+  do {                                        \
+    if (transposed) DQ_I4(DEC_, SHIFT_, true); \
+    DQ_I4(DEC_, SHIFT_, false);               \
+  } while (0)
+  switch (decode) {
+    case I4_UNSIGNED: DQ_I4T(I4_UNSIGNED, 0);
+    case I4_TWOS: DQ_I4T(I4_TWOS, 4);
+    case I4U_INTERLEAVED: DQ_I4T(I4U_INTERLEAVED, 0);
+    case I4S_INTERLEAVED: DQ_I4T(I4S_INTERLEAVED, 0);
+    default: DQ_FAIL("int4 gemm: unknown decode %d", decode);
   }
-  if (transposed) DQ_I4(false, 0, true);
-  DQ_I4(false, 0, false);
+#undef DQ_I4T
 #undef DQ_I4
 }
 

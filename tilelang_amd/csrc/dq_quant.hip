@@ -214,4 +214,43 @@ int mxfp4_quant(const void* W, void* B, void* S, int N, int K, int scale_bias, h
   return 0;
 }
 
+
+namespace {
+
+// Integer zero points of the "quantized" zeros mode -> the fp16 Zeros[N, groups] the kernels read.  The reference's
+// decoder folds the integer into the magic number, (0x6400 | q) + (0xe400 | qz) = q - qz exactly, then multiplies by
+// the scale once (examples/dequantize_gemm/quantize/lop3.py:339-354); fp16(qz) is exact for 0 <= qz <= 2048 and so
+// is q - fp16(qz), hence the "original" decoder fed with these zeros returns the same bits.
+// PACKED = false: one int16 per group (lop3.py:339-341 reads `int16_t zero_r = *((int16_t*)zeros)`).
+// PACKED = true: 4-bit zero points, two per byte, group g in bits 4 (g % 2) of byte g / 2 of the row
+// (lop3.py:381-385: `(qzeros >> (group_offset * 4)) & 0xf`).
+template <bool PACKED>
+__global__ __launch_bounds__(256) void unpack_qzeros_kernel(const void* __restrict__ QZ, half_t* __restrict__ Z, int N,
+                                                            int groups) {
+  const size_t total = (size_t)N * groups;
+  const int row_bytes = (groups + 1) / 2;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    int qz;
+    if constexpr (PACKED) {
+      const size_t n = i / groups;
+      const int g = (int)(i - n * groups);
+      qz = (((const uint8_t*)QZ)[n * row_bytes + (g >> 1)] >> (4 * (g & 1))) & 0xF;
+    } else {
+      qz = ((const int16_t*)QZ)[i];
+    }
+    Z[i] = (half_t)(float)qz;
+  }
+}
+
+}  // namespace
+
+int unpack_qzeros(const void* QZ, void* Z, int N, int groups, int packed, hipStream_t stream) {
+  const size_t total = (size_t)N * groups;
+  const unsigned blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+  if (packed) hipLaunchKernelGGL(unpack_qzeros_kernel<true>, dim3(blocks), dim3(256), 0, stream, QZ, (half_t*)Z, N, groups);
+  else hipLaunchKernelGGL(unpack_qzeros_kernel<false>, dim3(blocks), dim3(256), 0, stream, QZ, (half_t*)Z, N, groups);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 }  // namespace dq

@@ -18,6 +18,7 @@ from .adapter import KernelAdapter, KernelParam
 # ---- enums of include/dqgemm.h -------------------------------------------------------------
 W4_UNSIGNED, W4_SIGNED, W4_OFFSET8, W4_SCALE, W4_USCALE, W4_ZEROS_ORIGINAL, W4_ZEROS_RESCALE = range(7)
 LAYOUT_PLAIN, LAYOUT_INTERLEAVED = 0, 1
+I4_UNSIGNED, I4_TWOS, I4U_INTERLEAVED, I4S_INTERLEAVED = range(4)
 
 _DTYPES = {
     "float16": torch.float16,
@@ -43,7 +44,7 @@ def _w4_mode(source_format: str, fast_decoding: bool, with_scaling: bool, with_z
         if not with_scaling:
             raise ValueError("with_zeros requires with_scaling")
         if zeros_mode in ("original", "quantized"):
-            # "quantized" zeros are integers: (q - qz) is exact either way
+            # "quantized": integer zero points, unpacked to fp16 in front of the kernel (see _zeros_params)
             return W4_ZEROS_ORIGINAL
         if zeros_mode == "rescale":
             return W4_ZEROS_RESCALE
@@ -55,6 +56,31 @@ def _w4_mode(source_format: str, fast_decoding: bool, with_scaling: bool, with_z
     # the example's slow path sign-extends the nibble whatever source_format says
     # (examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:121-124)
     return W4_SIGNED
+
+
+QZEROS_INT16, QZEROS_PACKED4 = 0, 1
+
+
+def _zeros_params(N: int, groups: int, zeros_mode: str, qzeros_format: str):
+    """Parameters that carry the zero points: ``(Zeros as the caller passes it, fp16 workspace or None, format)``.
+
+    ``"original"`` / ``"rescale"``: fp16 ``Zeros[N, groups]``.  ``"quantized"``
+    (examples/dequantize_gemm/quantize/lop3.py:326-420): integer zero points, ``qzeros_format="int16"`` for
+    ``Zeros[N, groups]`` int16 (the ``int16_t zero_r`` of :339-341) or ``"packed4"`` for 4-bit zero points two per
+    byte, ``Zeros[N, ceil(groups / 2)]`` (:381-385); they are unpacked to fp16 into a workspace in front of the
+    kernel, which then runs its ``(q - z) * s`` decoder: the same bits, since ``q - qz`` is exact either way.
+    """
+    if zeros_mode != "quantized":
+        return KernelParam("Zeros", torch.float16, (N, groups)), None, None
+    if qzeros_format == "int16":
+        zp = KernelParam("Zeros", torch.int16, (N, groups))
+        fmt = QZEROS_INT16
+    elif qzeros_format == "packed4":
+        zp = KernelParam("Zeros", torch.uint8, (N, (groups + 1) // 2), packed=True)
+        fmt = QZEROS_PACKED4
+    else:
+        raise ValueError(f"unknown qzeros_format {qzeros_format!r} (expected 'int16' or 'packed4')")
+    return zp, KernelParam("ZerosFp16", torch.float16, (N, groups)), fmt
 
 
 def dequantize_gemv(
@@ -78,6 +104,7 @@ def dequantize_gemv(
     zeros_mode: str = "original",
     variant: int = -1,
     _formula_fast: bool | None = None,
+    qzeros_format: str = "int16",
 ) -> KernelAdapter:
     """W4A16 decode GEMV / small-batch GEMM: ``C[M,N] = A[M,K] @ dequant(B[N,K/2]).T``.
 
@@ -128,19 +155,27 @@ def dequantize_gemv(
     ]
     if with_scaling:
         params.append(KernelParam("Scale", torch.float16, (N, groups)))
+    zwork, zfmt = None, None
     if with_zeros:
-        params.append(KernelParam("Zeros", torch.float16, (N, groups)))
+        zparam, zwork, zfmt = _zeros_params(N, groups, zeros_mode, qzeros_format)
+        params.append(zparam)
+    c_idx = len(params)
     params.append(KernelParam("C", torch.float16, (M, N)))
+    if zwork is not None:
+        params.append(zwork)
 
     def launch(ptrs, stream):
         lib = _lib.get_library()
         a, b = ptrs[0], ptrs[1]
         s = ptrs[2] if with_scaling else None
         z = ptrs[3] if with_zeros else None
-        c = ptrs[-1]
-        return lib.call_dequantize_gemv_w4a16(a, b, s, z, c, M, N, K, group_size, mode, layout, variant, stream)
+        if zwork is not None:
+            if lib.call_unpack_qzeros(z, ptrs[-1], N, groups, zfmt, stream) != 0:
+                return -1
+            z = ptrs[-1]
+        return lib.call_dequantize_gemv_w4a16(a, b, s, z, ptrs[c_idx], M, N, K, group_size, mode, layout, variant, stream)
 
-    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
+    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error, workspace_idx=[-1] if zwork is not None else [])
 
 
 def _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dtype, source_format, fast_decoding,
@@ -148,7 +183,9 @@ def _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dty
     """The integer branch of :func:`dequantize_gemv` (``use_dp4a``: int8 activations, int32 accumulation,
     examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:47-48,126-133): ``C[M,N] int32 = A[M,K] int8 .
     decode(B)^T``, exact.  Two bits: every decoder and the ``interleave_weight(B, 2, "int8")`` layout of the fast path
-    (the BitNet decode kernel is this case); four bits: the slow path (two's-complement nibbles)."""
+    (the BitNet decode kernel is this case); four bits: the slow path (two's-complement nibbles) and the fast path on
+    ``interleave_weight(B, 4, "int8")`` words (``"uint"``: ``w = q``; ``"int"``: ``w = q - 7``, the constant of the
+    reference's decode_i4s_to_i8s)."""
     if _dtype(accum_dtype) != torch.int32 or _dtype(out_dtype) != torch.int32:
         raise ValueError("dequantize_gemv: int8 activations accumulate and return int32")
     if with_scaling or with_zeros:
@@ -167,11 +204,13 @@ def _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dty
             return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, layout, None, 1.0, 0, stream)
 
     elif num_bits == 4:
-        if fast_decoding:
-            raise ValueError("dequantize_gemv: int8 x int4 is built for the slow path only (fast_decoding=False)")
+        # slow path: two's-complement nibbles, plain words.  Fast path: the words went through
+        # interleave_weight(B, 4, "int8") and decode as decode_i4u_to_i8s (w = q) or decode_i4s_to_i8s (w = q - 7)
+        # (examples/dequantize_gemm/quantize/lop3.py:999-1047)
+        dec = I4_TWOS if not fast_decoding else (I4S_INTERLEAVED if source_format == "int" else I4U_INTERLEAVED)
 
         def launch(ptrs, stream):
-            return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, 1, 0, 0, stream)
+            return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, dec, 0, 0, stream)
 
     else:
         raise ValueError("dequantize_gemv: int8 activations are built for num_bits 4 and 2")
@@ -239,6 +278,7 @@ def dequantize_w4(
     zeros_mode: str = "original",
     storage_dtype="int8",
     _formula_fast: bool | None = None,
+    qzeros_format: str = "int16",
 ) -> KernelAdapter:
     """Dequantised weight tile ``W[N,K] fp16 = decode(B[N,K/2][, Scale[, Zeros]])``.
 
@@ -255,17 +295,26 @@ def dequantize_w4(
     params = [KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True)]
     if with_scaling:
         params.append(KernelParam("Scale", torch.float16, (N, groups)))
+    zwork, zfmt = None, None
     if with_zeros:
-        params.append(KernelParam("Zeros", torch.float16, (N, groups)))
+        zparam, zwork, zfmt = _zeros_params(N, groups, zeros_mode, qzeros_format)
+        params.append(zparam)
+    w_idx = len(params)
     params.append(KernelParam("W", torch.float16, (N, K)))
+    if zwork is not None:
+        params.append(zwork)
 
     def launch(ptrs, stream):
         lib = _lib.get_library()
         s = ptrs[1] if with_scaling else None
         z = ptrs[2] if with_zeros else None
-        return lib.call_dequantize_w4(ptrs[0], s, z, ptrs[-1], N, K, group_size, mode, layout, stream)
+        if zwork is not None:
+            if lib.call_unpack_qzeros(z, ptrs[-1], N, groups, zfmt, stream) != 0:
+                return -1
+            z = ptrs[-1]
+        return lib.call_dequantize_w4(ptrs[0], s, z, ptrs[w_idx], N, K, group_size, mode, layout, stream)
 
-    return KernelAdapter("dequantize_w4", params, [-1], launch, _lib.last_error)
+    return KernelAdapter("dequantize_w4", params, [w_idx], launch, _lib.last_error, workspace_idx=[-1] if zwork is not None else [])
 
 
 FP4_E2M1, FP4_SIMPLE, FP4_TWIDDLING = 0, 1, 2
@@ -416,6 +465,59 @@ def matmul_fp16_fp4(
     return KernelAdapter("matmul_fp16_fp4_splitk", params, [2], launch_split, _lib.last_error, workspace_idx=[3])
 
 
+_DT_CODE = {torch.float16: 0, torch.bfloat16: 1, torch.int8: 2, torch.float32: 3, torch.int32: 4}
+
+
+def matmul(
+    M: int,
+    N: int,
+    K: int,
+    block_M: int = 128,
+    block_N: int = 128,
+    block_K: int = 32,
+    trans_A: bool = False,
+    trans_B: bool = True,
+    in_dtype="float16",
+    out_dtype="float16",
+    accum_dtype="float32",
+    num_stages: int = 0,
+    threads: int = 128,
+    k_pack: int = 1,
+) -> KernelAdapter:
+    """Plain GEMM on the MFMA tile the dequantize GEMMs share: ``C[M,N] = op(A) @ op(B)``, ``C = kernel(A, B)``.
+
+    Same arguments as ``matmul`` of testing/python/kernel/test_tilelang_kernel_gemm.py:5-49 (``k_pack`` from
+    testing/python/amd/test_tilelang_test_amd.py:7-22): ``A`` is ``[K,M]`` when ``trans_A`` else ``[M,K]``, ``B`` is
+    ``[N,K]`` when ``trans_B`` else ``[K,N]``.  float16 / bfloat16 inputs give an output of the same type or
+    float32; int8 gives int32 (exact).  Accumulation is always fp32 / int32.  Tile, stage, thread and k_pack
+    arguments are accepted and ignored.
+    """
+    it, ot = _dtype(in_dtype), _dtype(out_dtype)
+    if it not in (torch.float16, torch.bfloat16, torch.int8):
+        raise ValueError(f"matmul: in_dtype must be float16, bfloat16 or int8 (got {in_dtype})")
+    if (it == torch.int8 and ot != torch.int32) or (it != torch.int8 and ot not in (it, torch.float32)):
+        raise ValueError(f"matmul: out_dtype {out_dtype} does not go with in_dtype {in_dtype}")
+    kmult = 128 if it == torch.int8 else 64
+    if K % kmult != 0:
+        raise ValueError(f"matmul: K={K} must be a multiple of {kmult}")
+    esz = 1 if it == torch.int8 else 2
+    ws_bytes = (((M * K * esz + 255) // 256 * 256) if trans_A else 0) + (0 if trans_B else (N * K * esz + 255) // 256 * 256)
+    params = [
+        KernelParam("A", it, (K, M) if trans_A else (M, K)),
+        KernelParam("B", it, (N, K) if trans_B else (K, N)),
+        KernelParam("C", ot, (M, N)),
+    ]
+    if ws_bytes:
+        params.append(KernelParam("Workspace", torch.uint8, (ws_bytes,)))
+
+    def launch(ptrs, stream):
+        ws = ptrs[3] if ws_bytes else None
+        return _lib.get_library().call_gemm_plain(ptrs[0], ptrs[1], ptrs[2], ws, M, N, K, _DT_CODE[it], _DT_CODE[ot],
+                                                  int(trans_A), int(trans_B), stream)
+
+    return KernelAdapter("matmul", params, [2], launch, _lib.last_error, workspace_idx=[3] if ws_bytes else [])
+
+
 def matmul_w4_fine_grained(
     M: int,
     N: int,
@@ -463,7 +565,7 @@ def matmul_w4_fine_grained(
 
 def matmul_w4a16(M: int, N: int, K: int, group_size: int = -1, source_format: str = "int", fast_decoding: bool = False,
                  with_scaling: bool = True, with_zeros: bool = False, zeros_mode: str = "original",
-                 storage_dtype="int8") -> KernelAdapter:
+                 storage_dtype="int8", qzeros_format: str = "int16") -> KernelAdapter:
     """W4A16 GEMM for any M through the 256x256 MFMA kernel (tile-exact fp16 dequantisation):
     ``kernel(A, B[, Scale[, Zeros]], C)``, same decode options as :func:`dequantize_gemv`."""
     if group_size == -1:
@@ -476,16 +578,26 @@ def matmul_w4a16(M: int, N: int, K: int, group_size: int = -1, source_format: st
     params = [KernelParam("A", torch.float16, (M, K)), KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True)]
     if with_scaling:
         params.append(KernelParam("Scale", torch.float16, (N, groups)))
+    zwork, zfmt = None, None
     if with_zeros:
-        params.append(KernelParam("Zeros", torch.float16, (N, groups)))
+        zparam, zwork, zfmt = _zeros_params(N, groups, zeros_mode, qzeros_format)
+        params.append(zparam)
+    c_idx = len(params)
     params.append(KernelParam("C", torch.float16, (M, N)))
+    if zwork is not None:
+        params.append(zwork)
 
     def launch(ptrs, stream):
+        lib = _lib.get_library()
         s = ptrs[2] if with_scaling else None
         z = ptrs[3] if with_zeros else None
-        return _lib.get_library().call_dequant_gemm_w4_fp16(ptrs[0], ptrs[1], s, z, ptrs[-1], M, N, K, group_size, mode, layout, stream)
+        if zwork is not None:
+            if lib.call_unpack_qzeros(z, ptrs[-1], N, groups, zfmt, stream) != 0:
+                return -1
+            z = ptrs[-1]
+        return lib.call_dequant_gemm_w4_fp16(ptrs[0], ptrs[1], s, z, ptrs[c_idx], M, N, K, group_size, mode, layout, stream)
 
-    return KernelAdapter("matmul_w4a16", params, [], launch, _lib.last_error)
+    return KernelAdapter("matmul_w4a16", params, [], launch, _lib.last_error, workspace_idx=[-1] if zwork is not None else [])
 
 
 def matmul_int8xint4(
