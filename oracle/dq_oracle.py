@@ -20,6 +20,12 @@ How each function is pinned (see tests/test_oracle_pins.py):
 * e2m1 encode/pack against
   testing/python/quantize/test_tilelang_quantize_nvfp4_scale_layout.py:881-887;
 * packing by round trip and by ``fast_decode(interleave(p)) == plain_decode(p)``;
+* ``decode_fp4_simple_bf16_bits``, ``decode_fp4_twiddling``, ``interleave_weight`` and ``general_compress`` also
+  against vectors the reference's own torch helpers wrote (tests/golden/reference_vectors.npz: all 256 bytes, all
+  65536 byte pairs, 4096 seeded words, seeded codes);
+* the rounding order of the scaled / zero-point uint4 decoders and of the BitLinear epilogue against the operation
+  order of the device snippets written out with exact rationals and an explicit round-to-nearest-even per fp16 /
+  fp32 instruction;
 * matmuls by reduction to int64 / float64 brute force on tiny shapes.
 
 Parity unpinned by any reference test or fixture (no in-tree caller exists; the

@@ -681,3 +681,63 @@ def test_dequant_lowbit_rounding_order():
     got_r = orc.dequant_lowbit(packed, 2, "unsigned", s, z, 4, "rescale").astype(np.float64)[0]
     np.testing.assert_array_equal(got_r, f16(f16(c * float(s[0, 0])) - float(z[0, 0])))
     assert not np.array_equal(got_r, f16(c * float(s[0, 0]) - float(z[0, 0])))  # a single rounding would differ
+
+
+# ---- vectors written by the reference's own pure-torch helpers (tests/golden/make_vectors.py) ----------------------
+
+def _reference_vectors():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.npz")
+    return np.load(path, allow_pickle=False)
+
+
+def test_reference_vectors_torch_convert_all_bytes():
+    """examples/dequantize_gemm/dequantize_utils.py:57-84 run on every byte value, plain and with block exponents
+    that reach the clamp at 255."""
+    v = _reference_vectors()
+    np.testing.assert_array_equal(orc.decode_fp4_simple_bf16_bits(v["convert_in"]), v["convert_out_bits"])
+    np.testing.assert_array_equal(orc.decode_fp4_simple_bf16_bits(v["convert_in"], v["convert_scale"], 32), v["convert_scaled_out_bits"])
+
+
+def test_reference_vectors_bit_twiddling_all_units():
+    """examples/dequantize_gemm/dequantize_utils.py:4-54 run on all 65 536 byte pairs."""
+    v = _reference_vectors()
+    want = orc.bf16_bits_to_f32(v["twiddling_out_bits"])
+    got = orc.decode_fp4_twiddling(v["twiddling_in"])
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))  # bit for bit, signs of zeros included
+
+
+def test_reference_vectors_interleave_weight():
+    """examples/dequantize_gemm/quantize/utils.py:71-125 run on 4096 seeded words.  Its byte-shuffle branches raise
+    TypeError in torch (`torch.int32(...)` is not callable), so the reference itself yields vectors for three of the
+    six cases only; the other three stay pinned by fast_decode(interleave(p)) == plain_decode(p)."""
+    v = _reference_vectors()
+    words = v["interleave_in"]
+    for nbits, target in ((4, "float16"), (4, "int8"), (2, "int8")):
+        got = orc.interleave_weight(words.view(np.int8), nbits, target).view(np.int32)
+        np.testing.assert_array_equal(got, v[f"interleave_{nbits}_{target}"])
+    raised = [str(x) for x in v["interleave_cases_the_reference_raises_on"]]
+    assert len(raised) == 3 and all("not callable" in x for x in raised)
+
+
+def test_reference_vectors_general_compress():
+    """examples/dequantize_gemm/quantize/utils.py:50-67 run on seeded codes for 1, 2 and 4 bits."""
+    v = _reference_vectors()
+    for bits in (1, 2, 4):
+        got = orc.general_compress(v[f"compress_in_{bits}"], bits)
+        np.testing.assert_array_equal(got.view(np.uint8), v[f"compress_out_{bits}"].view(np.uint8))
+
+
+def test_reference_vectors_match_the_library_helpers():
+    """The package's own host helpers (tilelang_amd.quantize) against the same vectors."""
+    import torch
+
+    from tilelang_amd import quantize
+
+    v = _reference_vectors()
+    words = v["interleave_in"]
+    for nbits, target in ((4, "float16"), (4, "int8"), (2, "int8")):
+        got = quantize.interleave_weight(torch.from_numpy(words.copy()).view(torch.int8), nbits, target).numpy().view(np.int32)
+        np.testing.assert_array_equal(got, v[f"interleave_{nbits}_{target}"])
+    for bits in (1, 2, 4):
+        got = quantize.general_compress(torch.from_numpy(v[f"compress_in_{bits}"].copy()), source_bits=bits).numpy()
+        np.testing.assert_array_equal(got.view(np.uint8), v[f"compress_out_{bits}"].view(np.uint8))
