@@ -223,9 +223,11 @@ def test_streaming_small_batch_kernel(cuda, variant, mode):
 
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
 @pytest.mark.parametrize("M", [1, 4, 9, 16])
-def test_register_resident_kernel(cuda, M, mode, variant=40):
+@pytest.mark.parametrize("variant", [40, 41, 42])
+def test_register_resident_kernel(cuda, M, mode, variant):
     """Activations resident in registers (M <= 16, K = 2048 / 4096 / 8192): one row block per workgroup and
-    several, both layouts."""
+    several, both layouts.  40: every weight rounded to fp16 as the reference's tile; 41: scale and zero point
+    applied per group in fp32."""
     _run_gemv(cuda, M, 16 * 37, 4096, 128, mode, variant=variant)
     _run_gemv(cuda, M, 48, 8192, 128, mode, variant=variant, interleaved=(mode in ("scale", "original")))
     _run_gemv(cuda, M, 16 * 600, 2048, 128, mode, variant=variant)  # more row blocks than workgroups
