@@ -223,7 +223,7 @@ def test_streaming_small_batch_kernel(cuda, variant, mode):
 
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
 @pytest.mark.parametrize("M", [1, 4, 9, 16])
-@pytest.mark.parametrize("variant", [40, 41, 42])
+@pytest.mark.parametrize("variant", [40, 41, 42, 43])
 def test_register_resident_kernel(cuda, M, mode, variant):
     """Activations resident in registers (M <= 16, K = 2048 / 4096 / 8192): one row block per workgroup and
     several, both layouts.  40: every weight rounded to fp16 as the reference's tile; 41: scale and zero point

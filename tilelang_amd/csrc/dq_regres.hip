@@ -196,7 +196,14 @@ constexpr uint32_t kOutOfRange = 0xFFFFF000u;   // an offset no matrix of this k
 // therefore straight-line code, and the waits the compiler places in front of each chunk count exactly the loads
 // that were issued after that chunk's (a load behind a branch makes it wait for all of them at the loop's end,
 // which exposes the whole memory latency once per row block).
-template <int WAVES, int NC, int DEPTH, int PARK, bool HAS_SCALE, bool HAS_ZEROS, bool FLIP, bool APERM>
+//
+// TR (one block in flight): the weights are fetched row-contiguously -- an instruction reads 1024 / S rows x S bytes,
+// S = 64 NC the bytes of a row in the wave's K slice (4 rows x 256 bytes at K = 8192) -- which streams at 6.0 TB/s
+// where the matrix instruction's own operand layout (16 rows x 64 bytes per instruction) streams at 4.8 TB/s, and a
+// block is transposed into that layout through a 16 S-byte LDS area of the wave's own: 16-byte writes as loaded,
+// 16-byte reads as multiplied, the pieces of row r XOR-swizzled with r so that neither side has bank conflicts.
+// LDS operations of one wave execute in order, so no barrier and no second area is needed.
+template <int WAVES, int NC, int DEPTH, int PARK, bool TR, bool HAS_SCALE, bool HAS_ZEROS, bool FLIP, bool APERM>
 __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                         const half_t* __restrict__ S, const half_t* __restrict__ Z,
                                                                         half_t* __restrict__ C, int M, int N, int K, int rbn,
@@ -210,6 +217,10 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   constexpr int kSzRow = 136;
   __shared__ __align__(16) unsigned char sz_lds[2][2][16 * kSzRow + 16];  // + a word that idle threads write to
   constexpr int NR = NC - PARK;  // chunks whose activations stay in registers
+  static_assert(!TR || DEPTH == 1, "the transposing form keeps one block in flight");
+  constexpr int LPR = 4 * NC;    // TR: lanes (16-byte pieces) per row of the wave's slice
+  constexpr int RPI = 64 / LPR;  // TR: rows per load instruction
+  __shared__ uint4_t wstage[TR ? WAVES : 1][TR ? 16 * LPR : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -235,7 +246,8 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   uint32_t s_stage = 0, z_stage = 0;
   Halves<NC> sc, zp;
   // per-lane byte offsets inside a row block (N is a multiple of 16 here); the block's own offset is uniform
-  const uint32_t w_voff = (uint32_t)r * row_bytes + (uint32_t)chunk0 * 64u + (uint32_t)g * 16u;
+  const uint32_t w_voff = TR ? (uint32_t)(lane / LPR) * row_bytes + (uint32_t)chunk0 * 64u + (uint32_t)(lane % LPR) * 16u
+                             : (uint32_t)r * row_bytes + (uint32_t)chunk0 * 64u + (uint32_t)g * 16u;
   const uint32_t sz_dwords = 8u * groups_per_row;  // dwords of scales of one row block
   const uint32_t s_voff = (uint32_t)tid < sz_dwords ? (uint32_t)tid * 4u : kOutOfRange;
   const int sz_shift = 31 - __builtin_clz(groups_per_row >> 1);  // log2(dwords of scales per row); K / 256 is a power of two here
@@ -243,8 +255,19 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   auto w_soff = [&](int rb) { return rb < nrb_wg ? (uint32_t)(rb0 + rb) * 16u * row_bytes : kOutOfRange; };
   auto s_soff = [&](int rb) { return rb < nrb_wg ? (uint32_t)(rb0 + rb) * 32u * groups_per_row : 0u; };
   auto load_chunk = [&](int d, int c, int rb) {
-    bq[d][c] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, w_voff + (uint32_t)c * 64u, w_soff(rb), 2 /* nt */);
+    if constexpr (TR) {  // load instruction c of the block: rows c RPI .. c RPI + RPI - 1
+      const uint32_t so = rb < nrb_wg ? (uint32_t)((rb0 + rb) * 16 + c * RPI) * row_bytes : kOutOfRange;
+      bq[d][c] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, w_voff, so, 2 /* nt */);
+    } else {
+      bq[d][c] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, w_voff + (uint32_t)c * 64u, w_soff(rb), 2 /* nt */);
+    }
   };
+  // TR: where load instruction i's 16 bytes go, and where chunk c's operand words of lane (g, r) are
+  auto stage_widx = [&](int i) {
+    const int row = i * RPI + lane / LPR, piece = lane % LPR;
+    return row * LPR + (piece ^ (row & (LPR - 1)));
+  };
+  auto stage_ridx = [&](int c) { return r * LPR + ((c * 4 + g) ^ (r & (LPR - 1))); };
   auto load_scales = [&](int rb) {  // into the staging registers (zeros past the buffer or past the block's values)
     if constexpr (HAS_SCALE) s_stage = __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, s_voff, s_soff(rb), 0);
     if constexpr (HAS_ZEROS) z_stage = __builtin_amdgcn_raw_buffer_load_b32(z_rsrc, s_voff, s_soff(rb), 0);
@@ -309,20 +332,37 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
       for (int i = 0; i < 4; ++i) total[i] = __builtin_fmaf(s, __builtin_fmaf(nz, asum[i], acc[i]), total[i]);
     };
     read_scales(rb);
+    if constexpr (TR) {
+      // the block as loaded goes to the wave's LDS area, and its registers take the next block at once
+#pragma unroll
+      for (int i = 0; i < NC; ++i) wstage[wave][stage_widx(i)] = bq[0][i];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NC; ++i) {
+        load_chunk(0, i, rb + 1);
+        if (i == 0) load_scales(rb + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       float4_t acc = {0.f, 0.f, 0.f, 0.f};
+      uint4_t wq;
+      if constexpr (TR) wq = wstage[wave][stage_ridx(c)];
+      else wq = bq[d][c];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint4_t a = c < NR ? y[c < NR ? c : 0][j] : ypark[wave][c < NR ? 0 : c - NR][j][lane];
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), decode_w4_bias64<FLIP>(bq[d][c][j]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), decode_w4_bias64<FLIP>(wq[j]), acc, 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
       if (c > 0) finish_group(c - 1, acc_prev);
-      // this chunk's registers are free: the same chunk, DEPTH blocks on (zeros from beyond the buffer after the
-      // workgroup's last block); the next block's scales and zeros travel behind the first chunk
-      load_chunk(d, c, rb + DEPTH);
-      if (c == 0) load_scales(rb + 1);
+      if constexpr (!TR) {
+        // this chunk's registers are free: the same chunk, DEPTH blocks on (zeros from beyond the buffer after the
+        // workgroup's last block); the next block's scales and zeros travel behind the first chunk
+        load_chunk(d, c, rb + DEPTH);
+        if (c == 0) load_scales(rb + 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
       acc_prev = acc;
     }
@@ -351,7 +391,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   }
 }
 
-template <int WAVES, int NC, int DEPTH, int PARK>
+template <int WAVES, int NC, int DEPTH, int PARK, bool TR>
 int launch_regres_fast(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int mode,
                        int layout, hipStream_t stream) {
   const int nrb = (N + 15) / 16;
@@ -359,7 +399,7 @@ int launch_regres_fast(const void* A, const void* B, const void* S, const void* 
   const dim3 grid((nrb + rbn - 1) / rbn), block(64 * WAVES);
   const bool plain = layout == LAYOUT_PLAIN;
 #define DQ_FAST2(HS, HZ, FL, AP, ZC)                                                                                        \
-  hipLaunchKernelGGL((w4a16_regres_fast_kernel<WAVES, NC, DEPTH, PARK, HS, HZ, FL, AP>), grid, block, 0, stream, (const half_t*)A, \
+  hipLaunchKernelGGL((w4a16_regres_fast_kernel<WAVES, NC, DEPTH, PARK, TR, HS, HZ, FL, AP>), grid, block, 0, stream, (const half_t*)A, \
                      (const uint8_t*)B, (const half_t*)S, (const half_t*)Z, (half_t*)C, M, N, K, rbn, ZC)
 #define DQ_FAST(HS, HZ, FL, ZC)                  \
   do {                                           \
@@ -423,17 +463,22 @@ int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, voi
   if (mode >= W4_SCALE && group != 128) return 1;
   if ((size_t)N * K / 2 >= (1ull << 32) - 8192) return 1;  // 32-bit offsets, and room for the out-of-range marker
   if (fast && mode != W4_ZEROS_RESCALE) {
-    // fast = 2: eight waves of 256 registers, two row blocks in flight; 1 (default): sixteen waves of 128 registers, one
-    // block in flight, one chunk of activations parked in LDS so that nothing spills
+    // fast = 1 (default): sixteen waves, row-contiguous loads transposed through LDS (at K = 2048 a wave's slice of a
+    // row is 64 bytes and the matrix instruction's own layout is already row-contiguous); 3: sixteen waves, loads in
+    // the matrix instruction's layout; 2: eight waves of 256 registers with two row blocks in flight, same layout
+    if (fast == 1) {
+      if (K == 8192) return launch_regres_fast<16, 4, 1, 0, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      if (K == 4096) return launch_regres_fast<16, 2, 1, 0, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    }
     if (fast != 2) {
-      if (K == 8192) return launch_regres_fast<16, 4, 1, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-      if (K == 4096) return launch_regres_fast<16, 2, 1, 0>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-      if (K == 2048) return launch_regres_fast<16, 1, 1, 0>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      if (K == 8192) return launch_regres_fast<16, 4, 1, 1, false>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      if (K == 4096) return launch_regres_fast<16, 2, 1, 0, false>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      if (K == 2048) return launch_regres_fast<16, 1, 1, 0, false>(A, B, S, Z, C, M, N, K, mode, layout, stream);
       return 1;
     }
-    if (K == 8192) return launch_regres_fast<8, 8, 2, 3>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    if (K == 4096) return launch_regres_fast<8, 4, 2, 0>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    if (K == 2048) return launch_regres_fast<8, 2, 2, 0>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    if (K == 8192) return launch_regres_fast<8, 8, 2, 3, false>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    if (K == 4096) return launch_regres_fast<8, 4, 2, 0, false>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    if (K == 2048) return launch_regres_fast<8, 2, 2, 0, false>(A, B, S, Z, C, M, N, K, mode, layout, stream);
     return 1;
   }
   if (K == 8192) return launch_regres<4>(A, B, S, Z, C, M, N, K, mode, layout, stream);
