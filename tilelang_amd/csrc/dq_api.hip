@@ -131,7 +131,7 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   // choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with
   // register-resident activations (M <= 16).  0, 4, 5, 10: a configuration of the tiled MFMA fallback kernel
   // (covers every shape).
-  if ((variant >= 40 && variant <= 43) || (variant < 0 && M >= 3 && M <= 16)) {
+  if ((variant >= 40 && variant <= 43) || (variant < 0 && M >= 2 && M <= 16)) {
     // a handful of rows: activations resident in registers (shapes it does not cover fall through).  40: the form
     // that reproduces the fp16 rounding of every weight; 41 and the default: scale and zero point applied per
     // group in fp32, weights fetched row-contiguously and transposed through LDS; 43: the same with the weights

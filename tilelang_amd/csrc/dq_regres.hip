@@ -220,7 +220,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   static_assert(!TR || DEPTH == 1, "the transposing form keeps one block in flight");
   constexpr int LPR = 4 * NC;    // TR: lanes (16-byte pieces) per row of the wave's slice
   constexpr int RPI = 64 / LPR;  // TR: rows per load instruction
-  __shared__ uint4_t wstage[TR ? WAVES : 1][TR ? 16 * LPR : 1];
+  __shared__ uint4_t wstage[TR ? WAVES : 1][TR ? 256 : 1];  // 16 rows x up to 256 bytes per wave
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -302,9 +302,30 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       float4_t sum = {0.f, 0.f, 0.f, 0.f};
+      uint4_t dd[4];
+      if constexpr (TR) {
+        // the chunk's 16 rows x 256 bytes are fetched row-contiguously too (an instruction reads 4 rows x 256 bytes
+        // instead of 16-byte pieces of 32 cache lines) and transposed through the wave's LDS area
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = i * 4 + (lane >> 4);
+          const uint32_t vo = row < M ? ((uint32_t)row * (uint32_t)K + (uint32_t)chunk0 * 128u) * 2u + (uint32_t)(lane & 15) * 16u : kOutOfRange;
+          dd[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, vo + (uint32_t)(c * 256), 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = i * 4 + (lane >> 4);
+          wstage[wave][row * 16 + ((lane & 15) ^ row)] = dd[i];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dd[j] = wstage[wave][r * 16 + ((g * 4 + j) ^ r)];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dd[j] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + (uint32_t)(c * 256 + j * 16), 0, 0);
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        uint4_t d = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_voff + (uint32_t)(c * 256 + j * 16), 0, 0);
+        uint4_t d = dd[j];
         if constexpr (APERM) d = permute_k8_16bit(d);
         if (c < NR) y[c < NR ? c : 0][j] = d;
         else ypark[wave][c - NR][j][lane] = d;
