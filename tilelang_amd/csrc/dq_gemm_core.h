@@ -207,12 +207,17 @@ __device__ __forceinline__ void take_k_slice(Params& p, int& bid) {
 //   decode(const uint32_t* words, int j, const Scale&)  -> B operand of MFMA step j; `words` are
 //       the lane's kBRowBytes/2 packed bytes as dwords
 //   Epilogue: out_t, kTransposed, finish(acc value, p, m, n) -> value stored
-template <class P, int kMBW, int kNBW>
-__global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
+// kKSplit = 2: eight waves, two per SIMD; waves 4..7 are a second copy of the pipeline (LDS stages of their own) that
+// takes the odd k-blocks while waves 0..3 take the even ones, and hands its accumulators over once, through LDS,
+// after the loop.  For problems that give each CU one small tile with a long K (BitNet at M = 256): the second wave
+// of a SIMD runs its matrix instructions under the first one's decode and waits.  Needs an even number of k-blocks.
+template <class P, int kMBW, int kNBW, int kKSplit = 1>
+__global__ __launch_bounds__(kThreads * kKSplit, 1) void gemm_kernel(const Params p_in) {
   Params p = p_in;
   int bid = blockIdx.x;
   take_k_slice<P>(p, bid);
-  extern __shared__ __align__(16) unsigned char smem[];
+  extern __shared__ __align__(16) unsigned char smem_all[];
+  static_assert(kKSplit == 1 || kKSplit == 2, "one or two copies of the pipeline");
   constexpr int BM = 64 * kMBW, BN = 64 * kNBW;  // 2 x 2 waves of kMBW x kNBW blocks of 32 x 32 (shadow the 256 x 256 default)
   constexpr int kAStage = BM * kARowBytes;
   constexpr int kBStage = BN * P::kBRowBytes;
@@ -223,7 +228,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
   constexpr int kBWords = P::kBRowBytes / 8;                    // dwords per lane: 4 or 8
   constexpr int kALoads = (P::kAPacked ? 4 : 8) * BM / 256;     // 16-byte global loads of A per thread
 
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & (kThreads - 1);
+  const int kh = kKSplit == 1 ? 0 : (int)(threadIdx.x / kThreads);  // which copy of the pipeline
+  unsigned char* const smem = smem_all + kh * (3 * kStage);
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves
@@ -233,7 +240,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
   int tm, tn;
   tile_of_block(bid, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  const int KB = K / P::kKPerBlock;
+  const int KB = K / P::kKPerBlock / kKSplit;  // k-blocks of this copy: kb -> global k-block kb * kKSplit + kh
   const size_t a_row_bytes = P::kAPacked ? (size_t)(p.ldk >> 1) : (size_t)p.ldk * (kARowBytes / P::kKPerBlock == 2 ? 2 : 1);
   const size_t b_row_bytes = (size_t)p.ldk * P::kBRowBytes / P::kKPerBlock;
 
@@ -272,7 +279,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
   }
 
   uint4_t a_reg[kALoads], b_reg[kBLoads];
-  auto load_tile = [&](int kb) {
+  auto load_tile = [&](int kb_local) {
+    const int kb = kb_local * kKSplit + kh;
     const size_t a_step = P::kAPacked ? 64 : 128;
 #pragma unroll
     for (int i = 0; i < kALoads; ++i) a_reg[i] = *reinterpret_cast<const uint4_t*>(a_src[i] + (size_t)kb * a_step);
@@ -357,8 +365,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
   load_tile(0);
 #pragma unroll
   for (int nb = 0; nb < kNBW; ++nb) {
-    sc_c[nb] = P::prep_scale(P::fetch_scale(p, w_row[nb], 0, g), p);
-    sc_raw1[nb] = P::fetch_scale(p, w_row[nb], KB > 1 ? 1 : 0, g);
+    sc_c[nb] = P::prep_scale(P::fetch_scale(p, w_row[nb], kh, g), p);
+    sc_raw1[nb] = P::fetch_scale(p, w_row[nb], (KB > 1 ? 1 : 0) * kKSplit + kh, g);
   }
   store_tile(0);
   if (KB > 1) {
@@ -384,7 +392,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
     if (kb + 2 < KB) {
       store_tile(stage2);
 #pragma unroll
-      for (int nb = 0; nb < kNBW; ++nb) sc_raw2[nb] = P::fetch_scale(p, w_row[nb], kb + 2, g);
+      for (int nb = 0; nb < kNBW; ++nb) sc_raw2[nb] = P::fetch_scale(p, w_row[nb], (kb + 2) * kKSplit + kh, g);
     }
     if (kb + 3 < KB) load_tile(kb + 3);
     const bool has_next = kb + 1 < KB;
@@ -425,7 +433,27 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_kernel(const Params p_in) {
     __syncthreads();
   }
 
-  DQ_GEMM_EPILOGUE
+  if constexpr (kKSplit == 2) {
+    // the second copy hands its accumulators to the first: [wave][mb][nb][lane] behind the epilogue's slabs
+    constexpr int kSlabBytes = 4 * 32 * (32 * kNBW + 4) * 4;
+    typename P::acc_t* red = reinterpret_cast<typename P::acc_t*>(smem_all + ((kSlabBytes + 63) & ~63)) + wave * (kMBW * kNBW * 64) + lane;
+    if (kh == 1) {
+#pragma unroll
+      for (int mb = 0; mb < kMBW; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < kNBW; ++nb) red[(mb * kNBW + nb) * 64] = acc[mb][nb];
+    }
+    __syncthreads();  // (the loop's last barrier already saw every wave done with the stages this area overlays)
+    if (kh == 1) return;
+#pragma unroll
+    for (int mb = 0; mb < kMBW; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < kNBW; ++nb) acc[mb][nb] = acc[mb][nb] + red[(mb * kNBW + nb) * 64];
+  }
+  {
+    unsigned char* const smem = smem_all;  // the slabs of the epilogue start at the front
+    DQ_GEMM_EPILOGUE
+  }
 }
 
 // ---- direct-to-LDS variant ---------------------------------------------------------------------
@@ -826,21 +854,23 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   DQ_GEMM_EPILOGUE
 }
 
-template <class P, int kMBW = 4, int kNBW = 4>
+template <class P, int kMBW = 4, int kNBW = 4, int kKSplit = 1>
 int launch(Params p, hipStream_t stream) {
   constexpr int kTileM = 64 * kMBW, kTileN = 64 * kNBW;
-  constexpr int kPipe = 3 * (kTileM * kARowBytes + kTileN * P::kBRowBytes);
-  constexpr int kSlabs = 4 * 32 * (32 * kNBW + 4) * 4;  // epilogue staging
+  constexpr int kPipe = kKSplit * 3 * (kTileM * kARowBytes + kTileN * P::kBRowBytes);
+  // epilogue staging, and behind it the accumulators the second copy of the pipeline hands over
+  constexpr int kSlabs = ((4 * 32 * (32 * kNBW + 4) * 4 + 63) & ~63) + (kKSplit - 1) * 4 * kMBW * kNBW * 64 * 64;
   constexpr int kLds = kPipe > kSlabs ? kPipe : kSlabs;
+  static_assert(kLds <= 160 * 1024, "LDS budget");
   p.tiles_m = (p.M + kTileM - 1) / kTileM;
   p.tiles_n = (p.N + kTileN - 1) / kTileN;
-  auto kern = gemm_kernel<P, kMBW, kNBW>;
+  auto kern = gemm_kernel<P, kMBW, kNBW, kKSplit>;
   static bool lds_limit_raised = false;  // once per kernel: legal under stream capture afterwards
   if (!lds_limit_raised) {
     DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
     lds_limit_raised = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(kThreads), kLds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(kThreads * kKSplit), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }
@@ -853,6 +883,12 @@ int launch_auto(const Params& p, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.split; };
   if (tiles(256, 256) >= 192) return launch<P, 4, 4>(p, stream);
   if (tiles(128, 128) >= 192) return launch<P, 2, 2>(p, stream);
+  // at most about one small tile per CU and a long K: two copies of the pipeline per workgroup, on alternate
+  // k-blocks (int8 x 2-bit at M = 256, N = K = 8192: 35 -> 28.5 us).  Integer accumulation only: there the order
+  // of the K sum does not show, while a float result would no longer match the other tile shapes bit for bit.
+  if constexpr (P::kBRowBytes <= 64 && std::is_same<typename P::acc_t, int16_t_>::value) {
+    if (tiles(128, 64) <= 320 && (p.K / P::kKPerBlock) % 2 == 0 && p.K / P::kKPerBlock >= 8) return launch<P, 2, 1, 2>(p, stream);
+  }
   return launch<P, 2, 1>(p, stream);
 }
 
