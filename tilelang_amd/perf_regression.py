@@ -22,6 +22,7 @@ from dataclasses import dataclass
 
 RESULTS_JSON_PREFIX = "__TILELANG_PERF_RESULTS_JSON__="
 MAX_RETRIES = 5
+_CASE_PREFIX = "regression_"
 
 
 @dataclass(frozen=True)
@@ -30,93 +31,113 @@ class PerfResult:
     latency: float
     case: str | None = None
 
+    def as_json_item(self) -> dict:
+        item = {"name": self.name, "latency": self.latency}
+        if self.case is not None:
+            item["case"] = self.case
+        return item
 
-_results: list[PerfResult] = []
-_current_case: str | None = None
+
+class _Recorder:
+    """What one run of :func:`regression` collects: the results so far and the case they belong to."""
+
+    def __init__(self):
+        self.items: list[PerfResult] = []
+        self.case: str | None = None
+
+    def add(self, name: str, latency: float) -> None:
+        self.items.append(PerfResult(name, latency, self.case))
+
+    def write(self, stream) -> None:
+        as_json = os.environ.get("TL_PERF_REGRESSION_FORMAT", "text").strip().lower() == "json"
+        if as_json:
+            payload = json.dumps([r.as_json_item() for r in self.items], separators=(",", ":"))
+            print(RESULTS_JSON_PREFIX + payload, file=stream)
+        else:
+            for r in self.items:
+                print(f"{r.name}: {r.latency}", file=stream)
+
+
+_recorder = _Recorder()
 
 
 def results() -> list[PerfResult]:
     """The results recorded since the last :func:`regression` started."""
-    return list(_results)
+    return list(_recorder.items)
 
 
-def _only_filters() -> list[str]:
-    raw = os.environ.get("TL_PERF_REGRESSION_ONLY", "").strip()
-    if not raw:
-        return []
-    try:
-        parsed = json.loads(raw)
-    except json.JSONDecodeError:
-        parsed = raw.split(",")
-    if isinstance(parsed, str):
-        parsed = [parsed]
-    if not isinstance(parsed, list):
-        return []
-    return [str(p).strip() for p in parsed if str(p).strip()]
+def _strip_prefix(name: str) -> str:
+    return name[len(_CASE_PREFIX):] if name.startswith(_CASE_PREFIX) else name
 
 
-def _selected(case: str, filters: list[str]) -> bool:
-    if not filters:
-        return True
-    names = (case.lower(), ("regression_" + case).lower())
-    return any(fnmatch.fnmatch(n, f.lower()) or f.lower() in n for f in filters for n in names)
+def _case_selector():
+    """Predicate on a case's function name built from ``TL_PERF_REGRESSION_ONLY``: a JSON list (or one JSON string)
+    or a comma-separated list of patterns; a pattern selects a case when it is a glob match or a substring of the
+    function name or of the name without ``regression_``, case-insensitively.  No patterns: every case."""
+    spec = os.environ.get("TL_PERF_REGRESSION_ONLY", "").strip()
+    patterns: list[str] = []
+    if spec:
+        try:
+            decoded = json.loads(spec)
+        except json.JSONDecodeError:
+            decoded = spec.split(",")
+        if isinstance(decoded, str):
+            decoded = [decoded]
+        if isinstance(decoded, list):
+            patterns = [text.lower() for text in (str(x).strip() for x in decoded) if text]
+
+    def wanted(func_name: str) -> bool:
+        if not patterns:
+            return True
+        for candidate in (func_name.lower(), _strip_prefix(func_name).lower()):
+            for pat in patterns:
+                if pat in candidate or fnmatch.fnmatch(candidate, pat):
+                    return True
+        return False
+
+    return wanted
 
 
 def process_func(func, name: str | None = None, /, **kwargs) -> None:
     """Run ``func(**kwargs)``, which returns a latency (any unit; only ratios matter), and record it under ``name``
     (default: the function's module, without a leading ``regression_``).  A non-positive latency is measured again,
-    up to five times, then dropped with a warning."""
-    label = getattr(func, "__module__", "<unknown>") if name is None else name
-    if label.startswith("regression_"):
-        label = label[len("regression_"):]
-    latency = float(func(**kwargs))
-    for _ in range(MAX_RETRIES):
-        if latency > 0.0:
-            break
+    up to five more times, then dropped with a warning."""
+    label = _strip_prefix(name if name is not None else getattr(func, "__module__", "<unknown>"))
+    latency = 0.0
+    for _attempt in range(1 + MAX_RETRIES):
         latency = float(func(**kwargs))
-    if latency <= 0.0:
-        warnings.warn(f"{label} has latency {latency} <= 0. Please verify the profiling results.", RuntimeWarning, 1)
-        return
-    _results.append(PerfResult(label, latency, _current_case))
+        if latency > 0.0:
+            _recorder.add(label, latency)
+            return
+    warnings.warn(f"{label} has latency {latency} <= 0. Please verify the profiling results.", RuntimeWarning, 1)
 
 
 def emit_results(stream=None) -> None:
-    stream = stream or sys.stdout
-    if os.environ.get("TL_PERF_REGRESSION_FORMAT", "text").strip().lower() == "json":
-        items = []
-        for r in _results:
-            item = {"name": r.name, "latency": r.latency}
-            if r.case is not None:
-                item["case"] = r.case
-            items.append(item)
-        print(RESULTS_JSON_PREFIX + json.dumps(items, separators=(",", ":")), file=stream)
-        return
-    for r in _results:
-        print(f"{r.name}: {r.latency}", file=stream)
+    _recorder.write(stream or sys.stdout)
 
 
 def regression(prefixes=("regression_",), verbose: bool = True, namespace: dict | None = None) -> None:
-    """Run the ``regression_*`` callables of the calling module (or of ``namespace``) and emit the results."""
-    global _current_case
+    """Run the ``regression_*`` callables of the calling module (or of ``namespace``), in name order, and emit the
+    results.  Warnings raised inside a case are muted; a progress line per case goes to stdout when ``verbose``."""
     if namespace is None:
         namespace = inspect.currentframe().f_back.f_globals
-    _results.clear()
-    filters = _only_filters()
-    cases = sorted((k, v) for k, v in namespace.items() if callable(v) and any(k.startswith(p) for p in prefixes))
-    cases = [(k, v) for k, v in cases if _selected(k[len("regression_"):] if k.startswith("regression_") else k, filters)]
-    for idx, (name, fn) in enumerate(cases, 1):
-        _current_case = name[len("regression_"):] if name.startswith("regression_") else name
+    wanted = _case_selector()
+    todo = [name for name in sorted(namespace)
+            if callable(namespace[name]) and name.startswith(tuple(prefixes)) and wanted(name)]
+    _recorder.items.clear()
+    for position, func_name in enumerate(todo, start=1):
+        _recorder.case = _strip_prefix(func_name)
         if verbose:
-            print(f"  ├─ [{idx}/{len(cases)}] {_current_case}", end="", flush=True)
-        t0 = time.perf_counter()
+            print(f"  ├─ [{position}/{len(todo)}] {_recorder.case}", end="", flush=True)
+        started = time.perf_counter()
         try:
             with warnings.catch_warnings():
                 warnings.simplefilter("ignore")
-                fn()
+                namespace[func_name]()
             if verbose:
-                print(f" ({time.perf_counter() - t0:.2f}s)", flush=True)
+                print(f" ({time.perf_counter() - started:.2f}s)", flush=True)
         finally:
-            _current_case = None
+            _recorder.case = None
     emit_results()
 
 

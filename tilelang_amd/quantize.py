@@ -67,20 +67,23 @@ def interleave_weight(qweight: torch.Tensor, nbits: int = 4, target_dtype: str =
     return out.view(orig_dtype).reshape(orig_shape)
 
 
+def _require(ok: bool, exc, text: str) -> None:
+    if not ok:
+        raise exc(text)
+
+
 def pack_int4(tensor: torch.Tensor) -> torch.Tensor:
     """Logical signed int4 held in int8 -> two per byte, even index in the low nibble."""
-    if tensor.dtype != torch.int8:
-        raise TypeError(f"Expected torch.int8 logical int4 tensor, but got {tensor.dtype}.")
-    if tensor.ndim == 0 or tensor.shape[-1] % 2 != 0:
-        raise ValueError("The last dimension of a logical int4 tensor must be even for int8 packing.")
+    _require(tensor.dtype == torch.int8, TypeError, f"pack_int4 takes int8 values in -8..7, not {tensor.dtype}")
+    _require(tensor.ndim >= 1 and tensor.shape[-1] % 2 == 0, ValueError,
+             f"pack_int4 puts two values in a byte: the last dimension of {tuple(tensor.shape)} must be even")
     t = tensor.to(torch.int16)
     return ((t[..., ::2] & 0x0F) | ((t[..., 1::2] & 0x0F) << 4)).to(torch.uint8).view(torch.int8).contiguous()
 
 
 def encode_fp4_e2m1_values(values: torch.Tensor) -> torch.Tensor:
     """float -> raw e2m1 nibble codes (uint8)."""
-    if not isinstance(values, torch.Tensor):
-        raise TypeError(f"values must be a torch.Tensor, got {type(values)!r}")
+    _require(isinstance(values, torch.Tensor), TypeError, f"encode_fp4_e2m1_values takes a tensor, not {type(values).__name__}")
     x = torch.nan_to_num(values.to(torch.float32), nan=0.0, posinf=6.0, neginf=-6.0)
     bounds = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], device=x.device)
     mag = torch.bucketize(x.abs(), bounds, right=True).to(torch.int32)
@@ -90,25 +93,19 @@ def encode_fp4_e2m1_values(values: torch.Tensor) -> torch.Tensor:
 
 def pack_fp4_e2m1_codes(codes: torch.Tensor) -> torch.Tensor:
     """e2m1 codes [N, K] uint8 -> int8 storage [N, K/2], low nibble first."""
-    if not isinstance(codes, torch.Tensor):
-        raise TypeError(f"codes must be a torch.Tensor, got {type(codes)!r}")
-    if codes.dtype != torch.uint8:
-        raise TypeError(f"codes must have dtype torch.uint8, got {codes.dtype}")
-    if codes.ndim != 2:
-        raise ValueError(f"codes must be a 2D tensor, got shape {tuple(codes.shape)}")
-    if codes.shape[1] % 2 != 0:
-        raise ValueError(f"FP4 packing requires an even K dimension, got {tuple(codes.shape)}")
+    _require(isinstance(codes, torch.Tensor) and codes.dtype == torch.uint8, TypeError,
+             "pack_fp4_e2m1_codes takes a uint8 tensor of e2m1 codes")
+    _require(codes.ndim == 2 and codes.shape[1] % 2 == 0, ValueError,
+             f"pack_fp4_e2m1_codes takes [N, K] with K even (two codes per byte), not {tuple(codes.shape)}")
     return ((codes[:, 0::2] & 0x0F) | ((codes[:, 1::2] & 0x0F) << 4)).contiguous().view(torch.int8)
 
 
 def decode_packed_fp4_e2m1(packed: torch.Tensor, cols: int | None = None) -> torch.Tensor:
     """Packed e2m1 -> float32 values."""
-    if packed.ndim != 2:
-        raise ValueError(f"packed must be a 2D tensor, got shape {tuple(packed.shape)}")
-    if cols is None:
-        cols = packed.shape[1] * 2
-    if cols != packed.shape[1] * 2:
-        raise ValueError(f"cols must equal packed.shape[1] * 2, got cols={cols}, packed shape={tuple(packed.shape)}")
+    _require(packed.ndim == 2, ValueError, f"decode_packed_fp4_e2m1 takes [N, K/2] bytes, not {tuple(packed.shape)}")
+    width = 2 * packed.shape[1]
+    _require(cols is None or cols == width, ValueError, f"{packed.shape[1]} bytes per row hold {width} codes, not {cols}")
+    cols = width
     u = packed.contiguous().view(torch.uint8)
     lut = torch.tensor(FP4_E2M1_VALUES, device=packed.device, dtype=torch.float32)
     nib = torch.stack((u & 0x0F, u >> 4), dim=-1).reshape(packed.shape[0], cols)
