@@ -12,6 +12,15 @@ namespace dq {
 static char g_error_buf[kErrorBufSize];
 char* error_buf() { return g_error_buf; }
 
+// Filled by the initialisers of LdsRequest<BYTES>::registered while the library loads (zero-initialised
+// before any of them runs).
+static int g_largest_lds_request;
+int register_lds_request(int bytes) {
+  if (bytes > g_largest_lds_request) g_largest_lds_request = bytes;
+  return bytes;
+}
+int largest_lds_request() { return g_largest_lds_request; }
+
 // kernels (defined in the .hip files next to this one)
 int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int fast, hipStream_t stream);
@@ -57,7 +66,6 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // address comes from hipGetSymbolAddress, once per device with that device current.
 constexpr size_t kStaticScratchBytes = DQ_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
-constexpr int kMaxDevices = 64;
 static void* g_scratch_ptr[kMaxDevices];
 
 static int scratch_of_current_device(const char* fn, void** out) {
@@ -106,9 +114,8 @@ extern "C" int init(void) {
     DQ_FAIL("init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
   int max_lds = 0;
   DQ_CHECK_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device));
-  const int kLargestLdsRequest = 160 * 1024;
-  if (kLargestLdsRequest > max_lds)
-    DQ_FAIL("Requested dynamic shared memory %d exceeds device limit %d", kLargestLdsRequest, max_lds);
+  if (largest_lds_request() > max_lds)
+    DQ_FAIL("Requested dynamic shared memory %d exceeds device limit %d", largest_lds_request(), max_lds);
   void* scratch_ptr = nullptr;
   if (scratch_of_current_device("init", &scratch_ptr)) return -1;
   return 0;

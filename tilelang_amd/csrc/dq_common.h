@@ -38,6 +38,34 @@ char* error_buf();  // static 1024-byte buffer, as in the reference adapter's ge
     if (e__ != hipSuccess) DQ_FAIL("%s failed: %s", #expr, hipGetErrorString(e__)); \
   } while (0)
 
+// ---- host side: dynamic LDS requests ------------------------------------------------------------------
+// A kernel that asks for more than 64 KiB of dynamic LDS needs its limit raised with hipFuncSetAttribute, once
+// per kernel and per device (the attribute belongs to the kernel's code object on that device).  Every launcher
+// does so through raise_lds_limit<BYTES>; instantiating it also enters BYTES into a table that is filled while
+// the library loads, so init() can compare the largest request of any kernel built into the library with what
+// the device offers before anything is launched.
+constexpr int kMaxDevices = 64;
+int register_lds_request(int bytes);  // returns bytes
+int largest_lds_request();
+
+template <int BYTES>
+struct LdsRequest {
+  static inline const int registered = register_lds_request(BYTES);
+};
+
+template <int BYTES, class Kernel>
+int raise_lds_limit(Kernel kern, bool (&raised)[kMaxDevices]) {
+  (void)LdsRequest<BYTES>::registered;  // forces the load-time registration of this instantiation
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
+  if (!raised[device]) {  // afterwards the launch makes no attribute call: legal under stream capture
+    DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, BYTES));
+    raised[device] = true;
+  }
+  return 0;
+}
+
 // ---- weight formats / modes (values are part of the C-ABI, see include/dqgemm.h) --
 enum W4Mode : int {
   W4_UNSIGNED = 0,        // w = q

@@ -466,6 +466,13 @@ __global__ __launch_bounds__(kThreads * kKSplit, 1) void gemm_kernel(const Param
 // loads are issued from inline assembly and tracked by hand (one s_waitcnt vmcnt per tile): the
 // kernel issues no other vector-memory load inside the main loop, so the counter only ever
 // holds these.  Requires K % 128 == 0 and A, B smaller than 4 GiB (32-bit lane offsets).
+//
+// M0 is written inside the statement and is not on its clobber list: clang treats M0 as a reserved register,
+// warns that a reserved register on a clobber list "may not be preserved" and promises nothing for it.  What
+// keeps this sound is that the statement sets M0 itself immediately before the one instruction that reads it,
+// and that nothing else in these kernels depends on M0 across the statement: they use no other LDS-direct load,
+// no GWS / sendmsg, no indirect register indexing and no v_readlane / v_writelane with M0 as the lane select,
+// and gfx950 LDS instructions do not read M0 (that was the pre-gfx9 bounds clamp).
 __device__ __forceinline__ void dma16(unsigned lds_addr, unsigned voff, const void* sbase) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
@@ -865,11 +872,8 @@ int launch(Params p, hipStream_t stream) {
   p.tiles_m = (p.M + kTileM - 1) / kTileM;
   p.tiles_n = (p.N + kTileN - 1) / kTileN;
   auto kern = gemm_kernel<P, kMBW, kNBW, kKSplit>;
-  static bool lds_limit_raised = false;  // once per kernel: legal under stream capture afterwards
-  if (!lds_limit_raised) {
-    DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-    lds_limit_raised = true;
-  }
+  static bool lds_limit_raised[kMaxDevices];
+  if (raise_lds_limit<kLds>(kern, lds_limit_raised)) return -1;
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(kThreads * kKSplit), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
@@ -912,11 +916,8 @@ int launch_dma_tile(Params p, hipStream_t stream) {
   p.tiles_m = (p.M + 64 * kMBW - 1) / (64 * kMBW);
   p.tiles_n = (p.N + BN - 1) / BN;
   auto kern = gemm_kernel_dma<P, kMBW, kNBW>;
-  static bool lds_limit_raised = false;
-  if (!lds_limit_raised) {
-    DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-    lds_limit_raised = true;
-  }
+  static bool lds_limit_raised[kMaxDevices];
+  if (raise_lds_limit<kLds>(kern, lds_limit_raised)) return -1;
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(64 * kWaves), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;

@@ -253,11 +253,8 @@ int launch_mx4(Params p, hipStream_t stream) {
   p.tiles_m = (p.M + 255) / 256;
   p.tiles_n = (p.N + 255) / 256;
   auto kern = mx4_gemm_kernel<P>;
-  static bool lds_limit_raised = false;  // once per kernel: legal under stream capture afterwards
-  if (!lds_limit_raised) {
-    DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-    lds_limit_raised = true;
-  }
+  static bool lds_limit_raised[kMaxDevices];
+  if (raise_lds_limit<kLds>(kern, lds_limit_raised)) return -1;
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), kLds, stream, p);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;

@@ -262,12 +262,8 @@ int launch_skinny(const void* A, const void* B, const void* S, const void* Z, vo
 #define DQ_LAUNCH2(MODE_, APERM_, G128_)                                                                             \
   do {                                                                                                               \
     auto kern = w4a16_skinny_kernel<MB, RB, WAVES, U, MODE_, APERM_, G128_>;                                         \
-    static bool lds_limit_raised = false; /* once per kernel: legal under stream capture afterwards */            \
-    if (!lds_limit_raised) {                                                                                         \
-      DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                          \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));                      \
-      lds_limit_raised = true;                                                                                       \
-    }                                                                                                                \
+    static bool lds_limit_raised[kMaxDevices];                                                                       \
+    if (raise_lds_limit<96 * 1024>(kern, lds_limit_raised)) return -1;                                               \
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,  \
                        (const half_t*)Z, (half_t*)C, M, N, K, group, KT);                                            \
   } while (0)

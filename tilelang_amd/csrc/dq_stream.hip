@@ -350,12 +350,8 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 #define DQ_LAUNCH2(MODE_, APERM_)                                                                                    \
   do {                                                                                                               \
     auto kern = w4a16_stream_kernel<MB, RBW, NST, KSPLIT, MODE_, APERM_>;                                                         \
-    static bool lds_limit_raised = false; /* once per kernel: legal under stream capture afterwards */            \
-    if (!lds_limit_raised) {                                                                                         \
-      DQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                          \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds));                           \
-      lds_limit_raised = true;                                                                                       \
-    }                                                                                                                \
+    static bool lds_limit_raised[kMaxDevices];                                                                       \
+    if (raise_lds_limit<kLds>(kern, lds_limit_raised)) return -1;                                                    \
     hipLaunchKernelGGL(kern, grid, block, kLds, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,       \
                        (const half_t*)Z, (half_t*)C, M, N, K);                                                       \
   } while (0)
