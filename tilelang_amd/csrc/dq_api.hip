@@ -26,6 +26,8 @@ int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, voi
                  int mode, int layout, int fast, hipStream_t stream);
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, hipStream_t stream);
+int w4a16_kslice(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
+                 int mode, int layout, hipStream_t stream);
 int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int variant, hipStream_t stream);
 int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
@@ -147,6 +149,12 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     const int rc = w4a16_regres(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant == 40 ? 0 : (variant >= 42 ? variant - 40 : 1), (hipStream_t)stream);
     if (rc <= 0) return rc;
     if (variant >= 40) DQ_FAIL("%s: the register-resident kernel does not cover M=%d N=%d K=%d group=%d", fn, M, N, K, group);
+  }
+  if (variant == 60) {
+    // 17 to 64 rows on a matrix with enough row blocks for every CU: K sliced over the waves of one workgroup per CU
+    const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
+    if (rc > 0) DQ_FAIL("%s: the K-sliced batch kernel does not cover M=%d N=%d K=%d group=%d mode=%d", fn, M, N, K, group, mode);
+    return rc;
   }
   if (variant >= 30 && variant < 40) {
     const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant - 30, (hipStream_t)stream);
