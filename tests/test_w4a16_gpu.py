@@ -140,8 +140,11 @@ def test_gemv_quantized_zeros(cuda, M, qfmt):
     np.testing.assert_allclose(C2.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
 
 
-def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False, scale_range=(0.005, 0.02)):
+def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False, scale_range=(0.005, 0.02),
+              zeros_offset=0.0):
     d = workloads.w4a16(M, N, K, group, seed=seed, scale_range=scale_range, zeros_range=(6, 10))
+    if zeros_offset:  # zero points that are not integers
+        d["Zeros"] = (d["Zeros"].astype(np.float32) + np.float32(zeros_offset)).astype(np.float16)
     kw = _mode_kwargs(mode)
     fast = kw.pop("fast_decoding", False)
     kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, fast_decoding=interleaved,
@@ -231,6 +234,38 @@ def test_register_resident_kernel(cuda, M, mode, variant):
     _run_gemv(cuda, M, 16 * 37, 4096, 128, mode, variant=variant)
     _run_gemv(cuda, M, 48, 8192, 128, mode, variant=variant, interleaved=(mode in ("scale", "original")))
     _run_gemv(cuda, M, 16 * 600, 2048, 128, mode, variant=variant)  # more row blocks than workgroups
+
+
+@pytest.mark.parametrize("mode", ["scale", "uscale", "original", "rescale"])
+@pytest.mark.parametrize("variant", [60, 61])
+def test_k_sliced_batch_kernel(cuda, variant, mode):
+    """17 to 64 rows with K sliced over the eight waves of one workgroup per CU (needs 1400 row blocks or more):
+    two, three and four blocks of activation rows, the smallest K (two slabs per K quarter) and a larger one, a last
+    workgroup with three of its seven row blocks, both layouts, and zero points that are not integers (those take
+    the copy of the loop that subtracts bias and zero point separately)."""
+    _run_gemv(cuda, 17, 16 * 1400, 2048, 128, mode, variant=variant)
+    _run_gemv(cuda, 64, 16 * 1403, 2048, 128, mode, variant=variant, interleaved=(mode in ("scale", "original")))
+    _run_gemv(cuda, 40, 16 * 1400, 3072, 128, mode, variant=variant, seed=3, zeros_offset=0.37)
+    if variant == 60 and mode == "original":
+        _run_gemv(cuda, 33, 16 * 1401, 4096, 128, mode, variant=variant, seed=4)
+
+
+@pytest.mark.parametrize("variant", [60, 61])
+@pytest.mark.parametrize("M", [48, 64])
+def test_k_sliced_batch_kernel_full_size(cuda, cfg3_full_size, M, variant):
+    """The K-sliced kernel at N = 28672, K = 8192 with (q - z) * s: every output against the oracle."""
+    d, W = cfg3_full_size
+    N, K, group = 28672, 8192, 128
+    print(f"cfg3 full size, K-sliced kernel: M={M} variant={variant}", flush=True)
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, source_format="uint",
+                              with_scaling=True, with_zeros=True, zeros_mode="original", variant=variant)
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(_dev(d["A"][:M], cuda), _dev(d["B"], cuda).view(torch.int8), _dev(d["Scale"], cuda), _dev(d["Zeros"], cuda), C)
+    torch.cuda.synchronize()
+    got = C.float().cpu().numpy()
+    ref = (d["A"][:M].astype(np.float32) @ W.T).astype(np.float16).astype(np.float32)
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
 
 
 def test_multi_tile_k(cuda):

@@ -27,7 +27,7 @@ int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, voi
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, hipStream_t stream);
 int w4a16_kslice(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
-                 int mode, int layout, hipStream_t stream);
+                 int mode, int layout, int deep, hipStream_t stream);
 int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int variant, hipStream_t stream);
 int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
@@ -137,7 +137,8 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   // below (two passes over the weights) is still the faster one.  50: the GEMM whatever M.
   if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread (r = 0: its own
-  // choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with
+  // choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  60, 61: the K-sliced batch kernel
+  // (M <= 64, N >= 22400) with two / more pairs of activation loads in flight.  40: the kernel with
   // register-resident activations (M <= 16).  0, 4, 5, 10: a configuration of the tiled MFMA fallback kernel
   // (covers every shape).
   if ((variant >= 40 && variant <= 43) || (variant < 0 && M >= 2 && M <= 16)) {
@@ -150,9 +151,14 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     if (rc <= 0) return rc;
     if (variant >= 40) DQ_FAIL("%s: the register-resident kernel does not cover M=%d N=%d K=%d group=%d", fn, M, N, K, group);
   }
-  if (variant == 60) {
+  if (variant < 0 && M > 16 && M <= 48) {
+    // measured at N = 28672, K = 8192: 11-18 % faster than the streaming kernel at M = 32 and 48, equal at M = 64
+    const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, 1, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
+  if (variant == 60 || variant == 61) {
     // 17 to 64 rows on a matrix with enough row blocks for every CU: K sliced over the waves of one workgroup per CU
-    const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
+    const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant - 60, (hipStream_t)stream);
     if (rc > 0) DQ_FAIL("%s: the K-sliced batch kernel does not cover M=%d N=%d K=%d group=%d mode=%d", fn, M, N, K, group, mode);
     return rc;
   }
