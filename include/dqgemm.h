@@ -104,6 +104,13 @@ int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale
 
 /* ---- further dequantize GEMMs (same 256x256 MFMA kernel, different decoders) ------------------ */
 
+/* bf16 x fp4 without block scales: C[M,N] bf16 = A[M,K] bf16 . bf16(fp4(B[N,K/2]))^T, fp32 accumulation.
+ * Replaces `kernel(A, qB)` of examples/dequantize_gemm/example_dequant_gemm_bf16_fp4_hopper.py:46-346
+ * (ref_program_twiddling / ref_program_simple, :348-386).  fp4_format as above: DQ_FP4_TWIDDLING is the example's
+ * fast_dequant=True layout, DQ_FP4_SIMPLE its fast_dequant=False conversion (exponent E + 126).  Requires K % 64 == 0. */
+int call_dequant_gemm_bf16_fp4(const void* A, const void* B, void* C, int M, int N, int K, int fp4_format,
+                               dq_stream_t stream);
+
 /* fp16 x "simple" fp4: C[M,N] (transposed = 0) or Ct[N,M] (transposed = 1) fp16 =
  * A[M,K] fp16 . fp16bits((s<<15)|((E+14)<<10)|(m<<9))(B[N,K/2])^T, fp32 accumulation.  Replaces
  * `call(A, B, Ct, stream)` of examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:179-215.

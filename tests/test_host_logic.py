@@ -210,6 +210,13 @@ def test_kernels_refuse_cpu_tensors_and_bad_factory_arguments():
         tl.dequantize_gemv(1, 64, 256, group_size=48, with_scaling=True)
     with pytest.raises(ValueError, match="multiple of 64"):
         tl.matmul_bf16_mxfp4(64, 64, 96)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        tl.matmul_bf16_fp4(64, 64, 96)
+    with pytest.raises(ValueError, match="must be bfloat16"):
+        tl.matmul_bf16_fp4(64, 64, 64, in_dtype="float16")
+    kern = tl.matmul_bf16_fp4(64, 32, 128)  # kernel(A, qB) -> C
+    assert [p.name for p in kern.params] == ["A", "B", "C"] and kern.result_idx == [2]
+    assert kern.params[1].shape == (32, 64)
     with pytest.raises(AssertionError):
         tl.dequantize_gemv(1, 64, 256, trans_A=True)
 

@@ -124,3 +124,41 @@ def test_full_size_properties(cuda):
     C2 = kern((A.float() * 2).to(torch.bfloat16), B, S, bias)
     torch.cuda.synchronize()
     assert torch.equal(C2.float(), C.float() * 2)
+
+
+# ---- bf16 x fp4 without block scales (the example with kernel(A, qB)) ------------------------------------------------
+
+@pytest.mark.parametrize("fast_dequant", [True, False])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (100, 300, 192), (512, 1024, 2048)])
+def test_unscaled_bf16_fp4(cuda, fast_dequant, M, N, K):
+    """examples/dequantize_gemm/example_dequant_gemm_bf16_fp4_hopper.py: main(256, 256, 256, fast_dequant) against
+    ref_program_twiddling / ref_program_simple, here the oracle's restatement of them (block exponent 0)."""
+    fmt = "twiddling" if fast_dequant else "simple"
+    d = workloads.mxfp4(M, N, K, seed=11, scale_exp_range=(0, 0), scale_bias=0)
+    B = orc.twiddle_pack_fp4(orc.unpack_u4(d["B"])) if fast_dequant else d["B"]
+    kern = tl.matmul_bf16_fp4(M, N, K, "bfloat16", "bfloat16", "float32", num_bits=4, fast_dequant=fast_dequant,
+                              block_M=256, block_N=128, block_K=128, num_stages=2, threads=256, split=1)
+    C = kern(_dev(d["A"], cuda).view(torch.bfloat16), _dev(B, cuda))
+    torch.cuda.synchronize()
+    zero_scale = np.zeros((N, K // 32), np.uint8)
+    ref = orc.bf16_bits_to_f32(orc.ref_mxfp4(d["A"], B, zero_scale, None, fmt=fmt, scale_bias=0))
+    got = C.float().cpu().numpy()
+    assert got.shape == (M, N) and np.isfinite(got).all()
+    np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
+
+
+def test_unscaled_bf16_fp4_reads_back_the_reference_vectors(cuda):
+    """A = identity makes the GEMM return the dequantised operand itself, exactly: against what the reference's own
+    torch_convert_bit_twiddling (all 65 536 byte pairs) and torch_convert (all 256 bytes) produce
+    (tests/golden/reference_vectors.npz, written by tests/golden/make_vectors.py)."""
+    import os
+
+    v = np.load(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.npz"))
+    for fast, qB, want_bits in ((True, v["twiddling_in"], v["twiddling_out_bits"]), (False, v["convert_in"], v["convert_out_bits"])):
+        N, K = qB.shape[0], qB.shape[1] * 2
+        kern = tl.matmul_bf16_fp4(K, N, K, fast_dequant=fast)
+        eye = torch.eye(K, dtype=torch.bfloat16, device=cuda)
+        C = kern(eye, _dev(qB, cuda))
+        torch.cuda.synchronize()
+        got = C.float().cpu().numpy().T  # [N, K]
+        np.testing.assert_array_equal(got, orc.bf16_bits_to_f32(want_bits))

@@ -14,6 +14,7 @@ from .kernels import (  # noqa: F401
     bitnet_158_int8xint2_prefill,
     dequantize_gemv,
     dequantize_w4,
+    matmul_bf16_fp4,
     matmul_bf16_mxfp4,
     matmul_mxfp4_mxfp4,
     matmul_fp16_fp4,

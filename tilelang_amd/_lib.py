@@ -31,6 +31,7 @@ SIGNATURES = {
     "call_unpack_qzeros": [_vp, _vp, _i, _i, _i, _vp],
     "call_dequantize_w4": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_bf16_mxfp4": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "call_dequant_gemm_bf16_fp4": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4_splitk": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_dequant_gemm_fp16_fp4_splitk_static": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],

@@ -38,6 +38,7 @@ int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, 
 int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
                int scale_bias, hipStream_t stream);
 
+int bf16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int fmt, hipStream_t stream);
 int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream);
 int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                 int mode, int layout, hipStream_t stream);
@@ -258,6 +259,19 @@ static int check_gemm_args(const char* fn, const void* A, const void* B, const v
   if (K % kmult != 0) DQ_FAIL("%s: K=%d must be a multiple of %d", fn, K, kmult);
   if (!aligned16(A) || !aligned16(B) || !aligned16(C)) DQ_FAIL("%s: A, B and C must be 16-byte aligned", fn);
   return 0;
+}
+
+extern "C" int call_dequant_gemm_bf16_fp4(const void* A, const void* B, void* C, int M, int N, int K, int fp4_format,
+                                         dq_stream_t stream) {
+  const char* fn = "call_dequant_gemm_bf16_fp4";
+  if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
+  if (!B) DQ_FAIL("%s: B is expected to have non-NULL data pointer", fn);
+  if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
+  if (M <= 0 || N <= 0 || K <= 0) DQ_FAIL("%s: M, N, K must be positive (got %d %d %d)", fn, M, N, K);
+  if (K % 64 != 0) DQ_FAIL("%s: K=%d must be a multiple of 64", fn, K);
+  if (fp4_format < FP4_E2M1 || fp4_format > FP4_TWIDDLING) DQ_FAIL("%s: unknown fp4 format %d", fn, fp4_format);
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C)) DQ_FAIL("%s: A, B and C must be 16-byte aligned", fn);
+  return bf16_fp4_gemm(A, B, C, M, N, K, fp4_format, (hipStream_t)stream);
 }
 
 extern "C" int call_dequant_gemm_fp16_fp4(const void* A, const void* B, void* C, int M, int N, int K, int transposed,

@@ -117,6 +117,26 @@ struct MxPolicy : Bf16Mfma, gemm::PlainA {
   }
 };
 
+// ---- fp4 x bf16 without block scales (examples/dequantize_gemm/example_dequant_gemm_bf16_fp4_hopper.py) ------------
+// The same three nibble formats as above with the exponent offset at zero: the twiddled layout of the example's
+// fast_dequant=True (:113-118) and the "simple" conversion of fast_dequant=False (:222-262: exponent E + 126).
+template <int FMT>
+struct Bf16Fp4Policy : Bf16Mfma, gemm::PlainA, gemm::NoScale {
+  static constexpr int kBRowBytes = 32;
+  static constexpr bool kTransposed = false;
+  using out_t = bf16_t;
+  __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
+  using gemm::NoScale::prep_scale;
+  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
+    if constexpr (FMT == FP4_E2M1) return cvt_e2m1x8(w[j], 1.f);
+    else if constexpr (FMT == FP4_TWIDDLING) return cvt_e2m1x8(twiddled_to_plain(w[j]), 1.f);
+    else return __builtin_bit_cast(frag_t, simple_fp4x8<7>(w[j], 0x3F003F00u));  // (E + 126) << 7
+  }
+  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params&, int, int) {
+    return (bf16_t)__builtin_bit_cast(float, raw);
+  }
+};
+
 // ---- "simple" fp4 x fp16 (examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py) ------------
 template <bool TRANSPOSED>
 struct Fp16Fp4Policy : F16Mfma, gemm::PlainA, gemm::NoScale {
@@ -199,6 +219,22 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
     default: DQ_FAIL("mxfp4 gemm: unknown weight format %d", fmt);
   }
 #undef DQ_MX
+}
+
+int bf16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int fmt, hipStream_t stream) {
+  Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
+#define DQ_F4(FMT_)                                                                                          \
+  do {                                                                                                       \
+    if (gemm::dma_eligible<Bf16Fp4Policy<FMT_>>(p)) return gemm::launch_dma<Bf16Fp4Policy<FMT_>>(p, stream); \
+    return gemm::launch_auto<Bf16Fp4Policy<FMT_>>(p, stream);                                                \
+  } while (0)
+  switch (fmt) {
+    case FP4_E2M1: DQ_F4(FP4_E2M1);
+    case FP4_SIMPLE: DQ_F4(FP4_SIMPLE);
+    case FP4_TWIDDLING: DQ_F4(FP4_TWIDDLING);
+    default: DQ_FAIL("bf16 x fp4 gemm: unknown weight format %d", fmt);
+  }
+#undef DQ_F4
 }
 
 int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream) {

@@ -379,6 +379,54 @@ def matmul_bf16_mxfp4(
     return KernelAdapter("matmul_bf16_mxfp4", params, [-1], launch, _lib.last_error)
 
 
+def matmul_bf16_fp4(
+    M: int,
+    N: int,
+    K: int,
+    in_dtype="bfloat16",
+    out_dtype="bfloat16",
+    accum_dtype="float32",
+    source_format="uint32",
+    num_bits: int = 4,
+    fast_dequant: bool = True,
+    block_M: int = 256,
+    block_N: int = 128,
+    block_K: int = 128,
+    num_stages: int = 2,
+    threads: int = 256,
+    split: int = 1,
+    weight_format: str | None = None,
+) -> KernelAdapter:
+    """FP4-weight GEMM without block scales: ``C[M,N] = A[M,K] @ bf16(fp4(B[N,K/2])).T``.
+
+    Same arguments as ``matmul`` of
+    examples/dequantize_gemm/example_dequant_gemm_bf16_fp4_hopper.py:46-62 (tile sizes, stages, threads and split are
+    accepted and ignored) and the same call, ``C = kernel(A, qB)`` with the example's ``out_idx=[-1]``.
+    ``fast_dequant=True`` reads the bit-twiddled layout that ``ref_program_twiddling`` (:348-366) decodes,
+    ``fast_dequant=False`` the plain nibbles of ``ref_program_simple`` (:369-386); ``weight_format`` ("twiddling",
+    "simple", "e2m1") overrides the choice as in ``matmul_bf16_mxfp4``.
+    """
+    if num_bits != 4:
+        raise ValueError("matmul_bf16_fp4: num_bits must be 4")
+    if _dtype(in_dtype) != torch.bfloat16 or _dtype(out_dtype) != torch.bfloat16:
+        raise ValueError("matmul_bf16_fp4: in_dtype and out_dtype must be bfloat16")
+    if K % 64 != 0:
+        raise ValueError(f"matmul_bf16_fp4: K={K} must be a multiple of 64")
+    if weight_format is None:
+        weight_format = "twiddling" if fast_dequant else "simple"
+    fmt = _FP4_FORMATS[weight_format]
+    params = [
+        KernelParam("A", torch.bfloat16, (M, K)),
+        KernelParam("B", torch.uint8, (N, K // 2), packed=True),
+        KernelParam("C", torch.bfloat16, (M, N)),
+    ]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_dequant_gemm_bf16_fp4(ptrs[0], ptrs[1], ptrs[2], M, N, K, fmt, stream)
+
+    return KernelAdapter("matmul_bf16_fp4", params, [-1], launch, _lib.last_error)
+
+
 def matmul_mxfp4_mxfp4(M: int, N: int, K: int, out_dtype="bfloat16", accum_dtype="float32", with_bias: bool = False) -> KernelAdapter:
     """Block-scaled MXFP4 x MXFP4 GEMM on the gfx950 scaled matrix instruction:
     ``C[M,N] = (e2m1(A[M,K/2]) * 2**(SFA[M,K/32] - 127)) @ (e2m1(B[N,K/2]) * 2**(SFB[N,K/32] - 127)).T (+ Bias)``.
