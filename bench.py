@@ -27,11 +27,26 @@ HBM_PEAK = 8.0e12        # B/s
 MFMA_BF16_PEAK = 2.5e15  # FLOP/s dense
 MFMA_I8_PEAK = 5.0e15    # OP/s dense
 MFMA_FP4_PEAK = 10.1e15  # FLOP/s dense, block-scaled fp4
-# HBM bytes per launch of the headline GEMV: not measured by this script (counters need the profiler) but quoted
-# from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary, scaled there by what the same counters read
-# for a plain 128 MiB copy kernel.  Re-measure and update all three fields whenever the kernel changes.
-GEMV_HBM_TRAFFIC = {"bytes": 121381888, "kernel": "w4a16_gemv_kernel<1,1,4,scale,g128,wide>",
-                    "source": "profiles/bench_all_configs_hbm_traffic.md"}
+# HBM bytes per launch of the headline GEMV: counters need the profiler, so this script cannot measure them; it READS
+# them from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary (scaled there by what the same counters read
+# for a plain 128 MiB copy kernel: 2 KiB and 1 KiB per count).  The row is looked up by workload and must name the
+# kernel this script launches, otherwise `traffic` is null: a figure of another kernel is never printed as this one's.
+GEMV_TRAFFIC_PROFILE = "profiles/bench_all_configs_hbm_traffic.md"
+GEMV_KERNEL = "w4a16_gemv_kernel<1,1,4,1,0,1,0,1>"  # MROWS, NP, R, HAS_SCALE, HAS_ZEROS, G128, FLIP, WIDE
+
+
+def gemv_hbm_traffic():
+    """(bytes per launch or None, source) of the headline GEMV from the committed counter summary."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), GEMV_TRAFFIC_PROFILE)
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.split("|")]
+                if len(cells) >= 6 and "(headline)" in cells[2] and GEMV_KERNEL in cells[1]:
+                    return int(round(float(cells[3]) * 2048 + float(cells[4]) * 1024)), GEMV_TRAFFIC_PROFILE
+    except (OSError, ValueError):
+        pass
+    return None, None
 
 
 def _time_launches(torch, fns, steps, warmup, min_launches=120, max_launches=None, settle_ms=50.0, replays=30):
@@ -394,9 +409,10 @@ def main():
     head = bench_w4a16(torch, tl, workloads, M, N, K, False, S, W, dev)
     us = head["us"]
     gbs = head["bytes"] / (us * 1e-6) / 1e9
+    traffic, traffic_source = gemv_hbm_traffic()
     roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": gbs * 1e9 / HBM_PEAK,
-            "traffic": GEMV_HBM_TRAFFIC["bytes"], "traffic_source": GEMV_HBM_TRAFFIC["source"],
-            "kernel": GEMV_HBM_TRAFFIC["kernel"], "algorithmic_bytes": head["bytes"],
+            "traffic": traffic, "traffic_source": traffic_source,
+            "kernel": GEMV_KERNEL, "algorithmic_bytes": head["bytes"],
             "us_min": head["timing"]["us_min"], "us_mean": head["timing"]["us_mean"]}
 
     if args.copy_calibration:
