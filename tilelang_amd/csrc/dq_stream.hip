@@ -35,6 +35,9 @@ namespace dq {
 
 namespace {
 
+// M0 is set inside each statement right before the one instruction that reads it and is not on the clobber list
+// (clang treats M0 as reserved there and promises nothing for it); nothing else in this kernel depends on M0 across
+// the statements: no other LDS-direct load, no GWS / sendmsg, no indirect register indexing.
 __device__ __forceinline__ void dma16(unsigned lds_addr, unsigned voff, const void* sbase) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
