@@ -114,7 +114,7 @@ def _copies(nbytes, min_total=640 << 20, lo=2, hi=24):
     return int(min(hi, max(lo, -(-min_total // max(nbytes, 1)))))
 
 
-def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False, **tk):
+def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False, fragments=False, **tk):
     group = 128
     d = workloads.w4a16(M, N, K, group, seed=0, scale_range=(0.002, 0.01) if zeros else (0.005, 0.02),
                         zeros_range=(6, 10) if zeros else None)
@@ -127,12 +127,18 @@ def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interl
         from tilelang_amd import quantize
 
         b0 = quantize.interleave_weight(b0, 4, "float16")
+    if fragments:
+        # offline re-ordering into the matrix instruction's operand order (the role of the reference's ladder weight
+        # transform, example_dequant_gemm_fine_grained.py:136-354)
+        from tilelang_amd import quantize
+
+        b0 = quantize.prepack_w4_fragments(b0)
     Bs = [b0.to(dev).clone() for _ in range(nc)]
     Ss = [torch.from_numpy(d["Scale"]).to(dev).clone() for _ in range(nc)]
     Zs = [torch.from_numpy(d["Zeros"]).to(dev).clone() for _ in range(nc)] if zeros else None
     C = torch.empty((M, N), dtype=torch.float16, device=dev)
     kern = tl.dequantize_gemv(M, N, K, group_size=group, source_format="uint" if zeros else "int",
-                              with_scaling=True, with_zeros=zeros, fast_decoding=interleaved)
+                              with_scaling=True, with_zeros=zeros, fast_decoding=interleaved, weight_fragments=fragments)
     if zeros:
         fns = [(lambda i=i: kern(A, Bs[i], Ss[i], Zs[i], C, skip_tensor_validation=True)) for i in range(nc)]
     else:
@@ -434,6 +440,10 @@ def main():
             row = _row(f"w4a16_zeros M={m} N=28672 K=8192", r, "hbm", MFMA_BF16_PEAK)
             row["frac_mfma"] = r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK
             shapes.append(row)
+        for m in (4, 16):
+            r = bench_w4a16(torch, tl, workloads, m, 28672, 8192, True, S, W, dev, fragments=True)
+            shapes.append(_row(f"w4a16_zeros M={m} N=28672 K=8192 (weights re-ordered offline into the matrix instruction's operand order)",
+                               r, "hbm", MFMA_BF16_PEAK))
         r = bench_w2a16(torch, tl, 1, 28672, 8192, S, W, dev)
         shapes.append(_row("w2a16_gemv M=1 N=28672 K=8192 (num_bits=2, interleaved words, (c-2)*s)", r, "hbm", MFMA_BF16_PEAK))
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)

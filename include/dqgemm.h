@@ -47,9 +47,16 @@ enum dq_w4_mode {
 
 enum dq_w4_layout {
   DQ_LAYOUT_PLAIN = 0,      /* nibble e of each 32-bit word is element e                         */
-  DQ_LAYOUT_INTERLEAVED = 1 /* words pre-permuted by interleave_weight (.., 4, "float16") for uint4,
+  DQ_LAYOUT_INTERLEAVED = 1, /* words pre-permuted by interleave_weight (.., 4, "float16") for uint4,
                                (.., 2, "int8") for 2-bit codes,
                                examples/dequantize_gemm/quantize/utils.py:71-125              */
+  DQ_LAYOUT_FRAGMENTS = 2    /* flag, added to one of the two above (call_dequantize_gemv_w4a16 only, M <= 16): the
+                               16-byte pieces of B re-ordered offline into the matrix instruction's operand order,
+                               B[N/16][K/128][64][16 bytes], entry 16 g + r of a 128-k chunk = bytes 16 g .. 16 g + 15
+                               of that chunk of row r of the block.  The role of the weight transform of
+                               examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:136-354
+                               (B[N/16][K/16][16][8], micro-tiles of the NVIDIA instruction), for this chip's 16x16x32
+                               instruction; its BitBLAS permutation inside a tile is third-party and not reproduced. */
 };
 
 /* ---- W4A16 ---------------------------------------------------------------------------- */

@@ -26,7 +26,10 @@ How each function is pinned (see tests/test_oracle_pins.py):
 * the rounding order of the scaled / zero-point uint4 decoders and of the BitLinear epilogue against the operation
   order of the device snippets written out with exact rationals and an explicit round-to-nearest-even per fp16 /
   fp32 instruction;
-* matmuls by reduction to int64 / float64 brute force on tiny shapes.
+* matmuls by reduction to int64 / float64 brute force on tiny shapes;
+* ``prepack_w4_fragments`` is this library's own layout (the reference's ladder transform is BitBLAS's and absent): the
+  index formula written as plain loops; what pins it is the kernel that reads the layout giving, bit for bit, what the
+  row-major kernel gives (tests/test_w4a16_gpu.py::test_fragment_ordered_weights).
 
 Parity unpinned by any reference test or fixture (no in-tree caller exists; the
 contract is the closed form plus the operation order of the device snippets):
@@ -830,3 +833,21 @@ def ref_bitnet(A_i8, packed, s_a, s_w, convention: str = "offset"):
     """BitNet W2A8 linear: exact int32 accumulation then the BitLinear epilogue -> fp16 [M, N]."""
     acc = ref_bitnet_int(A_i8, packed, convention)
     return post_quant_process(acc, np.asarray(s_a, dtype=np.float32).reshape(-1, 1), s_w)
+
+
+def prepack_w4_fragments(B):
+    """Packed uint4 weights [N, K/2] -> [N/16, K/128, 64, 16] bytes: entry 16 g + r of chunk c of block b holds bytes
+    64 c + 16 g .. + 15 of row 16 b + r -- the operand order of the 16x16x32 matrix instruction (lane 16 g + r owns
+    k = 32 g .. 32 g + 31 of a 128-k chunk of row r).  Plain loops over the index formula (test infrastructure: the
+    library's torch helper and its kernel are checked against this).  In the role of the reference's offline weight
+    transform, examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:178-179 (B_shape of the ladder kernel)."""
+    B = np.ascontiguousarray(B).view(np.uint8)
+    N, KB = B.shape
+    assert N % 16 == 0 and KB % 64 == 0
+    out = np.empty((N // 16, KB // 64, 64, 16), np.uint8)
+    for b in range(N // 16):
+        for c in range(KB // 64):
+            for g in range(4):
+                for r in range(16):
+                    out[b, c, 16 * g + r, :] = B[16 * b + r, 64 * c + 16 * g: 64 * c + 16 * g + 16]
+    return out

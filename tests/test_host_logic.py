@@ -306,3 +306,23 @@ def test_lowbit_gemv_factory_rejections():
     assert [p.shape for p in k.params if p.name == "Zeros"] == [(64, 4)]
     with pytest.raises(ValueError):
         tl.dequantize_gemv(1, 64, 1024, "int8", "int32", "int32", num_bits=2, with_scaling=True, group_size=128)
+
+
+def test_fragment_prepack_matches_the_oracle_and_inverts():
+    """quantize.prepack_w4_fragments against the oracle's index formula, its inverse, and the factory's shape rules."""
+    rng = np.random.default_rng(3)
+    B = rng.integers(0, 256, size=(80, 192), dtype=np.uint8)  # N = 80, K = 384
+    frag = quantize.prepack_w4_fragments(torch.from_numpy(B))
+    assert frag.shape == (5, 3, 64, 16)
+    np.testing.assert_array_equal(frag.numpy(), orc.prepack_w4_fragments(B))
+    np.testing.assert_array_equal(quantize.unpack_w4_fragments(frag).numpy(), B)
+    with pytest.raises(ValueError, match="N % 16 == 0"):
+        quantize.prepack_w4_fragments(torch.zeros(24, 64, dtype=torch.uint8))
+    kern = tl.dequantize_gemv(4, 64, 2048, group_size=128, source_format="int", with_scaling=True, weight_fragments=True)
+    assert kern.params[1].shape == (4, 16, 64, 16)
+    for bad in (dict(M=17), dict(K=1024), dict(group_size=64)):
+        args = dict(M=4, N=64, K=2048, group_size=128)
+        args.update(bad)
+        with pytest.raises(ValueError, match="fragment-ordered weights"):
+            tl.dequantize_gemv(args["M"], args["N"], args["K"], group_size=args["group_size"], source_format="int",
+                               with_scaling=True, weight_fragments=True)

@@ -141,17 +141,19 @@ def test_gemv_quantized_zeros(cuda, M, qfmt):
 
 
 def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False, scale_range=(0.005, 0.02),
-              zeros_offset=0.0):
+              zeros_offset=0.0, fragments=False):
     d = workloads.w4a16(M, N, K, group, seed=seed, scale_range=scale_range, zeros_range=(6, 10))
     if zeros_offset:  # zero points that are not integers
         d["Zeros"] = (d["Zeros"].astype(np.float32) + np.float32(zeros_offset)).astype(np.float16)
     kw = _mode_kwargs(mode)
     fast = kw.pop("fast_decoding", False)
     kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, fast_decoding=interleaved,
-                              _formula_fast=fast, variant=variant, **kw)
+                              _formula_fast=fast, variant=variant, weight_fragments=fragments, **kw)
     Bdev = _dev(d["B"], cuda).view(torch.int8)
     if interleaved:
         Bdev = tl.quantize.interleave_weight(Bdev, 4, "float16")
+    if fragments:
+        Bdev = tl.quantize.prepack_w4_fragments(Bdev)
     args = [_dev(d["A"], cuda), Bdev]
     if kw.get("with_scaling"):
         args.append(_dev(d["Scale"], cuda))
@@ -266,6 +268,42 @@ def test_k_sliced_batch_kernel_full_size(cuda, cfg3_full_size, M, variant):
     ref = (d["A"][:M].astype(np.float32) @ W.T).astype(np.float16).astype(np.float32)
     assert np.isfinite(got).all()
     np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original"])
+@pytest.mark.parametrize("M", [1, 4, 9, 16])
+def test_fragment_ordered_weights(cuda, M, mode):
+    """Weights re-ordered offline into the matrix instruction's operand order (quantize.prepack_w4_fragments): against
+    the oracle, and bit for bit against the same kernel reading the row-major weights in that layout (variant 43),
+    which differs in addresses only.  Every K the kernel covers, both word layouts, more row blocks than workgroups."""
+    for (N, K, il) in ((16 * 37, 4096, False), (48, 8192, mode in ("scale", "original")), (16 * 600, 2048, False)):
+        got = _run_gemv(cuda, M, N, K, 128, mode, interleaved=il, fragments=True)
+        same = _run_gemv(cuda, M, N, K, 128, mode, interleaved=il, variant=43)
+        np.testing.assert_array_equal(got.view(np.uint16), same.view(np.uint16))
+
+
+def test_fragment_ordered_weights_full_size(cuda, cfg3_full_size):
+    """N = 28672, K = 8192 with zero points, M = 16: every output against the oracle."""
+    d, W = cfg3_full_size
+    M, N, K, group = 16, 28672, 8192, 128
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, source_format="uint",
+                              with_scaling=True, with_zeros=True, zeros_mode="original", weight_fragments=True)
+    Bf = tl.quantize.prepack_w4_fragments(_dev(d["B"], cuda).view(torch.int8))
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(_dev(d["A"][:M], cuda), Bf, _dev(d["Scale"], cuda), _dev(d["Zeros"], cuda), C)
+    torch.cuda.synchronize()
+    ref = (d["A"][:M].astype(np.float32) @ W.T).astype(np.float16).astype(np.float32)
+    np.testing.assert_allclose(C.float().cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_fragment_ordered_weights_are_refused_where_no_kernel_reads_them(cuda):
+    kern = tl.dequantize_gemv(8, 64, 2048, group_size=128, source_format="int", with_scaling=True, weight_fragments=True, variant=36)
+    A = torch.zeros(8, 2048, dtype=torch.float16, device=cuda)
+    B = torch.zeros(4, 16, 64, 16, dtype=torch.int8, device=cuda)
+    S = torch.ones(64, 16, dtype=torch.float16, device=cuda)
+    C = torch.empty(8, 64, dtype=torch.float16, device=cuda)
+    with pytest.raises(RuntimeError, match="fragment-ordered weights"):
+        kern(A, B, S, C)
 
 
 def test_multi_tile_k(cuda):

@@ -131,9 +131,20 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
   if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
   if (M <= 0) DQ_FAIL("%s: M must be positive (got %d)", fn, M);
-  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
+  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout & ~LAYOUT_FRAGMENTS)) return -1;
   if (K % 128 != 0) DQ_FAIL("%s: K=%d must be a multiple of 128", fn, K);
   if (!aligned16(A) || !aligned16(C)) DQ_FAIL("%s: A and C must be 16-byte aligned", fn);
+  if (layout & LAYOUT_FRAGMENTS) {
+    // weights re-ordered offline into the matrix instruction's operand order: read by the register-resident
+    // small-batch kernel only
+    const int rc = (variant < 0 || variant == 44) && M <= 16
+                       ? w4a16_regres(A, B, Scale, Zeros, C, M, N, K, group, mode, layout & 1, 4, (hipStream_t)stream)
+                       : 1;
+    if (rc > 0)
+      DQ_FAIL("%s: fragment-ordered weights are read at M <= 16, N %% 16 == 0, K = 2048 / 4096 / 8192, group 128 and every mode "
+              "but \"rescale\" only (got M=%d N=%d K=%d group=%d mode=%d)", fn, M, N, K, group, mode);
+    return rc;
+  }
   // prefill-sized M: the tiled MFMA GEMM (same tile-exact decoders); up to 128 rows the streaming kernel
   // below (two passes over the weights) is still the faster one.  50: the GEMM whatever M.
   if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);

@@ -81,6 +81,8 @@ enum W4Mode : int {
 enum W4Layout : int {
   LAYOUT_PLAIN = 0,        // nibble e of a 32-bit word is element e
   LAYOUT_INTERLEAVED = 1,  // word already permuted for the fast 16-bit decoder (elements 0,2,4,6,1,3,5,7)
+  LAYOUT_FRAGMENTS = 2,    // flag, added to one of the above: 16-byte pieces re-ordered offline into the matrix
+                           // instruction's operand order, [N / 16][K / 128][64 lanes][16 bytes] (uint4, decode GEMV only)
 };
 
 enum Fp4Format : int {

@@ -203,7 +203,10 @@ constexpr uint32_t kOutOfRange = 0xFFFFF000u;   // an offset no matrix of this k
 // block is transposed into that layout through a 16 S-byte LDS area of the wave's own: 16-byte writes as loaded,
 // 16-byte reads as multiplied, the pieces of row r XOR-swizzled with r so that neither side has bank conflicts.
 // LDS operations of one wave execute in order, so no barrier and no second area is needed.
-template <int WAVES, int NC, int DEPTH, int PARK, bool TR, bool HAS_SCALE, bool HAS_ZEROS, bool FLIP, bool APERM>
+// FRAG: the weights were re-ordered offline into the matrix instruction's operand order (quantize.prepack_w4_fragments:
+// [N / 16][K / 128][64 lanes][16 bytes], lane 16 g + r holding piece g of row r of the chunk), so an instruction reads
+// 1 KiB contiguous straight into the operand layout and nothing is transposed.
+template <int WAVES, int NC, int DEPTH, int PARK, bool TR, bool FRAG, bool HAS_SCALE, bool HAS_ZEROS, bool FLIP, bool APERM>
 __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                         const half_t* __restrict__ S, const half_t* __restrict__ Z,
                                                                         half_t* __restrict__ C, int M, int N, int K, int rbn,
@@ -218,9 +221,10 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   __shared__ __align__(16) unsigned char sz_lds[2][2][16 * kSzRow + 16];  // + a word that idle threads write to
   constexpr int NR = NC - PARK;  // chunks whose activations stay in registers
   static_assert(!TR || DEPTH == 1, "the transposing form keeps one block in flight");
+  static_assert(!(TR && FRAG), "fragment-ordered weights need no transposition");
   constexpr int LPR = 4 * NC;    // TR: lanes (16-byte pieces) per row of the wave's slice
   constexpr int RPI = 64 / LPR;  // TR: rows per load instruction
-  __shared__ uint4_t wstage[TR ? WAVES : 1][TR ? 256 : 1];  // 16 rows x up to 256 bytes per wave
+  __shared__ uint4_t wstage[(TR || FRAG) ? WAVES : 1][(TR || FRAG) ? 256 : 1];  // 16 rows x up to 256 bytes per wave
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -246,8 +250,10 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   uint32_t s_stage = 0, z_stage = 0;
   Halves<NC> sc, zp;
   // per-lane byte offsets inside a row block (N is a multiple of 16 here); the block's own offset is uniform
+  constexpr uint32_t kChunkStep = FRAG ? 1024u : 64u;  // bytes from one 128-k chunk of a block to the next
   const uint32_t w_voff = TR ? (uint32_t)(lane / LPR) * row_bytes + (uint32_t)chunk0 * 64u + (uint32_t)(lane % LPR) * 16u
-                             : (uint32_t)r * row_bytes + (uint32_t)chunk0 * 64u + (uint32_t)g * 16u;
+                             : (FRAG ? (uint32_t)chunk0 * 1024u + (uint32_t)lane * 16u
+                                     : (uint32_t)r * row_bytes + (uint32_t)chunk0 * 64u + (uint32_t)g * 16u);
   const uint32_t sz_dwords = 8u * groups_per_row;  // dwords of scales of one row block
   const uint32_t s_voff = (uint32_t)tid < sz_dwords ? (uint32_t)tid * 4u : kOutOfRange;
   const int sz_shift = 31 - __builtin_clz(groups_per_row >> 1);  // log2(dwords of scales per row); K / 256 is a power of two here
@@ -259,7 +265,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
       const uint32_t so = rb < nrb_wg ? (uint32_t)((rb0 + rb) * 16 + c * RPI) * row_bytes : kOutOfRange;
       bq[d][c] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, w_voff, so, 2 /* nt */);
     } else {
-      bq[d][c] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, w_voff + (uint32_t)c * 64u, w_soff(rb), 2 /* nt */);
+      bq[d][c] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, w_voff + (uint32_t)c * kChunkStep, w_soff(rb), 2 /* nt */);
     }
   };
   // TR: where load instruction i's 16 bytes go, and where chunk c's operand words of lane (g, r) are
@@ -303,7 +309,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
     for (int c = 0; c < NC; ++c) {
       float4_t sum = {0.f, 0.f, 0.f, 0.f};
       uint4_t dd[4];
-      if constexpr (TR) {
+      if constexpr (TR || FRAG) {
         // the chunk's 16 rows x 256 bytes are fetched row-contiguously too (an instruction reads 4 rows x 256 bytes
         // instead of 16-byte pieces of 32 cache lines) and transposed through the wave's LDS area
 #pragma unroll
@@ -412,7 +418,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   }
 }
 
-template <int WAVES, int NC, int DEPTH, int PARK, bool TR>
+template <int WAVES, int NC, int DEPTH, int PARK, bool TR, bool FRAG = false>
 int launch_regres_fast(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int mode,
                        int layout, hipStream_t stream) {
   const int nrb = (N + 15) / 16;
@@ -420,7 +426,7 @@ int launch_regres_fast(const void* A, const void* B, const void* S, const void* 
   const dim3 grid((nrb + rbn - 1) / rbn), block(64 * WAVES);
   const bool plain = layout == LAYOUT_PLAIN;
 #define DQ_FAST2(HS, HZ, FL, AP, ZC)                                                                                        \
-  hipLaunchKernelGGL((w4a16_regres_fast_kernel<WAVES, NC, DEPTH, PARK, TR, HS, HZ, FL, AP>), grid, block, 0, stream, (const half_t*)A, \
+  hipLaunchKernelGGL((w4a16_regres_fast_kernel<WAVES, NC, DEPTH, PARK, TR, FRAG, HS, HZ, FL, AP>), grid, block, 0, stream, (const half_t*)A, \
                      (const uint8_t*)B, (const half_t*)S, (const half_t*)Z, (half_t*)C, M, N, K, rbn, ZC)
 #define DQ_FAST(HS, HZ, FL, ZC)                  \
   do {                                           \
@@ -477,16 +483,24 @@ int launch_regres(const void* A, const void* B, const void* S, const void* Z, vo
 // Returns 1 when the shape is not covered: needs M <= 16, N a multiple of 16, K = 2048, 4096 or 8192 (whole
 // 128-k chunks per wave, activations within the register budget) and group 128 when the mode reads scales
 // (one scale per chunk).
-// `fast`: the variant that applies scale and zero point per group in fp32 (not for "rescale").
+// `fast`: the variant that applies scale and zero point per group in fp32 (not for "rescale"); 4: the same for weights
+// in fragment order (no other kernel reads that order).
 int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int fast, hipStream_t stream) {
   if (M < 1 || M > 16 || N < 16 || N % 16 != 0) return 1;
   if (mode >= W4_SCALE && group != 128) return 1;
   if ((size_t)N * K / 2 >= (1ull << 32) - 8192) return 1;  // 32-bit offsets, and room for the out-of-range marker
+  if (fast == 4 && mode == W4_ZEROS_RESCALE) return 1;  // the exact kernels read the row-major order only
   if (fast && mode != W4_ZEROS_RESCALE) {
     // fast = 1 (default): sixteen waves, row-contiguous loads transposed through LDS (at K = 2048 a wave's slice of a
     // row is 64 bytes and the matrix instruction's own layout is already row-contiguous); 3: sixteen waves, loads in
     // the matrix instruction's layout; 2: eight waves of 256 registers with two row blocks in flight, same layout
+    if (fast == 4) {  // fragment-ordered weights
+      if (K == 8192) return launch_regres_fast<16, 4, 1, 0, false, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      if (K == 4096) return launch_regres_fast<16, 2, 1, 0, false, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      if (K == 2048) return launch_regres_fast<16, 1, 1, 0, false, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+      return 1;
+    }
     if (fast == 1) {
       if (K == 8192) return launch_regres_fast<16, 4, 1, 0, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);
       if (K == 4096) return launch_regres_fast<16, 2, 1, 0, true>(A, B, S, Z, C, M, N, K, mode, layout, stream);

@@ -17,7 +17,7 @@ from .adapter import KernelAdapter, KernelParam
 
 # ---- enums of include/dqgemm.h -------------------------------------------------------------
 W4_UNSIGNED, W4_SIGNED, W4_OFFSET8, W4_SCALE, W4_USCALE, W4_ZEROS_ORIGINAL, W4_ZEROS_RESCALE = range(7)
-LAYOUT_PLAIN, LAYOUT_INTERLEAVED = 0, 1
+LAYOUT_PLAIN, LAYOUT_INTERLEAVED, LAYOUT_FRAGMENTS = 0, 1, 2
 I4_UNSIGNED, I4_TWOS, I4U_INTERLEAVED, I4S_INTERLEAVED = range(4)
 
 _DTYPES = {
@@ -105,6 +105,7 @@ def dequantize_gemv(
     variant: int = -1,
     _formula_fast: bool | None = None,
     qzeros_format: str = "int16",
+    weight_fragments: bool = False,
 ) -> KernelAdapter:
     """W4A16 decode GEMV / small-batch GEMM: ``C[M,N] = A[M,K] @ dequant(B[N,K/2]).T``.
 
@@ -122,6 +123,10 @@ def dequantize_gemv(
     ``interleave_weight(B, 4, "float16")``; otherwise B is the plain low-nibble-first
     layout.  Accumulation is always fp32.  ``source_format="int"`` with scaling is the
     zero-point-8 decode ``w = (q - 8) * s``.
+
+    ``weight_fragments=True``: B went through ``quantize.prepack_w4_fragments`` (after ``interleave_weight`` when
+    ``fast_decoding``) and is ``[N/16, K/128, 64, 16]`` bytes, the matrix instruction's operand order; read at
+    M <= 16, K in {2048, 4096, 8192}, group 128 only (the library refuses other shapes).
     """
     assert trans_A is False, "Dequantize only implement for trans_A=False currently"
     assert trans_B is True, "Dequantize only implement for trans_B=TRue currently"
@@ -148,10 +153,17 @@ def dequantize_gemv(
     mode = _w4_mode(source_format, formula_fast, with_scaling, with_zeros, zeros_mode)
     layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
     groups = K // group_size
+    b_shape = (N, K // 2)
+    if weight_fragments:
+        if M > 16 or N % 16 != 0 or K not in (2048, 4096, 8192) or group_size != 128 or (with_zeros and zeros_mode == "rescale"):
+            raise ValueError("dequantize_gemv: fragment-ordered weights need M <= 16, N % 16 == 0, K in {2048, 4096, 8192}, "
+                             "group_size 128 and a zeros_mode other than \"rescale\"")
+        layout |= LAYOUT_FRAGMENTS
+        b_shape = (N // 16, K // 128, 64, 16)
 
     params = [
         KernelParam("A", torch.float16, (M, K)),
-        KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True),
+        KernelParam("B", _dtype(storage_dtype), b_shape, packed=True),
     ]
     if with_scaling:
         params.append(KernelParam("Scale", torch.float16, (N, groups)))

@@ -4,7 +4,8 @@ Same names and argument meaning as the helpers the reference's examples import:
 ``general_compress`` / ``interleave_weight`` (examples/dequantize_gemm/quantize/utils.py:50-125),
 ``pack_int4`` (examples/gemm_int4/example_tilelang_gemm_int4.py:59-67), the e2m1
 helpers of examples/dequantize_gemm/quantize/nvfp4.py:120-177, and ``gen_quant4``
-(examples/dequantize_gemm/quantize/utils.py:1-47) with a packer from its layout to this library's.
+(examples/dequantize_gemm/quantize/utils.py:1-47) with a packer from its layout to this library's, and the offline
+re-ordering of packed uint4 weights into the matrix instruction's operand order (``prepack_w4_fragments``).
 """
 
 from __future__ import annotations
@@ -152,3 +153,29 @@ def pack_gen_quant4(q: torch.Tensor, s: torch.Tensor, saturate: bool = False):
             raise ValueError("pack_gen_quant4: code 16 does not fit 4 bits (pass saturate=True to store 15)")
         codes = codes.clamp(max=15)
     return general_compress(codes.to(torch.int8), 4), s.t().contiguous().to(torch.float16)
+
+
+def prepack_w4_fragments(qweight: torch.Tensor) -> torch.Tensor:
+    """Packed uint4 weights ``[N, K/2]`` -> ``[N/16, K/128, 64, 16]`` bytes in the operand order of the 16x16x32 matrix
+    instruction: entry ``16*g + r`` of chunk ``c`` of block ``b`` holds bytes ``64*c + 16*g .. + 15`` of row ``16*b + r``.
+
+    The offline weight transform in the role of the one the reference's ladder kernel consumes
+    (examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:136-354, ``B_shape = (N/16, K/16, 16, 8)``): a wave
+    then fetches 1 KiB contiguous straight into operand registers.  Works on plain and on interleaved words alike (whole
+    16-byte pieces move).  N must be a multiple of 16, K of 128.
+    """
+    _require(qweight.dim() == 2, ValueError, "prepack_w4_fragments expects a 2-D packed tensor [N, K/2]")
+    n, kb = qweight.shape
+    _require(n % 16 == 0 and kb % 64 == 0, ValueError,
+             f"prepack_w4_fragments needs N % 16 == 0 and K % 128 == 0 (got N={n}, K={2 * kb})")
+    pieces = qweight.contiguous().view(torch.uint8).reshape(n // 16, 16, kb // 64, 4, 16)  # [b, r, c, g, byte]
+    return pieces.permute(0, 2, 3, 1, 4).reshape(n // 16, kb // 64, 64, 16).contiguous().view(qweight.dtype)
+
+
+def unpack_w4_fragments(fragments: torch.Tensor) -> torch.Tensor:
+    """Inverse of ``prepack_w4_fragments``: ``[N/16, K/128, 64, 16]`` -> ``[N, K/2]``."""
+    _require(fragments.dim() == 4 and fragments.shape[2:] == (64, 16), ValueError,
+             "unpack_w4_fragments expects [N/16, K/128, 64, 16]")
+    nb, nc = fragments.shape[:2]
+    pieces = fragments.contiguous().view(torch.uint8).reshape(nb, nc, 4, 16, 16)  # [b, c, g, r, byte]
+    return pieces.permute(0, 3, 1, 2, 4).reshape(nb * 16, nc * 64).contiguous().view(fragments.dtype)
