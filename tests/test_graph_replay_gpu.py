@@ -68,3 +68,48 @@ def test_graph_replays_match_eager(cuda):
         torch.cuda.synchronize()
         for got, want in zip([C1, C2, c3_g, o4_g], eager):
             assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_graph_replays_match_eager_batch_kernels(cuda):
+    """The K-sliced batch kernel (a voting barrier and 159 KiB of dynamic LDS), the register-resident kernel on
+    fragment-ordered weights and the unscaled bf16 x fp4 GEMM under capture."""
+    M1, N1, K1 = 32, 16 * 1400, 2048
+    d1 = workloads.w4a16(M1, N1, K1, 128, seed=5, zeros_range=(6, 10))
+    ks = tl.dequantize_gemv(M1, N1, K1, group_size=128, source_format="uint", with_scaling=True, with_zeros=True)
+    A1, B1, S1, Z1 = _dev(d1["A"], cuda), _dev(d1["B"], cuda).view(torch.int8), _dev(d1["Scale"], cuda), _dev(d1["Zeros"], cuda)
+    C1 = torch.empty((M1, N1), dtype=torch.float16, device=cuda)
+
+    M2, N2, K2 = 4, 1024, 4096
+    d2 = workloads.w4a16(M2, N2, K2, 128, seed=6)
+    fr = tl.dequantize_gemv(M2, N2, K2, group_size=128, source_format="int", with_scaling=True, weight_fragments=True)
+    A2, S2 = _dev(d2["A"], cuda), _dev(d2["Scale"], cuda)
+    B2 = tl.quantize.prepack_w4_fragments(_dev(d2["B"], cuda).view(torch.int8))
+    C2 = torch.empty((M2, N2), dtype=torch.float16, device=cuda)
+
+    M3, N3, K3 = 256, 256, 256
+    d3 = workloads.mxfp4(M3, N3, K3, seed=7, scale_bias=0)
+    f4 = tl.matmul_bf16_fp4(M3, N3, K3, fast_dequant=False)
+    A3, B3 = _dev(d3["A"], cuda).view(torch.bfloat16), _dev(d3["B"], cuda)
+
+    def run():
+        ks(A1, B1, S1, Z1, C1)
+        fr(A2, B2, S2, C2)
+        return f4(A3, B3)
+
+    c3_e = run()
+    torch.cuda.synchronize()
+    eager = [C1.clone(), C2.clone(), c3_e.clone()]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            c3_g = run()
+    for _ in range(3):
+        C1.fill_(float("nan"))
+        C2.fill_(float("nan"))
+        c3_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip([C1, C2, c3_g], eager):
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
