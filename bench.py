@@ -210,7 +210,7 @@ def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev, *
     return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
-def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True, **tk):
+def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True, kernel=None, **tk):
     """BitLinear forward on quantised operands: int8 x 2-bit (offset-binary ternary), fused acc/s_a/s_w epilogue.
 
     ``interleaved``: the packed words went through ``interleave_weight(qw, 2, "int8")`` on the host, once, as in
@@ -225,7 +225,7 @@ def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=
         B0 = tl.quantize.interleave_weight(B0, 2, "int8")
     Bs = [B0.to(dev).clone() for _ in range(nc)]
     s_a = torch.from_numpy(np.asarray(d["s_a"], dtype=np.float32)).to(dev)
-    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset", interleaved=interleaved)
+    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset", interleaved=interleaved, kernel=kernel)
     out = [None]
 
     def mk(i):

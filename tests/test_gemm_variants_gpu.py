@@ -309,3 +309,35 @@ def test_bitnet_decode_full_size(cuda):
     np.testing.assert_array_equal(C.cpu().numpy(), ref)
     np.testing.assert_allclose(out.float().cpu().numpy(), orc.post_quant_process(ref, d["s_a"].reshape(-1, 1), d["s_w"]).astype(np.float32),
                                rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
+@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288), (1, 8, 4096)])
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_bitnet_k_sliced_kernel_exact(cuda, convention, M, N, K, interleaved):
+    """The kernel that slices K over the waves of a workgroup (the library's choice at a few hundred rows), named
+    explicitly so that small and ragged shapes reach it: every int32 entry against the integer oracle, all codes,
+    the int8 range of A including -128, and the fused BitLinear epilogue against the tiled kernel's bits."""
+    rng = np.random.default_rng(M + K)
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    s_a = torch.tensor(rng.uniform(0.5, 3.0, size=M).astype(np.float32), device=cuda)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 2, "int8")
+    print(f"bitnet k-sliced: M={M} N={N} K={K} {convention} interleaved={interleaved}", flush=True)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention=convention, kernel="ksliced")(_dev(A, cuda), Bdev, C)
+    out = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="ksliced")(_dev(A, cuda), Bdev, s_a)
+    out_tiled = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="tiled")(_dev(A, cuda), Bdev, s_a)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
+    assert torch.equal(out.view(torch.int16), out_tiled.view(torch.int16))
+
+
+def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):
+    A = torch.zeros((64, 2048), dtype=torch.int8, device=cuda)
+    B = torch.zeros((128, 512), dtype=torch.int8, device=cuda)
+    C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError, match="K-sliced kernel needs"):
+        tl.bitnet_158_int8xint2_prefill(64, 128, 2048, convention="offset", kernel="ksliced")(A, B, C)

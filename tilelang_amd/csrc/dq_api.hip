@@ -46,6 +46,8 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int bitnet_epilogue, hipStream_t stream);
 int wlow_gemv(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M, int N, int K, int group,
               int bits, int convention, int layout, int zeros_rescale, hipStream_t stream);
+int i2_gemm_kslice(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
+                   float s_w, int bitnet_epilogue, int force, hipStream_t stream);
 int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int out_kind, hipStream_t stream);
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
@@ -337,11 +339,24 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
   if (convention < I2_UNSIGNED || convention > I2_TWOS) DQ_FAIL("%s: unknown code convention %d", fn, convention);
   if (layout != LAYOUT_PLAIN && layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
+  // bits 4 and 5 of out_kind name a kernel (tests and measurements): K sliced over the waves / the tiled GEMM
+  const int kernel_choice = out_kind & (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
+  out_kind &= ~(DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
   if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
+  if (kernel_choice == (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED)) DQ_FAIL("%s: out_kind names two kernels", fn);
   if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);
   if (out_kind == 1 && !(s_w != 0.f)) DQ_FAIL("%s: s_w must be non-zero", fn);
-  if (M <= 4) {  // decode: the streaming dot4 kernel
+  if (kernel_choice == DQ_I2_KERNEL_KSLICED) {
+    const int rc = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 1, (hipStream_t)stream);
+    if (rc > 0) DQ_FAIL("%s: the K-sliced kernel needs K %% 4096 == 0, K < 131072 and operands below 4 GiB (got M=%d N=%d K=%d)", fn, M, N, K);
+    return rc;
+  }
+  if (M <= 4 && !kernel_choice) {  // decode: the streaming dot4 kernel
     const int rc = i2_gemv(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
+  if (!kernel_choice) {  // a few hundred rows: K sliced over the waves of a workgroup
+    const int rc = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 0, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
   return i2_gemm(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);

@@ -727,6 +727,7 @@ def bitnet_158_int8xint2_prefill(
     warp_col_tiles: int = 32,
     chunk: int = 64,
     convention: str = "unsigned",
+    kernel: str | None = None,
 ) -> KernelAdapter:
     """BitNet W2A8 GEMM: ``C[M,N] int32 = A[M,K] int8 @ decode(B[N,K/4]).T``, exact; ``kernel(A, B, C)``.
 
@@ -734,7 +735,8 @@ def bitnet_158_int8xint2_prefill(
     tilelang_bitnet_158_int8xint2_prefill.py:72-85.  As there, ``fast_decoding=True`` takes B as
     ``interleave_weight(general_compress(W, 2), 2, "int8")`` (:372-374); ``fast_decoding=False`` takes the plain
     packing ``general_compress(W, 2)``.  ``convention``: ``"unsigned"`` (what the example's kernel decodes),
-    ``"offset"`` (``w = c - 2``, ternary weights stored as ``w + 2``) or ``"twos"``.
+    ``"offset"`` (``w = c - 2``, ternary weights stored as ``w + 2``) or ``"twos"``.  ``kernel`` (tests and
+    measurements): ``"ksliced"`` or ``"tiled"`` instead of the library's choice by shape; same bits either way.
     """
     if _dtype(in_dtype) != torch.int8 or _dtype(out_dtype) != torch.int32:
         raise ValueError("bitnet_158_int8xint2_prefill: int8 in, int32 out")
@@ -746,27 +748,40 @@ def bitnet_158_int8xint2_prefill(
               KernelParam("C", torch.int32, (M, N))]
 
     def launch(ptrs, stream):
-        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, layout, None, 1.0, 0, stream)
+        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, layout, None, 1.0, choice, stream)
 
+    choice = _i2_kernel_choice("bitnet_158_int8xint2_prefill", kernel)
     return KernelAdapter("bitnet_158_int8xint2_prefill", params, [], launch, _lib.last_error)
 
 
-def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "offset", interleaved: bool = False) -> KernelAdapter:
+_I2_KERNELS = {None: 0, "ksliced": 16, "tiled": 32}  # DQ_I2_KERNEL_* of include/dqgemm.h
+
+
+def _i2_kernel_choice(fn: str, kernel: str | None) -> int:
+    if kernel not in _I2_KERNELS:
+        raise ValueError(f"{fn}: kernel must be None, 'ksliced' or 'tiled' (got {kernel!r})")
+    return _I2_KERNELS[kernel]
+
+
+def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "offset", interleaved: bool = False,
+                        kernel: str | None = None) -> KernelAdapter:
     """BitLinear forward after activation quantisation: ``out[M,N] fp16 = ((A int8 @ W.T) / s_a[m]) / s_w``.
 
     The matmul plus ``post_quant_process`` of examples/bitnet-1.58b/utils_quant.py:165-170,199-209 in one
     kernel.  ``out = kernel(A, B, s_a)`` with ``s_a`` fp32 ``[M]`` (the per-row activation scale).
-    ``interleaved``: B went through ``interleave_weight(.., 2, "int8")``.
+    ``interleaved``: B went through ``interleave_weight(.., 2, "int8")``.  ``kernel``: as for
+    :func:`bitnet_158_int8xint2_prefill`.
     """
     if K % 128 != 0:
         raise ValueError(f"bitlinear_int8xint2: K={K} must be a multiple of 128")
     conv = _I2_CONVENTIONS[convention]
+    choice = _i2_kernel_choice("bitlinear_int8xint2", kernel)
     params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 4), packed=True),
               KernelParam("s_a", torch.float32, (M,)), KernelParam("out", torch.float16, (M, N))]
 
     def launch(ptrs, stream):
         return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv,
-                                                      LAYOUT_INTERLEAVED if interleaved else LAYOUT_PLAIN, ptrs[2], float(s_w), 1, stream)
+                                                      LAYOUT_INTERLEAVED if interleaved else LAYOUT_PLAIN, ptrs[2], float(s_w), 1 | choice, stream)
 
     return KernelAdapter("bitlinear_int8xint2", params, [-1], launch, _lib.last_error)
 
