@@ -202,12 +202,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0;
 
   // ---- issue order ------------------------------------------------------------------------------------------------
-  // The load unit takes a row per step and is the busiest unit of this kernel, so the loads are spread out: a block is
-  // eight groups of four matrix instructions, and group g of block t is followed by load g of A(t + 2), into the stage
-  // block t was read from; every second group by one weight load: during the second block of pair P the X loads of
-  // pair P + 2 (into the registers of the first block's operands, which are done), during the first block of pair
-  // P + 1 its Y loads (into those of the second block's operands of pair P).  Every block thus issues twelve loads, and
-  // at the start of a block the twelve of the block before may still be in flight: what it needs is older.
+  // A block is eight groups of four matrix instructions; group g of block t is followed by load g of A(t + 2), into
+  // the stage block t was read from, and every second group by one weight load: during the second block of pair P the
+  // X loads of pair P + 2 (into the registers of the first block's operands, which are done), during the first block of
+  // pair P + 1 its Y loads (into those of the second block's operands of pair P).  Every block thus issues twelve
+  // loads, and at the start of a block the twelve of the block before may still be in flight: what it needs is older.
+  // (The compiler is free to move matrix instructions across the loads; pinning them with scheduling barriers
+  // measured 5 % slower.)
   constexpr int kPerBlock = kAOps + kNB;
   // The prologue issues what block 0 needs first and then twelve more loads (block 1's activations and the X loads of
   // pair 1), as the block before block 0 would have.
@@ -248,14 +249,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
 #pragma unroll
             for (int mb = 0; mb < kMB; ++mb) acc[mb][nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf, af[mb][s], acc[mb][nb], 0, 0, 0);
           }
-          __builtin_amdgcn_sched_barrier(0);
           load_a(t + 2, g);
           if constexpr ((g & 1) == 1) {
             constexpr int nbw = g >> 1;  // the fourth of the block's weight loads this is
             if constexpr (b == 1) load_w(q_tag, std::integral_constant<int, 2 * nbw>{}, pair + 2);
             else load_w(std::integral_constant<int, q ^ 1>{}, std::integral_constant<int, 2 * nbw + 1>{}, pair + 1);
           }
-          __builtin_amdgcn_sched_barrier(0);
         });
       });
     });
