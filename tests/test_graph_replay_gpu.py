@@ -72,7 +72,7 @@ def test_graph_replays_match_eager(cuda):
 
 def test_graph_replays_match_eager_batch_kernels(cuda):
     """The K-sliced batch kernel (a voting barrier and 159 KiB of dynamic LDS), the register-resident kernel on
-    fragment-ordered weights and the unscaled bf16 x fp4 GEMM under capture."""
+    fragment-ordered weights, the unscaled bf16 x fp4 GEMM and the K-sliced BitNet GEMM under capture."""
     M1, N1, K1 = 32, 16 * 1400, 2048
     d1 = workloads.w4a16(M1, N1, K1, 128, seed=5, zeros_range=(6, 10))
     ks = tl.dequantize_gemv(M1, N1, K1, group_size=128, source_format="uint", with_scaling=True, with_zeros=True)
@@ -91,25 +91,31 @@ def test_graph_replays_match_eager_batch_kernels(cuda):
     f4 = tl.matmul_bf16_fp4(M3, N3, K3, fast_dequant=False)
     A3, B3 = _dev(d3["A"], cuda).view(torch.bfloat16), _dev(d3["B"], cuda)
 
+    # BitLinear at 64 tiles of 64 x 128 with a long K: the kernel that slices K over the waves (128 KiB of LDS, loads
+    # counted by hand)
+    M5, N5, K5 = 64, 8192, 4096
+    d5 = workloads.bitnet(M5, N5, K5, seed=8)
+    bl = tl.bitlinear_int8xint2(M5, N5, K5, float(d5["s_w"]))
+    A5, B5, sa5 = _dev(d5["A"], cuda), _dev(d5["B"], cuda).view(torch.int8), _dev(d5["s_a"], cuda)
+
     def run():
         ks(A1, B1, S1, Z1, C1)
         fr(A2, B2, S2, C2)
-        return f4(A3, B3)
+        return f4(A3, B3), bl(A5, B5, sa5)
 
-    c3_e = run()
+    c3_e, c5_e = run()
     torch.cuda.synchronize()
-    eager = [C1.clone(), C2.clone(), c3_e.clone()]
+    eager = [C1.clone(), C2.clone(), c3_e.clone(), c5_e.clone()]
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            c3_g = run()
+            c3_g, c5_g = run()
     for _ in range(3):
-        C1.fill_(float("nan"))
-        C2.fill_(float("nan"))
-        c3_g.fill_(float("nan"))
+        for t in (C1, C2, c3_g, c5_g):
+            t.fill_(float("nan"))
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for got, want in zip([C1, C2, c3_g], eager):
+        for got, want in zip([C1, C2, c3_g, c5_g], eager):
             assert torch.equal(got.view(torch.int16), want.view(torch.int16))
