@@ -31,16 +31,18 @@ struct Int32Out {
 
 // BitLinear: out = (float(acc) / s_a[m]) / s_w -> fp16, two fp32 divides in that order
 // (examples/bitnet-1.58b/utils_quant.py:165-170).  p.S = s_a (float[M]), p.f0 = s_w.
-struct BitnetOut {
+template <int SHIFT>
+struct BitnetOutS {
   static constexpr bool kTransposed = false;
   using out_t = half_t;
   __device__ static __forceinline__ out_t finish(uint32_t raw, const Params& p, int m, int) {
-    float v = (float)(int32_t)raw;
+    float v = (float)((int32_t)raw >> SHIFT);  // operands decoded as 2^SHIFT x value: exact
     v = v / ((const float*)p.S)[m];
     v = v / p.f0;
     return (half_t)v;
   }
 };
+using BitnetOut = BitnetOutS<0>;
 
 // ---- int8 x 2-bit ---------------------------------------------------------------------------------
 // Plain layout: packed byte j of a row holds codes 4j..4j+3 at bits 0, 2, 4, 6; (w >> 2i) & 0x03030303
@@ -49,8 +51,12 @@ struct BitnetOut {
 // kernel_benchmark/tilelang_bitnet_158_int8xint2_decode.py:196-234: element e at byte e % 4, slot
 // e / 4), the layout the reference's kernels consume; the same shift-and-mask yields elements
 // 4i..4i+3 in natural order and A needs no transform.
-template <int CONV, class EPI, bool INTERLEAVED>
+// TOP (signed conventions, K < 131072): the codes are shifted to the top two bits of their byte instead, where the
+// int8 reading of the byte is 64 sext2(c) (offset binary: c - 2 = sext2(c ^ 2), the flip in the same three-input bit
+// operation as the mask): two instructions per dword instead of three, and the epilogue shifts the sum back by 6.
+template <int CONV, class EPI, bool INTERLEAVED, bool TOP = false>
 struct I2Policy : I8Mfma, gemm::NoScale, EPI {
+  static_assert(!TOP || CONV != I2_UNSIGNED, "unsigned codes are masked in place");
   static constexpr int kBRowBytes = 32;
   static constexpr bool kAPacked = false;
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : transpose4x4_bytes(v); }
@@ -63,6 +69,12 @@ struct I2Policy : I8Mfma, gemm::NoScale, EPI {
   }
   __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
     frag_t o;
+    if constexpr (TOP) {
+      constexpr uint32_t flip = CONV == I2_OFFSET ? 0x80808080u : 0u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = (int)(((w[j] << (6 - 2 * i)) & 0xC0C0C0C0u) ^ flip);
+      return o;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       uint32_t d = (w[j] >> (2 * i)) & 0x03030303u;
@@ -131,14 +143,25 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int bitnet_epilogue, hipStream_t stream) {
   Params p = gemm::make_params(A, B, s_a, nullptr, nullptr, C, M, N, K);
   p.f0 = s_w;
-#define DQ_I2L(CONV_, IL_)                                                                      \
+#define DQ_I2P(POL_BITNET_, POL_INT32_)                                                         \
   do {                                                                                          \
-    if (gemm::dma_eligible<I2Policy<CONV_, BitnetOut, IL_>>(p)) {                               \
-      if (bitnet_epilogue) return gemm::launch_dma<I2Policy<CONV_, BitnetOut, IL_>>(p, stream); \
-      return gemm::launch_dma<I2Policy<CONV_, Int32Out<0, false>, IL_>>(p, stream);             \
+    if (gemm::dma_eligible<POL_BITNET_>(p)) {                                                   \
+      if (bitnet_epilogue) return gemm::launch_dma<POL_BITNET_>(p, stream);                     \
+      return gemm::launch_dma<POL_INT32_>(p, stream);                                           \
     }                                                                                           \
-    if (bitnet_epilogue) return gemm::launch_auto<I2Policy<CONV_, BitnetOut, IL_>>(p, stream);  \
-    return gemm::launch_auto<I2Policy<CONV_, Int32Out<0, false>, IL_>>(p, stream);              \
+    if (bitnet_epilogue) return gemm::launch_auto<POL_BITNET_>(p, stream);                      \
+    return gemm::launch_auto<POL_INT32_>(p, stream);                                            \
+  } while (0)
+#define DQ_I2L(CONV_, IL_)                                                                            \
+  do {                                                                                                \
+    using PlainB = I2Policy<CONV_, BitnetOut, IL_>;                                                   \
+    using PlainI = I2Policy<CONV_, Int32Out<0, false>, IL_>;                                          \
+    if constexpr (CONV_ != I2_UNSIGNED) {                                                             \
+      using TopB = I2Policy<CONV_, BitnetOutS<6>, IL_, true>;                                         \
+      using TopI = I2Policy<CONV_, Int32Out<6, false>, IL_, true>;                                    \
+      if (K < 131072) DQ_I2P(TopB, TopI); /* 128 x 128 x K stays below 2^31 */                          \
+    }                                                                                                 \
+    DQ_I2P(PlainB, PlainI);                                                                           \
   } while (0)
 #define DQ_I2(CONV_)                                        \
   do {                                                      \
@@ -153,6 +176,7 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
   }
 #undef DQ_I2
 #undef DQ_I2L
+#undef DQ_I2P
 }
 
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int decode, int a_packed, int transposed,
