@@ -341,3 +341,24 @@ def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):
     C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
     with pytest.raises(RuntimeError, match="K-sliced kernel needs"):
         tl.bitnet_158_int8xint2_prefill(64, 128, 2048, convention="offset", kernel="ksliced")(A, B, C)
+
+
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_bitnet_default_dispatch_takes_the_k_sliced_kernel_on_ragged_shapes(cuda, interleaved):
+    """165 tiles of 64 x 128 with K = 4096: the library's own choice is the K-sliced kernel; M and N are ragged and N is
+    not a multiple of 8 (element-wise stores).  Every int32 entry against the oracle and the tiled kernel."""
+    M, N, K = 300, 4100, 4096
+    rng = np.random.default_rng(7)
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 2, "int8")
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    Ct = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    print(f"bitnet default dispatch: M={M} N={N} K={K} interleaved={interleaved}", flush=True)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention="offset")(_dev(A, cuda), Bdev, C)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention="offset", kernel="tiled")(_dev(A, cuda), Bdev, Ct)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, "offset"))
+    assert torch.equal(C, Ct)
