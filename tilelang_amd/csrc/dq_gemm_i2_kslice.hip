@@ -19,8 +19,8 @@
 //   * weights: a load instruction that puts 32 different rows into adjacent lanes costs the load unit as much as four
 //     that read whole lines (it handles a row per step, whatever the row's share of the instruction), and with 32
 //     bytes per row and block that alone took as long as the matrix instructions.  So a weight load covers 16 rows x
-//     64 bytes (two blocks of 128 k; lane l: row l / 4, piece l % 4), two loads X, Y per block of 32 rows, kept two
-//     blocks ahead in registers; one ds_bpermute_b32 per dword regroups the lanes of a register as
+//     64 bytes (two blocks of 128 k; lane l: row l / 4, piece l % 4), two loads X, Y per block of 32 rows, two to
+//     four blocks ahead in registers; one ds_bpermute_b32 per dword regroups the lanes of a register as
 //     [k half h][block b][row] and one v_permlane16_swap_b32 per dword pair exchanges the odd quarters of X with the
 //     even quarters of Y, which leaves the operand of block 0 (rows 0..31 x halves 0, 1) in one register and that of
 //     block 1 in the other.  Dword s of an operand feeds step s: the contraction index of step s is labelled
@@ -28,9 +28,10 @@
 //   * both streams are issued from inline assembly and tracked by hand: loads return in order, every issue point
 //     issues the same number of loads (past the end of the slice: the last block again, unused), and one
 //     s_waitcnt vmcnt per block lets the loads that are younger than the ones needed stay in flight.
-//   * decode: 7-8 instructions per 16 weights.  Signed codes are moved to the top two bits of their byte, where the
-//     int8 reading of the byte is 64 sext2(c) (offset binary: c - 2 = sext2(c ^ 2), one XOR per packed dword); the
-//     accumulators then hold 64 x the sum and are shifted back once, exactly.  Unsigned codes are masked in place.
+//   * decode: 7 instructions per 16 weights.  Signed codes are moved to the top two bits of their byte, where the
+//     int8 reading of the byte is 64 sext2(c) (offset binary: c - 2 = sext2(c ^ 2), the flip in the same three-input
+//     bit operation as the mask); the accumulators then hold 64 x the sum and are shifted back once, exactly.
+//     Unsigned codes are masked in place.
 //   * the matrix instruction takes the weights as its row operand, so a lane's four consecutive accumulator values
 //     are four consecutive output columns of one row: the partial sums go to LDS as 16-byte pieces and come back as
 //     two pieces (8 columns) per lane, summed over the eight K slices in integer arithmetic (any order is exact),
