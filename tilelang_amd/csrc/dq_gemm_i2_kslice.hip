@@ -341,8 +341,8 @@ int i2_gemm_kslice(const void* A, const void* B, void* C, int M, int N, int K, i
   if ((uint64_t)(M + kTileM) * (uint64_t)K >= (1ull << 32) || (uint64_t)(N + kTileN) * (uint64_t)(K >> 2) >= (1ull << 32)) return 1;
   const long tiles = (long)((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
   // worth it where the tiles are few enough that a tiled kernel leaves each CU one long chain (measured at
-  // N = K = 8192: ahead of the tiled kernel up to M = 768, three tiles per CU)
-  if (!force && (tiles < 64 || tiles > 768 || K < 4096)) return 1;
+  // N = K = 8192: ahead of the tiled kernel up to M = 448, level with it there, behind from M = 512 on)
+  if (!force && (tiles < 64 || tiles > 448 || K < 4096)) return 1;
 #define DQ_I2K(CONV_, IL_)                                                                                              \
   do {                                                                                                                  \
     if (bitnet_epilogue)                                                                                                \
