@@ -46,6 +46,20 @@ def test_w2a16_exact_integers(cuda, M, N, K, fast, fmt):
     np.testing.assert_array_equal(got.astype(np.float64), acc.astype(np.float16).astype(np.float64))
 
 
+@pytest.mark.parametrize("N", [1, 2, 7, 9, 31, 513, 4099, 7919, 57347])
+@pytest.mark.parametrize("K", [512, 4096, 8192, 16384])
+def test_w2a16_rows_split_over_workgroups(cuda, N, K):
+    """The grid hands every workgroup an even share of the rows whatever N is (row counts that are odd, prime,
+    smaller than a batch, or too many for 512 workgroups): each output row must come out once and exact, with K
+    chosen so that a row takes a quarter of a wave, one wave, two waves and two chunks per thread."""
+    A, packed = _inputs(1, N, K, seed=N + K, integer_a=True)
+    B = orc.interleave_weight(packed.view(np.int8), 2, "float16").view(np.uint8)
+    kernel = tl.dequantize_gemv(1, N, K, "float16", "float16", "float32", num_bits=2, source_format="int", fast_decoding=True)
+    got = _run(kernel, cuda, A, B)
+    acc = A.astype(np.int64) @ orc.decode_i2(packed, "offset").astype(np.int64).T
+    np.testing.assert_array_equal(got.astype(np.float64), acc.astype(np.float16).astype(np.float64))
+
+
 @pytest.mark.parametrize("M,N,K,group", [(1, 1024, 1024, 128), (1, 28672, 8192, 128), (2, 300, 4096, 64), (4, 1024, 8192, 8192),
                                          (1, 512, 11008, 64)])
 @pytest.mark.parametrize("fast,fmt", [(False, "int"), (True, "int"), (True, "uint")])
