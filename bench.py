@@ -210,12 +210,13 @@ def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev, *
     return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
-def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True, kernel=None, **tk):
+def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=True, kernel=None, fragments=False, **tk):
     """BitLinear forward on quantised operands: int8 x 2-bit (offset-binary ternary), fused acc/s_a/s_w epilogue.
 
     ``interleaved``: the packed words went through ``interleave_weight(qw, 2, "int8")`` on the host, once, as in
     the reference's kernel benchmarks (examples/bitnet-1.58b/kernel_benchmark/
-    tilelang_bitnet_158_int8xint2_prefill.py:372-373, ..._decode.py:249-250); False: the plain packing."""
+    tilelang_bitnet_158_int8xint2_prefill.py:372-373, ..._decode.py:249-250); False: the plain packing.
+    ``fragments``: the words then re-ordered offline into the matrix instruction's operand order."""
     d = workloads.bitnet(M, N, K, seed=0)
     nbytes = workloads.bitnet_bytes(M, N, K)
     nc = _copies(nbytes, hi=40)
@@ -223,9 +224,12 @@ def bench_bitnet(torch, tl, workloads, M, N, K, steps, warmup, dev, interleaved=
     B0 = torch.from_numpy(d["B"]).view(torch.int8)
     if interleaved:
         B0 = tl.quantize.interleave_weight(B0, 2, "int8")
+    if fragments:
+        B0 = tl.quantize.prepack_i2_fragments(B0)
     Bs = [B0.to(dev).clone() for _ in range(nc)]
     s_a = torch.from_numpy(np.asarray(d["s_a"], dtype=np.float32)).to(dev)
-    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset", interleaved=interleaved, kernel=kernel)
+    kern = tl.bitlinear_int8xint2(M, N, K, float(d["s_w"]), convention="offset", interleaved=interleaved, kernel=kernel,
+                                  weight_fragments=fragments)
     out = [None]
 
     def mk(i):
@@ -451,6 +455,9 @@ def main():
         for m in (1, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m == 1 else gemm))
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        r = bench_bitnet(torch, tl, workloads, 256, 8192, 8192, S, W, dev, fragments=True, **gemm)
+        shapes.append(_row("bitnet_w2a8 M=256 N=8192 K=8192 (weights re-ordered offline into the matrix instruction's operand order)",
+                           r, "mfma", MFMA_I8_PEAK))
         r = bench_bitnet(torch, tl, workloads, 2048, 8192, 8192, S, W, dev, interleaved=False, **gemm)
         shapes.append(_row("bitnet_w2a8 M=2048 N=8192 K=8192 (plain packing, not interleaved)", r, "mfma", MFMA_I8_PEAK))
         r = bench_w4a16(torch, tl, workloads, 4096, 8192, 8192, True, S, W, dev, **gemm)

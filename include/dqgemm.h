@@ -56,7 +56,11 @@ enum dq_w4_layout {
                                of that chunk of row r of the block.  The role of the weight transform of
                                examples/dequantize_gemm/example_dequant_gemm_fine_grained.py:136-354
                                (B[N/16][K/16][16][8], micro-tiles of the NVIDIA instruction), for this chip's 16x16x32
-                               instruction; its BitBLAS permutation inside a tile is third-party and not reproduced. */
+                               instruction; its BitBLAS permutation inside a tile is third-party and not reproduced.
+                               call_gemm_int8xint2 takes the flag too, with the order of the 32x32x32 int8 instruction:
+                               B[(N+31)/32][K/128][64][16 bytes], entry 32 h + r of a 128-k chunk = bytes 16 h .. + 15
+                               of that chunk (32 bytes) of row r of the block of 32, rows past N zero; the K-sliced
+                               kernel is the one that reads it (K % 4096 == 0).                                      */
 };
 
 /* ---- W4A16 ---------------------------------------------------------------------------- */

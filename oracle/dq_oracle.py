@@ -851,3 +851,22 @@ def prepack_w4_fragments(B):
                 for r in range(16):
                     out[b, c, 16 * g + r, :] = B[16 * b + r, 64 * c + 16 * g: 64 * c + 16 * g + 16]
     return out
+
+
+def prepack_i2_fragments(B):
+    """Packed 2-bit weights [N, K/4] -> [ceil(N/32), K/128, 64, 16] bytes: entry 32 h + r of chunk c of block b holds bytes
+    32 c + 16 h .. + 15 of row 32 b + r (rows past N: zeros) -- the operand order of the 32x32x32 int8 matrix instruction
+    (lane 32 h + r owns k = 64 h .. 64 h + 63 of a 128-k chunk of row r).  Plain loops over the index formula (test
+    infrastructure, as prepack_w4_fragments above); the reference has no counterpart for its BitNet kernels."""
+    B = np.ascontiguousarray(B).view(np.uint8)
+    N, KB = B.shape
+    assert KB % 32 == 0
+    blocks = (N + 31) // 32
+    out = np.zeros((blocks, KB // 32, 64, 16), np.uint8)
+    for b in range(blocks):
+        for c in range(KB // 32):
+            for h in range(2):
+                for r in range(32):
+                    if 32 * b + r < N:
+                        out[b, c, 32 * h + r, :] = B[32 * b + r, 32 * c + 16 * h: 32 * c + 16 * h + 16]
+    return out

@@ -335,6 +335,46 @@ def test_bitnet_k_sliced_kernel_exact(cuda, convention, M, N, K, interleaved):
     assert torch.equal(out.view(torch.int16), out_tiled.view(torch.int16))
 
 
+@pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
+@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288)])
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_bitnet_fragment_ordered_weights_exact(cuda, convention, M, N, K, interleaved):
+    """Weights re-ordered offline into the matrix instruction's operand order (``prepack_i2_fragments``; N ragged, so
+    the last block of 32 rows is padded): every int32 entry against the integer oracle, and the fused BitLinear
+    epilogue against the bits of the row-major path."""
+    rng = np.random.default_rng(M + K + 1)
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    s_a = torch.tensor(rng.uniform(0.5, 3.0, size=M).astype(np.float32), device=cuda)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 2, "int8")
+    Bfrag = quantize.prepack_i2_fragments(Bdev)
+    assert Bfrag.shape == ((N + 31) // 32, K // 128, 64, 16)
+    assert torch.equal(quantize.unpack_i2_fragments(Bfrag, N), Bdev)
+    print(f"bitnet fragments: M={M} N={N} K={K} {convention} interleaved={interleaved}", flush=True)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention=convention, weight_fragments=True)(_dev(A, cuda), Bfrag, C)
+    out = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, weight_fragments=True)(_dev(A, cuda), Bfrag, s_a)
+    out_rows = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="ksliced")(_dev(A, cuda), Bdev, s_a)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
+    assert torch.equal(out.view(torch.int16), out_rows.view(torch.int16))
+
+
+def test_bitnet_fragment_ordered_weights_need_the_k_sliced_kernel(cuda):
+    """Through the C-ABI: a K the K-sliced kernel cannot slice, and the tiled kernel named together with the flag."""
+    lib = tl._lib.get_library()
+    A = torch.zeros((64, 2048), dtype=torch.int8, device=cuda)
+    B = torch.zeros((4, 16, 64, 16), dtype=torch.int8, device=cuda)
+    C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 2048, 1, 2, None, 1.0, 0, stream) == -1
+    assert "K-sliced kernel needs" in tl._lib.last_error()
+    assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 4096, 1, 2, None, 1.0, 32, stream) == -1
+    assert "K-sliced kernel only" in tl._lib.last_error()
+
+
 def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):
     A = torch.zeros((64, 2048), dtype=torch.int8, device=cuda)
     B = torch.zeros((128, 512), dtype=torch.int8, device=cuda)

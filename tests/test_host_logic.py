@@ -330,3 +330,27 @@ def test_fragment_prepack_matches_the_oracle_and_inverts():
         with pytest.raises(ValueError, match="fragment-ordered weights"):
             tl.dequantize_gemv(args["M"], args["N"], args["K"], group_size=args["group_size"], source_format="int",
                                with_scaling=True, weight_fragments=True)
+
+
+
+def test_i2_fragment_prepack_matches_the_oracle_and_inverts():
+    """quantize.prepack_i2_fragments against the oracle's index formula (N ragged: the last block of 32 rows is padded
+    with zeros), its inverse, and the factories' shape rules."""
+    rng = np.random.default_rng(5)
+    B = rng.integers(0, 256, size=(70, 96), dtype=np.uint8)  # N = 70, K = 384
+    frag = quantize.prepack_i2_fragments(torch.from_numpy(B))
+    assert frag.shape == (3, 3, 64, 16)
+    np.testing.assert_array_equal(frag.numpy(), orc.prepack_i2_fragments(B))
+    np.testing.assert_array_equal(quantize.unpack_i2_fragments(frag, 70).numpy(), B)
+    assert quantize.unpack_i2_fragments(frag).shape == (96, 96)
+    with pytest.raises(ValueError, match="K % 128 == 0"):
+        quantize.prepack_i2_fragments(torch.zeros(32, 48, dtype=torch.uint8))
+    with pytest.raises(ValueError, match="does not fit"):
+        quantize.unpack_i2_fragments(frag, 64)
+    kern = tl.bitnet_158_int8xint2_prefill(256, 1001, 8192, weight_fragments=True)
+    assert kern.params[1].shape == (32, 64, 64, 16)
+    assert tl.bitlinear_int8xint2(256, 128, 4096, 1.0, weight_fragments=True).params[1].shape == (4, 32, 64, 16)
+    with pytest.raises(ValueError, match="K % 4096 == 0"):
+        tl.bitnet_158_int8xint2_prefill(256, 128, 2048, weight_fragments=True)
+    with pytest.raises(ValueError, match="K-sliced kernel only"):
+        tl.bitlinear_int8xint2(256, 128, 4096, 1.0, kernel="tiled", weight_fragments=True)

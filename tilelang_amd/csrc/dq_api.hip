@@ -338,10 +338,15 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   const char* fn = "call_gemm_int8xint2";
   if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
   if (convention < I2_UNSIGNED || convention > I2_TWOS) DQ_FAIL("%s: unknown code convention %d", fn, convention);
-  if (layout != LAYOUT_PLAIN && layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
+  const int word_layout = layout & ~LAYOUT_FRAGMENTS;
+  if (word_layout != LAYOUT_PLAIN && word_layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
   // bits 4 and 5 of out_kind name a kernel (tests and measurements): K sliced over the waves / the tiled GEMM
-  const int kernel_choice = out_kind & (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
+  int kernel_choice = out_kind & (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
   out_kind &= ~(DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
+  if (layout & LAYOUT_FRAGMENTS) {  // only the K-sliced kernel reads the fragment order
+    if (kernel_choice == DQ_I2_KERNEL_TILED) DQ_FAIL("%s: fragment-ordered weights are read by the K-sliced kernel only", fn);
+    kernel_choice = DQ_I2_KERNEL_KSLICED;
+  }
   if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
   if (kernel_choice == (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED)) DQ_FAIL("%s: out_kind names two kernels", fn);
   if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);

@@ -37,6 +37,10 @@
 //     two pieces (8 columns) per lane, summed over the eight K slices in integer arithmetic (any order is exact),
 //     finished by the epilogue and stored 16 bytes (fp16) or 32 bytes (int32) per lane.
 //
+//   * FRAG: the weights were re-ordered offline into the operand order, B[(N + 31) / 32][K / 128][64 lanes][16 bytes]
+//     (lane 32 h + r of block (nb, kb): bytes 32 kb + 16 h .. + 15 of row 32 nb + r, rows past N zero).  A load is then
+//     1 KiB contiguous, lands as the operand it is, and nothing is regrouped; same loads at the same points of the loop.
+//
 // Rows beyond M or N are read as the last row (their results are not stored).
 #include <type_traits>
 #include <utility>
@@ -126,7 +130,7 @@ struct Int32Finish {
   __device__ __forceinline__ out_t operator()(int acc, int) const { return acc; }
 };
 
-template <int CONV, bool IL, class FIN>
+template <int CONV, bool IL, bool FRAG, class FIN>
 __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                    typename FIN::out_t* __restrict__ C, int M, int N, int K,
                                                                    int tiles_m, int tiles_n, FIN fin) {
@@ -166,16 +170,27 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
 #pragma unroll
   for (int s = 0; s < 4; ++s) a_rd[s] = (uint32_t)r * 128u + (uint32_t)(((4 * h + s) ^ ((r >> 1) & 7)) << 4);
 
-  // ---- weights: load i of block of rows nb: lane l has piece l % 4 (64 k) of row 32 nb + 16 i + l / 4 --------------
+  // ---- weights: load o of a pair of blocks.  Row-major: rows 16 o .. + 15 of the tile, lane l has piece l % 4 (64 k of
+  // the pair's 256) of row 16 o + l / 4.  Fragment order: block o % 2 of the pair for the 32 rows o / 2, 1 KiB as stored.
   uint4_t w_raw[2][kWOps];
-  const uint32_t w_row_bytes = (uint32_t)(K >> 2);
-  uint32_t w_voff[kWOps];
-#pragma unroll
-  for (int o = 0; o < kWOps; ++o) w_voff[o] = (uint32_t)min(n0 + 16 * o + (lane >> 2), N - 1) * w_row_bytes + (uint32_t)(lane & 3) * 16u;
-  const uint8_t* const w_base = B + (size_t)wave * (kslice >> 2);
   const int npair = nblk >> 1;
-  auto load_w = [&](auto q_tag, auto o_tag, int pair) {  // load o of a pair of blocks
-    load16(w_raw[decltype(q_tag)::value][decltype(o_tag)::value], w_voff[decltype(o_tag)::value], w_base + min(pair, npair - 1) * 64);
+  uint32_t w_voff[kWOps];
+  const uint8_t* w_base;
+  if constexpr (FRAG) {
+    const int row_blocks = (N + 31) >> 5;
+#pragma unroll
+    for (int o = 0; o < kWOps; ++o)
+      w_voff[o] = ((uint32_t)min((n0 >> 5) + (o >> 1), row_blocks - 1) * (uint32_t)(K >> 7) + (uint32_t)(o & 1)) * 1024u + (uint32_t)lane * 16u;
+    w_base = B + (size_t)wave * nblk * 1024;
+  } else {
+    const uint32_t w_row_bytes = (uint32_t)(K >> 2);
+#pragma unroll
+    for (int o = 0; o < kWOps; ++o) w_voff[o] = (uint32_t)min(n0 + 16 * o + (lane >> 2), N - 1) * w_row_bytes + (uint32_t)(lane & 3) * 16u;
+    w_base = B + (size_t)wave * (kslice >> 2);
+  }
+  constexpr int kPairBytes = FRAG ? 2048 : 64;  // from one pair of blocks to the next, per load
+  auto load_w = [&](auto q_tag, auto o_tag, int pair) {
+    load16(w_raw[decltype(q_tag)::value][decltype(o_tag)::value], w_voff[decltype(o_tag)::value], w_base + min(pair, npair - 1) * kPairBytes);
   };
   // lane (h, b, j) = 32 h + 16 b + j of the regrouped register takes lane 4 j + 2 b + h of the loaded one
   const int w_from = ((lane & 15) * 4 + ((lane >> 4) & 1) * 2 + (lane >> 5)) * 4;
@@ -228,7 +243,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
         constexpr int b = decltype(b_tag)::value;
         const int t = 2 * pair + b;
         wait_loads<kPerBlock>(w_raw);
-        if constexpr (b == 0) regroup_w(q_tag);
+        if constexpr (b == 0 && !FRAG) regroup_w(q_tag);
         const unsigned char* const st = ring + b * kStage;  // t % 2 == b
         int4_t af[kMB][4];
 #pragma unroll
@@ -317,9 +332,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
   });
 }
 
-template <int CONV, bool IL, class FIN>
+template <int CONV, bool IL, bool FRAG, class FIN>
 int launch_i2_kslice(const void* A, const void* B, void* C, int M, int N, int K, FIN fin, hipStream_t stream) {
-  auto kern = i2_kslice_kernel<CONV, IL, FIN>;
+  auto kern = i2_kslice_kernel<CONV, IL, FRAG, FIN>;
   static bool raised[kMaxDevices] = {};
   if (raise_lds_limit<kLds>(kern, raised)) return -1;
   const int tiles_m = (M + kTileM - 1) / kTileM, tiles_n = (N + kTileN - 1) / kTileN;
@@ -343,16 +358,21 @@ int i2_gemm_kslice(const void* A, const void* B, void* C, int M, int N, int K, i
   // worth it where the tiles are few enough that a tiled kernel leaves each CU one long chain (measured at
   // N = K = 8192: ahead of the tiled kernel up to M = 448, level with it there, behind from M = 512 on)
   if (!force && (tiles < 64 || tiles > 448 || K < 4096)) return 1;
-#define DQ_I2K(CONV_, IL_)                                                                                              \
+#define DQ_I2K(CONV_, IL_, FRAG_)                                                                                       \
   do {                                                                                                                  \
     if (bitnet_epilogue)                                                                                                \
-      return launch_i2_kslice<CONV_, IL_>(A, B, C, M, N, K, BitnetFinish{(const float*)s_a, s_w}, stream);              \
-    return launch_i2_kslice<CONV_, IL_>(A, B, C, M, N, K, Int32Finish{}, stream);                                       \
+      return launch_i2_kslice<CONV_, IL_, FRAG_>(A, B, C, M, N, K, BitnetFinish{(const float*)s_a, s_w}, stream);       \
+    return launch_i2_kslice<CONV_, IL_, FRAG_>(A, B, C, M, N, K, Int32Finish{}, stream);                                \
   } while (0)
-#define DQ_I2KL(CONV_)                                   \
-  do {                                                   \
-    if (layout == LAYOUT_INTERLEAVED) DQ_I2K(CONV_, true); \
-    DQ_I2K(CONV_, false);                                \
+#define DQ_I2KL(CONV_)                                                  \
+  do {                                                                  \
+    const bool il = (layout & ~LAYOUT_FRAGMENTS) == LAYOUT_INTERLEAVED; \
+    if (layout & LAYOUT_FRAGMENTS) {                                    \
+      if (il) DQ_I2K(CONV_, true, true);                                \
+      DQ_I2K(CONV_, false, true);                                       \
+    }                                                                   \
+    if (il) DQ_I2K(CONV_, true, false);                                 \
+    DQ_I2K(CONV_, false, false);                                        \
   } while (0)
   switch (convention) {
     case I2_UNSIGNED: DQ_I2KL(I2_UNSIGNED);

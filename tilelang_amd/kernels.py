@@ -728,6 +728,7 @@ def bitnet_158_int8xint2_prefill(
     chunk: int = 64,
     convention: str = "unsigned",
     kernel: str | None = None,
+    weight_fragments: bool = False,
 ) -> KernelAdapter:
     """BitNet W2A8 GEMM: ``C[M,N] int32 = A[M,K] int8 @ decode(B[N,K/4]).T``, exact; ``kernel(A, B, C)``.
 
@@ -737,6 +738,8 @@ def bitnet_158_int8xint2_prefill(
     packing ``general_compress(W, 2)``.  ``convention``: ``"unsigned"`` (what the example's kernel decodes),
     ``"offset"`` (``w = c - 2``, ternary weights stored as ``w + 2``) or ``"twos"``.  ``kernel`` (tests and
     measurements): ``"ksliced"`` or ``"tiled"`` instead of the library's choice by shape; same bits either way.
+    ``weight_fragments=True``: B went through ``quantize.prepack_i2_fragments`` (after ``interleave_weight`` when
+    ``fast_decoding``) and has the shape ``[ceil(N/32), K/128, 64, 16]``; read by the K-sliced kernel (K % 4096 == 0).
     """
     if _dtype(in_dtype) != torch.int8 or _dtype(out_dtype) != torch.int32:
         raise ValueError("bitnet_158_int8xint2_prefill: int8 in, int32 out")
@@ -744,7 +747,12 @@ def bitnet_158_int8xint2_prefill(
         raise ValueError(f"bitnet_158_int8xint2_prefill: K={K} must be a multiple of 128")
     conv = _I2_CONVENTIONS[convention]
     layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
-    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 4), packed=True),
+    b_shape = (N, K // 4)
+    if weight_fragments:
+        _i2_fragments_ok("bitnet_158_int8xint2_prefill", K, kernel)
+        layout |= LAYOUT_FRAGMENTS
+        b_shape = ((N + 31) // 32, K // 128, 64, 16)
+    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, b_shape, packed=True),
               KernelParam("C", torch.int32, (M, N))]
 
     def launch(ptrs, stream):
@@ -757,6 +765,13 @@ def bitnet_158_int8xint2_prefill(
 _I2_KERNELS = {None: 0, "ksliced": 16, "tiled": 32}  # DQ_I2_KERNEL_* of include/dqgemm.h
 
 
+def _i2_fragments_ok(fn: str, K: int, kernel: str | None) -> None:
+    if K % 4096 != 0 or K >= 131072:
+        raise ValueError(f"{fn}: weight_fragments needs K % 4096 == 0 and K < 131072 (got K={K})")
+    if kernel == "tiled":
+        raise ValueError(f"{fn}: weight_fragments is read by the K-sliced kernel only")
+
+
 def _i2_kernel_choice(fn: str, kernel: str | None) -> int:
     if kernel not in _I2_KERNELS:
         raise ValueError(f"{fn}: kernel must be None, 'ksliced' or 'tiled' (got {kernel!r})")
@@ -764,24 +779,30 @@ def _i2_kernel_choice(fn: str, kernel: str | None) -> int:
 
 
 def bitlinear_int8xint2(M: int, N: int, K: int, s_w: float, convention: str = "offset", interleaved: bool = False,
-                        kernel: str | None = None) -> KernelAdapter:
+                        kernel: str | None = None, weight_fragments: bool = False) -> KernelAdapter:
     """BitLinear forward after activation quantisation: ``out[M,N] fp16 = ((A int8 @ W.T) / s_a[m]) / s_w``.
 
     The matmul plus ``post_quant_process`` of examples/bitnet-1.58b/utils_quant.py:165-170,199-209 in one
     kernel.  ``out = kernel(A, B, s_a)`` with ``s_a`` fp32 ``[M]`` (the per-row activation scale).
-    ``interleaved``: B went through ``interleave_weight(.., 2, "int8")``.  ``kernel``: as for
+    ``interleaved``: B went through ``interleave_weight(.., 2, "int8")``.  ``kernel`` and ``weight_fragments``: as for
     :func:`bitnet_158_int8xint2_prefill`.
     """
     if K % 128 != 0:
         raise ValueError(f"bitlinear_int8xint2: K={K} must be a multiple of 128")
     conv = _I2_CONVENTIONS[convention]
     choice = _i2_kernel_choice("bitlinear_int8xint2", kernel)
-    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, (N, K // 4), packed=True),
+    layout = LAYOUT_INTERLEAVED if interleaved else LAYOUT_PLAIN
+    b_shape = (N, K // 4)
+    if weight_fragments:
+        _i2_fragments_ok("bitlinear_int8xint2", K, kernel)
+        layout |= LAYOUT_FRAGMENTS
+        b_shape = ((N + 31) // 32, K // 128, 64, 16)
+    params = [KernelParam("A", torch.int8, (M, K)), KernelParam("B", torch.int8, b_shape, packed=True),
               KernelParam("s_a", torch.float32, (M,)), KernelParam("out", torch.float16, (M, N))]
 
     def launch(ptrs, stream):
-        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv,
-                                                      LAYOUT_INTERLEAVED if interleaved else LAYOUT_PLAIN, ptrs[2], float(s_w), 1 | choice, stream)
+        return _lib.get_library().call_gemm_int8xint2(ptrs[0], ptrs[1], ptrs[3], M, N, K, conv, layout, ptrs[2], float(s_w),
+                                                      1 | choice, stream)
 
     return KernelAdapter("bitlinear_int8xint2", params, [-1], launch, _lib.last_error)
 

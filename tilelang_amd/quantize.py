@@ -179,3 +179,37 @@ def unpack_w4_fragments(fragments: torch.Tensor) -> torch.Tensor:
     nb, nc = fragments.shape[:2]
     pieces = fragments.contiguous().view(torch.uint8).reshape(nb, nc, 4, 16, 16)  # [b, c, g, r, byte]
     return pieces.permute(0, 3, 1, 2, 4).reshape(nb * 16, nc * 64).contiguous().view(fragments.dtype)
+
+
+def prepack_i2_fragments(qweight: torch.Tensor) -> torch.Tensor:
+    """Packed 2-bit weights ``[N, K/4]`` -> ``[ceil(N/32), K/128, 64, 16]`` bytes in the operand order of the 32x32x32
+    int8 matrix instruction: entry ``32*h + r`` of chunk ``c`` of block ``b`` holds bytes ``32*c + 16*h .. + 15`` of row
+    ``32*b + r`` (64 codes); rows past N are zero.
+
+    The same offline transform as :func:`prepack_w4_fragments`, for the BitNet W2A8 GEMM that slices K over the waves
+    of a workgroup: a wave fetches 1 KiB contiguous straight into an operand register.  Works on plain and on
+    interleaved words alike (whole 16-byte pieces move).  K must be a multiple of 128.
+    """
+    _require(qweight.dim() == 2, ValueError, "prepack_i2_fragments expects a 2-D packed tensor [N, K/4]")
+    n, kb = qweight.shape
+    _require(kb % 32 == 0, ValueError, f"prepack_i2_fragments needs K % 128 == 0 (got K={4 * kb})")
+    blocks = (n + 31) // 32
+    rows = qweight.contiguous().view(torch.uint8)
+    if blocks * 32 != n:
+        rows = torch.cat([rows, rows.new_zeros((blocks * 32 - n, kb))])
+    pieces = rows.reshape(blocks, 32, kb // 32, 2, 16)  # [b, r, c, h, byte]
+    return pieces.permute(0, 2, 3, 1, 4).reshape(blocks, kb // 32, 64, 16).contiguous().view(qweight.dtype)
+
+
+def unpack_i2_fragments(fragments: torch.Tensor, n: int | None = None) -> torch.Tensor:
+    """Inverse of :func:`prepack_i2_fragments`: ``[ceil(N/32), K/128, 64, 16]`` -> ``[N, K/4]`` (``n`` drops the padding rows)."""
+    _require(fragments.dim() == 4 and fragments.shape[2:] == (64, 16), ValueError,
+             "unpack_i2_fragments expects [ceil(N/32), K/128, 64, 16]")
+    nb, nc = fragments.shape[:2]
+    pieces = fragments.contiguous().view(torch.uint8).reshape(nb, nc, 2, 32, 16)  # [b, c, h, r, byte]
+    rows = pieces.permute(0, 3, 1, 2, 4).reshape(nb * 32, nc * 32)
+    if n is not None:
+        _require(nb * 32 - 31 <= n <= nb * 32, ValueError, f"unpack_i2_fragments: n={n} does not fit {nb} blocks of 32 rows")
+        rows = rows[:n]
+    return rows.contiguous().view(fragments.dtype)
+
