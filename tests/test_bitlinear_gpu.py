@@ -50,3 +50,26 @@ def test_bitlinear_forward(cuda, interleave, batch):
     acc = xq.astype(np.int64) @ wq.astype(np.int64).T
     ref = orc.post_quant_process(acc, sa, sw).astype(np.float32) + bias.astype(np.float32)[None, :]
     np.testing.assert_allclose(out.float().cpu().numpy().reshape(-1, out_f), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_bitlinear_layer_with_fragment_ordered_copy(cuda):
+    """``prefill_fragments=True``: the layer keeps a second, fragment-ordered copy of its weights and hands it to the
+    K-sliced kernel at the batch sizes that kernel serves (here 256 rows: 64 tiles), the row-major copy elsewhere
+    (8 rows); both layers must give the same bits at both sizes."""
+    in_f, out_f = 4096, 2048
+    rng = np.random.default_rng(11)
+    W = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
+    plain = tl.BitLinear(in_f, out_f)
+    frag = tl.BitLinear(in_f, out_f, prefill_fragments=True)
+    for layer in (plain, frag):
+        layer.load_float_weight(torch.from_numpy(W))
+        layer.to(cuda)
+    assert frag.qweight_fragments is not None and frag.qweight_fragments.is_cuda and plain.qweight_fragments is None
+    assert frag._takes_fragments(256) and not frag._takes_fragments(8) and not plain._takes_fragments(256)
+    for M in (256, 8):
+        x = torch.from_numpy(rng.standard_normal((M, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
+        a, b = plain(x), frag(x)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert not tl.BitLinear(1024, 768, prefill_fragments=True).prefill_fragments  # in_features the kernel cannot slice
+
