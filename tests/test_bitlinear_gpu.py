@@ -64,12 +64,22 @@ def test_bitlinear_layer_with_fragment_ordered_copy(cuda):
     for layer in (plain, frag):
         layer.load_float_weight(torch.from_numpy(W))
         layer.to(cuda)
-    assert frag.qweight_fragments is not None and frag.qweight_fragments.is_cuda and plain.qweight_fragments is None
     assert frag._takes_fragments(256) and not frag._takes_fragments(8) and not plain._takes_fragments(256)
     for M in (256, 8):
         x = torch.from_numpy(rng.standard_normal((M, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
         a, b = plain(x), frag(x)
         torch.cuda.synchronize()
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert frag.qweight_fragments is not None and frag.qweight_fragments.is_cuda and plain.qweight_fragments is None
+    # weights replaced through the state dict: the fragment copy follows
+    W2 = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
+    plain.load_float_weight(torch.from_numpy(W2))
+    plain.to(cuda)
+    frag.load_state_dict(plain.state_dict())
+    assert frag._sw_value == plain._sw_value
+    x = torch.from_numpy(rng.standard_normal((256, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
+    a, b = plain(x), frag(x)
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     assert not tl.BitLinear(1024, 768, prefill_fragments=True).prefill_fragments  # in_features the kernel cannot slice
 

@@ -49,9 +49,11 @@ class BitLinear(nn.Module):
         self.weight_bits, self.input_bits = weight_bits, input_bits
         self.interleave = interleave
         self.prefill_fragments = bool(prefill_fragments) and in_features % 4096 == 0 and in_features < 131072
-        self.qweight_fragments = None
+        self.qweight_fragments = None  # built on first use from qweight, rebuilt when qweight is replaced or moved
+        self._fragments_of = None
         self.register_buffer("qweight", torch.zeros((out_features, in_features // 4), dtype=torch.int8))
         self.register_buffer("sw", torch.ones((), dtype=torch.float32))
+        self._sw_value = 1.0
         self.bias = None
         self._kernels = {}
 
@@ -70,16 +72,29 @@ class BitLinear(nn.Module):
         if self.interleave:
             packed = quantize.interleave_weight(packed, 2, "int8")
         self.qweight = packed.to(self.qweight.device).contiguous()
-        self.qweight_fragments = quantize.prepack_i2_fragments(self.qweight) if self.prefill_fragments else None
         self.sw = sw.to(torch.float32).to(self.sw.device)
         self._sw_value = float(self.sw)
         self.bias = None if bias is None else bias.detach().to(self.qweight.device)
         self._kernels.clear()
 
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        # the weight scale is baked into the kernels as a number
+        self._sw_value = float(self.sw)
+        self._kernels.clear()
+
     def _takes_fragments(self, M: int) -> bool:
         # the shapes the library gives to the kernel that slices K over the waves (tiles of 64 x 128)
         tiles = ((M + 63) // 64) * ((self.out_features + 127) // 128)
-        return self.qweight_fragments is not None and 64 <= tiles <= 448
+        return self.prefill_fragments and 64 <= tiles <= 448
+
+    def _fragments(self) -> torch.Tensor:
+        """The fragment-ordered copy of ``qweight`` (not part of the state dict: it follows whatever ``qweight`` holds)."""
+        key = (self.qweight.data_ptr(), self.qweight._version, str(self.qweight.device))
+        if self._fragments_of != key:
+            self.qweight_fragments = quantize.prepack_i2_fragments(self.qweight)
+            self._fragments_of = key
+        return self.qweight_fragments
 
     def _get_kernels(self, M: int):
         k = self._kernels.get(M)
@@ -90,11 +105,6 @@ class BitLinear(nn.Module):
             self._kernels[M] = k
         return k
 
-    def _apply(self, fn, *args, **kwargs):  # the fragment copy is a plain attribute: it follows .to() / .cuda()
-        super()._apply(fn, *args, **kwargs)
-        if self.qweight_fragments is not None:
-            self.qweight_fragments = fn(self.qweight_fragments)
-        return self
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         x = input.reshape(-1, self.in_features)
@@ -102,7 +112,7 @@ class BitLinear(nn.Module):
             x = x.to(torch.float16)
         quant, gemm = self._get_kernels(x.shape[0])
         x_q, s_a = quant(x.contiguous())
-        out = gemm(x_q, self.qweight_fragments if self._takes_fragments(x.shape[0]) else self.qweight, s_a)
+        out = gemm(x_q, self._fragments() if self._takes_fragments(x.shape[0]) else self.qweight, s_a)
         if self.bias is not None:
             out += self.bias.view(1, -1).expand_as(out)
         return out.reshape(*input.shape[:-1], self.out_features)
