@@ -114,7 +114,8 @@ def _copies(nbytes, min_total=640 << 20, lo=2, hi=24):
     return int(min(hi, max(lo, -(-min_total // max(nbytes, 1)))))
 
 
-def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False, fragments=False, **tk):
+def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interleaved=False, fragments=False,
+                zeros_mode="original", **tk):
     group = 128
     d = workloads.w4a16(M, N, K, group, seed=0, scale_range=(0.002, 0.01) if zeros else (0.005, 0.02),
                         zeros_range=(6, 10) if zeros else None)
@@ -138,7 +139,8 @@ def bench_w4a16(torch, tl, workloads, M, N, K, zeros, steps, warmup, dev, interl
     Zs = [torch.from_numpy(d["Zeros"]).to(dev).clone() for _ in range(nc)] if zeros else None
     C = torch.empty((M, N), dtype=torch.float16, device=dev)
     kern = tl.dequantize_gemv(M, N, K, group_size=group, source_format="uint" if zeros else "int",
-                              with_scaling=True, with_zeros=zeros, fast_decoding=interleaved, weight_fragments=fragments)
+                              with_scaling=True, with_zeros=zeros, fast_decoding=interleaved, weight_fragments=fragments,
+                              zeros_mode=zeros_mode)
     if zeros:
         fns = [(lambda i=i: kern(A, Bs[i], Ss[i], Zs[i], C, skip_tensor_validation=True)) for i in range(nc)]
     else:

@@ -42,7 +42,14 @@ enum dq_w4_mode {
   DQ_W4_SCALE = 3,          /* w = rne16((q-8)*s)         lop3.py:41-75 (i4s_scale)                    */
   DQ_W4_USCALE = 4,         /* w = rne16(q*s)             lop3.py:77-81 (i4u_scale)                    */
   DQ_W4_ZEROS_ORIGINAL = 5, /* w = rne16(rne16(q-z)*s)    lop3.py:136-176, quantization.py:321-330     */
-  DQ_W4_ZEROS_RESCALE = 6   /* w = rne16(fma(q,s,-z))     lop3.py:233-271                              */
+  DQ_W4_ZEROS_RESCALE = 6,  /* w = rne16(fma(q,s,-z))     lop3.py:233-271                              */
+  DQ_W4_ZEROS_FOLDED = 7    /* w = rne16(fma(q,s,-rne16(z*s))): the "original" formula (q-z)*s with the zero point
+                               folded into one fused multiply-add per weight.  No counterpart in the reference: it
+                               differs from DQ_W4_ZEROS_ORIGINAL by the rounding of z*s (relative 2^-11 of z*s, shared
+                               by the weights of a group) and saves four instructions per packed word.  The batch
+                               kernels of call_dequantize_gemv_w4a16 above 16 rows use it for DQ_W4_ZEROS_ORIGINAL
+                               when `variant` < 0 (results stay inside rtol = atol = 1e-2 of the reference); the tiled
+                               GEMM and call_dequantize_w4 use it only when asked for by this value.             */
 };
 
 enum dq_w4_layout {
@@ -62,6 +69,12 @@ enum dq_w4_layout {
                                of that chunk (32 bytes) of row r of the block of 32, rows past N zero; the K-sliced
                                kernel is the one that reads it (K % 4096 == 0).                                      */
 };
+
+/* Flag for the `layout` of call_dequantize_w4 only: decode with the fp8-converter decoder (a nibble in a byte read as
+ * OCP e4m3 is q * 2^-9; the streaming batch kernel and the tiled W4 GEMM decode this way) instead of the mantissa-mask
+ * decoder of the other kernels.  The two produce the same bits in every mode; the flag exists so that a test can
+ * see both. */
+#define DQ_DECODER_CONVERTER 4
 
 /* ---- W4A16 ---------------------------------------------------------------------------- */
 

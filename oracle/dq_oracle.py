@@ -466,6 +466,8 @@ def dequant_u4_scale_zeros(packed: np.ndarray, scale: np.ndarray, zeros: np.ndar
     ``original``:  ``RNE16(RNE16(q - z) * s)``      (lop3.py:136-176, sub then fma)
     ``rescale``:   ``RNE16(fma(q, s, -z))``          (lop3.py:233-271)
     ``quantized``: ``RNE16((q - qz) * s)``, qz int   (lop3.py:326-363)
+    ``folded``:    ``RNE16(fma(q, s, -RNE16(z * s)))``: not a reference formula; the library's cheaper form of
+                   ``original`` (DQ_W4_ZEROS_FOLDED), restated here so that its tile can be checked bit for bit.
     Also examples/dequantize_gemm/quantize/quantization.py:321-330.
     PARITY UNPINNED by reference tests (no caller in the reference).
     """
@@ -482,6 +484,10 @@ def dequant_u4_scale_zeros(packed: np.ndarray, scale: np.ndarray, zeros: np.ndar
     if mode == "quantized":
         qz = _expand_groups(np.asarray(zeros).astype(np.int32), K, group).astype(np.float32)
         return (((q - qz) * s) + np.float32(0.0)).astype(np.float16)
+    if mode == "folded":
+        z = _expand_groups(np.asarray(zeros, dtype=np.float16), K, group).astype(np.float32)
+        zs = (z * s).astype(np.float16).astype(np.float64)  # z * s is exact in fp32 (11 x 11 bits): one rounding
+        return (q.astype(np.float64) * s.astype(np.float64) - zs).astype(np.float16)  # exact in fp64: one rounding
     raise ValueError(mode)
 
 

@@ -169,7 +169,7 @@ def test_fp16_fp4_weights_exact(cuda):
     np.testing.assert_array_equal(out.cpu().numpy().astype(np.float32), orc.decode_fp4_simple_f16(B).astype(np.float32))
 
 
-@pytest.mark.parametrize("mode", ["scale", "original", "rescale", "signed"])
+@pytest.mark.parametrize("mode", ["scale", "original", "rescale", "signed", "folded"])
 @pytest.mark.parametrize("interleaved", [False, True])
 @pytest.mark.parametrize("M,N,K", [(200, 320, 512), (1500, 2000, 256), (3581, 3589, 128), (3581, 3589, 768),
                                    (3584, 3584, 256)])  # 128x64, 128x128, 256x256 tiles; the last two: direct-to-LDS kernel
@@ -179,6 +179,7 @@ def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
     d = workloads.w4a16(M, N, K, group, seed=2, scale_range=(0.002, 0.01), zeros_range=(6, 10))
     kw = {"scale": dict(source_format="int"), "original": dict(source_format="uint", with_zeros=True),
           "rescale": dict(source_format="uint", with_zeros=True, zeros_mode="rescale"),
+          "folded": dict(source_format="uint", with_zeros=True, zeros_mode="folded"),
           "signed": dict(with_scaling=False)}[mode]
     Bdev = _dev(d["B"], cuda).view(torch.int8)
     if interleaved:
@@ -196,6 +197,38 @@ def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
     torch.cuda.synchronize()
     ref = orc.ref_w4a16(d["A"], d["B"], d["Scale"], d["Zeros"], group, mode)
     np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("mode", ["scale", "original", "rescale", "folded"])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("N", [300, 3584])  # register-staged tiles / the direct-to-LDS kernel
+def test_w4a16_large_m_tile_exact_through_identity(cuda, mode, interleaved, N):
+    """An identity for A makes the GEMM write its dequantised tile: C[k, n] = W[n, k], every bit, with scales that
+    exercise the rounding (and fractional, negative zero points)."""
+    K, group = 512, 128
+    M = 3584 if N == 3584 else K
+    d = workloads.w4a16(1, N, K, group, seed=11, scale_range=(0.002, 0.02), zeros_range=(6, 10))
+    B, S, Z = d["B"], d["Scale"], d["Zeros"]
+    B[1, :] = np.arange(K // 2, dtype=np.uint8)
+    S[2, :] = np.array([6.1e-5, 1.0, -0.013, 655.0], dtype=np.float16)
+    Z[3, :] = np.array([7.5, -3.25, 0.0, 15.0], dtype=np.float16)
+    kw = {"scale": dict(source_format="int"), "original": dict(source_format="uint", with_zeros=True),
+          "rescale": dict(source_format="uint", with_zeros=True, zeros_mode="rescale"),
+          "folded": dict(source_format="uint", with_zeros=True, zeros_mode="folded")}[mode]
+    W = orc.dequant_u4_scale(B, S, group) if mode == "scale" else orc.dequant_u4_scale_zeros(B, S, Z, group, mode)
+    A = np.zeros((M, K), dtype=np.float16)
+    A[np.arange(K), np.arange(K)] = 1.0
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 4, "float16")
+    kern = tl.matmul_w4a16(M, N, K, group_size=group, fast_decoding=interleaved, **kw)
+    args = [_dev(A, cuda), Bdev, _dev(S, cuda)] + ([_dev(Z, cuda)] if kw.get("with_zeros") else [])
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(*args, C)
+    torch.cuda.synchronize()
+    got = C.cpu().numpy()
+    np.testing.assert_array_equal(got[:K].view(np.uint16), np.ascontiguousarray(W.T).view(np.uint16))
+    assert not got[K:].any()
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])

@@ -30,6 +30,7 @@ def _mode_kwargs(mode):
         "uscale": dict(source_format="uint", with_scaling=True),
         "original": dict(source_format="uint", with_scaling=True, with_zeros=True, zeros_mode="original"),
         "rescale": dict(source_format="uint", with_scaling=True, with_zeros=True, zeros_mode="rescale"),
+        "folded": dict(source_format="uint", with_scaling=True, with_zeros=True, zeros_mode="folded"),
     }[mode]
 
 
@@ -49,9 +50,12 @@ def _oracle_tile(mode, B, S, Z, group):
     return orc.dequant_u4_scale_zeros(B, S, Z, group, mode)
 
 
-@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
+@pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale", "folded"])
 @pytest.mark.parametrize("interleaved", [False, True])
-def test_dequant_tile_bit_exact(cuda, mode, interleaved):
+@pytest.mark.parametrize("decoder", ["mask", "converter"])
+def test_dequant_tile_bit_exact(cuda, mode, interleaved, decoder):
+    """Both device decoders (nibbles OR-ed into an fp16 mantissa; nibbles read as fp8 by the hardware converter)
+    against the oracle's tile, bit for bit, in every mode and both word layouts."""
     N, K, group = 96, 512, 128
     d = workloads.w4a16(1, N, K, group, seed=3, scale_range=(0.002, 0.02), zeros_range=(6, 10))
     B, S, Z = d["B"], d["Scale"], d["Zeros"]
@@ -68,7 +72,7 @@ def test_dequant_tile_bit_exact(cuda, mode, interleaved):
     if interleaved:
         Bdev = tl.quantize.interleave_weight(Bdev, 4, "float16")
     # the tile kernel takes the layout from fast_decoding; the decode formula from the rest
-    kern = tl.dequantize_w4(N, K, group, fast_decoding=interleaved, _formula_fast=fast, **kw)
+    kern = tl.dequantize_w4(N, K, group, fast_decoding=interleaved, _formula_fast=fast, decoder=decoder, **kw)
     args = [Bdev]
     if kw.get("with_scaling"):
         args.append(_dev(S, cuda))
@@ -211,7 +215,7 @@ def test_kernel_variants(cuda, variant):
     _run_gemv(cuda, 1, 1000, 2048 + 128, 128, "original", variant=variant)
 
 
-@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35, 36])
+@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35, 36, 70, 72, 74, 76])
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
 def test_streaming_small_batch_kernel(cuda, variant, mode):
     """The direct-to-LDS kernel: ragged M and N, a single K step, fewer steps than ring stages, many steps,
@@ -224,6 +228,40 @@ def test_streaming_small_batch_kernel(cuda, variant, mode):
     _run_gemv(cuda, 5, 64, 256 * 9, 128, mode, variant=variant, interleaved=True)
     _run_gemv(cuda, 16, 256, 4096, 128, mode, variant=variant)
     _run_gemv(cuda, 20, 300, 11008, 128, mode, variant=variant)
+
+
+@pytest.mark.parametrize("variant,mode", [(32, "original"), (36, "original"), (31, "scale"), (36, "rescale"), (33, "signed"),
+                                          (72, "original"), (76, "original"), (36, "folded")])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_streaming_small_batch_kernel_tile_exact_through_identity(cuda, variant, mode, interleaved):
+    """Rows of an identity for A make the streaming kernel write its dequantised tile: C[m, n] = W[n, k0 + m], every
+    bit.  Variants 30..36 keep the reference's rounding of every weight in every mode; 70..76 decode "original" with
+    the zero point folded into a fused multiply-add and must equal the oracle's "folded" tile."""
+    N, K, group, M = 200, 1536, 128, 64
+    d = workloads.w4a16(1, N, K, group, seed=12, scale_range=(0.002, 0.02), zeros_range=(6, 10))
+    B, S, Z = d["B"], d["Scale"], d["Zeros"]
+    B[1, :] = np.arange(K // 2, dtype=np.uint8)
+    S[2, :4] = np.array([6.1e-5, 1.0, -0.013, 655.0], dtype=np.float16)
+    Z[3, :4] = np.array([7.5, -3.25, 0.0, 15.0], dtype=np.float16)
+    tile_mode = "folded" if (variant >= 70 and mode == "original") else mode
+    W = _oracle_tile(tile_mode, B, S, Z, group)
+    kw = _mode_kwargs(mode)
+    fast = kw.pop("fast_decoding", False)
+    if mode == "signed" and interleaved:
+        pytest.skip("the sign-extending decoder is the plain-layout slow path")
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, fast_decoding=interleaved,
+                              _formula_fast=fast, variant=variant, **kw)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = tl.quantize.interleave_weight(Bdev, 4, "float16")
+    for k0 in (0, 200, K - M):  # columns of the identity block: every position inside a word and a group is hit
+        A = np.zeros((M, K), dtype=np.float16)
+        A[np.arange(M), k0 + np.arange(M)] = 1.0
+        args = [_dev(A, cuda), Bdev] + ([_dev(S, cuda)] if kw.get("with_scaling") else []) + ([_dev(Z, cuda)] if kw.get("with_zeros") else [])
+        C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+        kern(*args, C)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(C.cpu().numpy().view(np.uint16), np.ascontiguousarray(W[:, k0:k0 + M].T).view(np.uint16))
 
 
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])

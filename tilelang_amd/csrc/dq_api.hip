@@ -136,6 +136,10 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout & ~LAYOUT_FRAGMENTS)) return -1;
   if (K % 128 != 0) DQ_FAIL("%s: K=%d must be a multiple of 128", fn, K);
   if (!aligned16(A) || !aligned16(C)) DQ_FAIL("%s: A and C must be 16-byte aligned", fn);
+  // "folded" differs from "original" in the rounding of z * s only; the kernels below that have no folded decoder
+  // of their own run "original" for it (tile-exact or fp32 arithmetic, either way inside the folded form's error)
+  const int asked_mode = mode;
+  if (mode == W4_ZEROS_FOLDED) mode = W4_ZEROS_ORIGINAL;
   if (layout & LAYOUT_FRAGMENTS) {
     // weights re-ordered offline into the matrix instruction's operand order: read by the register-resident
     // small-batch kernel only
@@ -149,7 +153,7 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   }
   // prefill-sized M: the tiled MFMA GEMM (same tile-exact decoders); up to 128 rows the streaming kernel
   // below (two passes over the weights) is still the faster one.  50: the GEMM whatever M.
-  if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, (hipStream_t)stream);
+  if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread (r = 0: its own
   // choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  60, 61: the K-sliced batch kernel
   // (M <= 64, N >= 22400) with two / more pairs of activation loads in flight.  40: the kernel with
@@ -176,8 +180,17 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     if (rc > 0) DQ_FAIL("%s: the K-sliced batch kernel does not cover M=%d N=%d K=%d group=%d mode=%d", fn, M, N, K, group, mode);
     return rc;
   }
+  // 70..76: as 30..36 with the zero point folded into one fused multiply-add per weight pair (only "original"
+  // differs from the tile-exact form: RNE16(q s - RNE16(z s)) instead of RNE16(RNE16(q - z) s)); the default
+  // above 16 rows
+  const int folded_mode = mode == W4_ZEROS_ORIGINAL ? W4_ZEROS_FOLDED : mode;
+  if (variant >= 70 && variant < 80) {
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, folded_mode, layout, variant - 70, (hipStream_t)stream);
+    if (rc > 0) DQ_FAIL("%s: the streaming small-batch kernel does not cover N=%d K=%d group=%d", fn, N, K, group);
+    return rc;
+  }
   if (variant >= 30 && variant < 40) {
-    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant - 30, (hipStream_t)stream);
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, variant - 30, (hipStream_t)stream);
     if (rc > 0) DQ_FAIL("%s: the streaming small-batch kernel does not cover N=%d K=%d group=%d", fn, N, K, group);
     return rc;
   }
@@ -191,7 +204,7 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
     const bool wide = N >= 128 * 200;
     const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : 6);
-    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, config, (hipStream_t)stream);
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, folded_mode, layout, config, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
   return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
@@ -229,7 +242,7 @@ extern "C" int call_dequantize_w4(const void* B, const void* Scale, const void* 
                                   int mode, int layout, dq_stream_t stream) {
   const char* fn = "call_dequantize_w4";
   if (!W) DQ_FAIL("%s: W is expected to have non-NULL data pointer", fn);
-  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout)) return -1;
+  if (check_w4_args(fn, B, Scale, Zeros, N, K, group, mode, layout & ~DECODER_CONVERTER)) return -1;
   if (K % 8 != 0) DQ_FAIL("%s: K=%d must be a multiple of 8", fn, K);
   if (!aligned16(W)) DQ_FAIL("%s: W must be 16-byte aligned", fn);
   return w4_dequant(B, Scale, Zeros, W, N, K, group, mode, layout, (hipStream_t)stream);

@@ -75,7 +75,9 @@ enum W4Mode : int {
   W4_USCALE = 4,          // w = RNE16(q * s)
   W4_ZEROS_ORIGINAL = 5,  // w = RNE16(RNE16(q - z) * s)
   W4_ZEROS_RESCALE = 6,   // w = RNE16(fma(q, s, -z))
-  W4_MODE_COUNT = 7,
+  W4_ZEROS_FOLDED = 7,    // w = RNE16(fma(q, s, -RNE16(z * s))): (q - z) * s with the zero point folded into one
+                          // fused multiply-add; differs from W4_ZEROS_ORIGINAL by the rounding of z * s
+  W4_MODE_COUNT = 8,
 };
 
 enum W4Layout : int {
@@ -83,6 +85,7 @@ enum W4Layout : int {
   LAYOUT_INTERLEAVED = 1,  // word already permuted for the fast 16-bit decoder (elements 0,2,4,6,1,3,5,7)
   LAYOUT_FRAGMENTS = 2,    // flag, added to one of the above: 16-byte pieces re-ordered offline into the matrix
                            // instruction's operand order, [N / 16][K / 128][64 lanes][16 bytes] (uint4, decode GEMV only)
+  DECODER_CONVERTER = 4,   // flag of call_dequantize_w4 only: dump the tile with the fp8-converter decoder
 };
 
 enum Fp4Format : int {
@@ -157,11 +160,71 @@ __device__ __forceinline__ half8_t decode_w4(uint32_t w, half_t s, half_t z) {
       const half2_t b2 = {bias, bias};
       const half2_t z2 = {z, z};
       r[i] = __builtin_elementwise_fma((x - b2) - z2, s2, zero2);
+    } else if constexpr (MODE == W4_ZEROS_FOLDED) {
+      const half2_t b2 = {bias, bias};
+      const half_t nzs = (half_t)(-(z * s));
+      const half2_t nzs2 = {nzs, nzs};
+      r[i] = __builtin_elementwise_fma(x - b2, s2, nzs2);
     } else {  // W4_ZEROS_RESCALE
       const half2_t b2 = {bias, bias};
       const half2_t nz2 = {(half_t)(-z), (half_t)(-z)};
       r[i] = __builtin_elementwise_fma(x - b2, s2, nz2);
     }
+  }
+  half8_t o;
+  o[0] = r[0][0]; o[1] = r[0][1]; o[2] = r[1][0]; o[3] = r[1][1];
+  o[4] = r[2][0]; o[5] = r[2][1]; o[6] = r[3][0]; o[7] = r[3][1];
+  return o;
+}
+
+// ---- uint4 -> fp16 through the fp8 converter ------------------------------------------------------------
+// A byte 0x0q read as OCP e4m3 is q * 2^-9 for every q in 0..15 (q < 8 is subnormal, q >= 8 sits in the first
+// binade: together one linear range).  v_cvt_scalef32_pk_f16_fp8 multiplies by the power of two of its scale
+// operand (the scale's mantissa is ignored by the hardware), so with scale 512 two bytes become the exact
+// integers as an fp16 pair: eight weights cost 3 bit operations and 4 conversions.  The even nibbles of a word
+// land in one source dword and the odd ones in another; NATURAL spends two v_perm_b32 on the bytes so that the
+// result is in element order 0..7 for either word layout (the activations then need no permutation).  Without
+// NATURAL a plain word yields elements (0 2 4 6 1 3 5 7) and an interleaved word (0 4 1 5 2 6 3 7).
+template <bool INTERLEAVED, bool NATURAL>
+__device__ __forceinline__ void u4x8_to_half_cvt(uint32_t w, half2_t out[4]) {
+  const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+  uint32_t x = even, y = odd;
+  if constexpr (NATURAL) {
+    // plain: even = (n0 n2 n4 n6), odd = (n1 n3 n5 n7); interleaved: even = (e0 e4 e1 e5), odd = (e2 e6 e3 e7)
+    x = __builtin_amdgcn_perm(odd, even, INTERLEAVED ? 0x06040200u : 0x05010400u);
+    y = __builtin_amdgcn_perm(odd, even, INTERLEAVED ? 0x07050301u : 0x07030602u);
+  }
+  out[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, 512.0f, false);
+  out[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x, 512.0f, true);
+  out[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(y, 512.0f, false);
+  out[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(y, 512.0f, true);
+}
+
+// The second operand of decode_w4_cvt for a (row, group): computed once and used for every word of the group.
+template <int MODE>
+__device__ __forceinline__ half_t w4_cvt_addend(half_t s, half_t z) {
+  if constexpr (MODE == W4_SCALE) return (half_t)((half_t)-8.f * s);       // exact: a power of two times s
+  else if constexpr (MODE == W4_ZEROS_FOLDED) return (half_t)(-(z * s));   // one rounding
+  else if constexpr (MODE == W4_ZEROS_ORIGINAL || MODE == W4_ZEROS_RESCALE) return (half_t)(-z);
+  else return (half_t)0.f;
+}
+
+// Decode one word of eight uint4 weights with the converter above.  Same values, bit for bit, as decode_w4<MODE>
+// in every mode of the C-ABI: (q - 8) * s is one fused multiply-add with the exact addend -8 s, (q - z) * s is an
+// addition (the reference's first rounding) and a multiplication (its second), fma(q, s, -z) is itself.
+template <int MODE, bool INTERLEAVED, bool NATURAL>
+__device__ __forceinline__ half8_t decode_w4_cvt(uint32_t w, half_t s, half_t addend) {
+  half2_t r[4];
+  u4x8_to_half_cvt<INTERLEAVED, NATURAL>(MODE == W4_SIGNED ? (w ^ 0x88888888u) : w, r);
+  const half2_t s2 = {s, s}, a2 = {addend, addend};
+  const half2_t m8 = {(half_t)-8.f, (half_t)-8.f}, zero2 = {(half_t)0.f, (half_t)0.f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (MODE == W4_SIGNED || MODE == W4_OFFSET8) r[i] = r[i] + m8;  // sext4(q) = (q ^ 8) - 8
+    // the reference multiplies with fma(x, s, +0): a zero product comes out as +0 whatever the sign of s
+    else if constexpr (MODE == W4_USCALE) r[i] = __builtin_elementwise_fma(r[i], s2, zero2);
+    else if constexpr (MODE == W4_ZEROS_ORIGINAL) r[i] = __builtin_elementwise_fma(r[i] + a2, s2, zero2);
+    else if constexpr (MODE != W4_UNSIGNED) r[i] = __builtin_elementwise_fma(r[i], s2, a2);  // SCALE, RESCALE, FOLDED
   }
   half8_t o;
   o[0] = r[0][0]; o[1] = r[0][1]; o[2] = r[1][0]; o[3] = r[1][1];

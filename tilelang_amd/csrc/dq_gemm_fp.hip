@@ -162,24 +162,22 @@ struct W4F16Policy : F16Mfma {
   static constexpr bool kAPacked = false;
   using out_t = half_t;
   struct ScaleRaw { half_t s, z; };
-  using Scale = ScaleRaw;
+  struct Scale { half_t s, addend; };  // what the decoder multiplies by and adds (w4_cvt_addend)
   // direct-to-LDS kernel: with one scale (and zero) per 128 k the fp16 values travel by DMA, a dword per row
   // (two groups = four tiles of 64 k) at a time; other group sizes stay on the register-staged kernel
   static constexpr int kScaleDma = MODE >= W4_ZEROS_ORIGINAL ? 3 : (MODE >= W4_SCALE ? 2 : 0);
   static bool dma_ok(const Params& p) { return kScaleDma == 0 || (p.p0 == 7 && p.K % 256 == 0); }
   __device__ static __forceinline__ Scale ring_scale(const unsigned char* s_at, const unsigned char* z_at) {
-    Scale r{(half_t)1.f, (half_t)0.f};
+    ScaleRaw r{(half_t)1.f, (half_t)0.f};
     r.s = *reinterpret_cast<const half_t*>(s_at);
     if constexpr (kScaleDma == 3) r.z = *reinterpret_cast<const half_t*>(z_at);
-    return r;
+    return Scale{r.s, w4_cvt_addend<MODE>(r.s, r.z)};
   }
   __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return Scale{(half_t)1.f, (half_t)0.f}; }
-  // the plain-layout decoder emits nibble pairs (e, e+4): activations get the same order, on their way to LDS
-  // (register-staged kernel) or fragment by fragment after the LDS read (direct-to-LDS kernel)
-  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : permute_k8_16bit(v); }
-  __device__ static __forceinline__ frag_t fix_a(frag_t f) {
-    return INTERLEAVED ? f : __builtin_bit_cast(frag_t, permute_k8_16bit(__builtin_bit_cast(uint4_t, f)));
-  }
+  // the decoder emits the eight weights of a word in element order for either word layout: the activations go to
+  // LDS and into the matrix instruction untouched
+  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return v; }
+  __device__ static __forceinline__ frag_t fix_a(frag_t f) { return f; }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
   __device__ static __forceinline__ ScaleRaw fetch_scale(const Params& p, int row, int kb, int g) {
     ScaleRaw r{(half_t)1.f, (half_t)0.f};
@@ -188,9 +186,11 @@ struct W4F16Policy : F16Mfma {
     if constexpr (MODE >= W4_ZEROS_ORIGINAL) r.z = ((const half_t*)p.Z)[idx];
     return r;
   }
-  __device__ static __forceinline__ Scale prep_scale(ScaleRaw r, const Params&) { return r; }
+  __device__ static __forceinline__ Scale prep_scale(ScaleRaw r, const Params&) {
+    return Scale{r.s, w4_cvt_addend<MODE>(r.s, r.z)};
+  }
   __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale& s) {
-    return decode_w4<MODE>(w[j], s.s, s.z);
+    return decode_w4_cvt<MODE, INTERLEAVED, true>(w[j], s.s, s.addend);
   }
   __device__ static __forceinline__ out_t finish(uint32_t raw, const Params&, int, int) {
     return (half_t)__builtin_bit_cast(float, raw);
@@ -314,6 +314,7 @@ int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void
     case W4_USCALE: DQ_W4(W4_USCALE);
     case W4_ZEROS_ORIGINAL: DQ_W4(W4_ZEROS_ORIGINAL);
     case W4_ZEROS_RESCALE: DQ_W4(W4_ZEROS_RESCALE);
+    case W4_ZEROS_FOLDED: DQ_W4(W4_ZEROS_FOLDED);
     default: DQ_FAIL("w4 fp16 gemm: unknown mode %d", mode);
   }
 #undef DQ_W4

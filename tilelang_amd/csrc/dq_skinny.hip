@@ -223,7 +223,9 @@ __global__ __launch_bounds__(WAVES * 64) void w4a16_skinny_kernel(const half_t* 
 
 // Materialise the dequantised fp16 tile W[N, K] with the very same decoder the GEMV uses
 // (one thread per 32-bit word).  `plain order` output: element k of row n.
-template <int MODE, bool INTERLEAVED>
+// CVT: the decoder built on the fp8 converter (decode_w4_cvt: the streaming batch kernel and the tiled GEMM use
+// it) instead of the mantissa-mask decoder (decode_w4: every other kernel); the two agree bit for bit.
+template <int MODE, bool INTERLEAVED, bool CVT>
 __global__ void w4_dequant_kernel(const uint8_t* __restrict__ B, const half_t* __restrict__ S,
                                   const half_t* __restrict__ Z, half_t* __restrict__ W, int N, int K, int group) {
   const size_t words_per_row = (size_t)K >> 3;
@@ -237,8 +239,12 @@ __global__ void w4_dequant_kernel(const uint8_t* __restrict__ B, const half_t* _
   half_t s = (half_t)1.f, z = (half_t)0.f;
   if constexpr (ModeTraits<MODE>::kHasScale) s = S[n * groups_per_row + gi];
   if constexpr (ModeTraits<MODE>::kHasZeros) z = Z[n * groups_per_row + gi];
-  const half8_t x = decode_w4<MODE>(w, s, z);
   half_t* dst = W + n * (size_t)K + (size_t)kw * 8;
+  if constexpr (CVT) {  // element order for either word layout
+    *reinterpret_cast<half8_t*>(dst) = decode_w4_cvt<MODE, INTERLEAVED, true>(w, s, w4_cvt_addend<MODE>(s, z));
+    return;
+  }
+  const half8_t x = decode_w4<MODE>(w, s, z);
   if constexpr (INTERLEAVED) {
     *reinterpret_cast<half8_t*>(dst) = x;
   } else {
@@ -338,14 +344,20 @@ int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int 
                hipStream_t stream) {
   const size_t words = (size_t)N * (K >> 3);
   const dim3 block(256), grid((unsigned)((words + 255) / 256));
+  const bool converter = (layout & DECODER_CONVERTER) != 0;
+  const int word_layout = layout & ~DECODER_CONVERTER;
+#define DQ_DQ3(MODE_, IL_, CVT_)                                                                                   \
+  hipLaunchKernelGGL((w4_dequant_kernel<MODE_, IL_, CVT_>), grid, block, 0, stream, (const uint8_t*)B,           \
+                     (const half_t*)S, (const half_t*)Z, (half_t*)W, N, K, group)
 #define DQ_DQ(MODE_)                                                                                               \
   do {                                                                                                             \
-    if (layout == LAYOUT_PLAIN)                                                                                    \
-      hipLaunchKernelGGL((w4_dequant_kernel<MODE_, false>), grid, block, 0, stream, (const uint8_t*)B,            \
-                         (const half_t*)S, (const half_t*)Z, (half_t*)W, N, K, group);                             \
-    else                                                                                                           \
-      hipLaunchKernelGGL((w4_dequant_kernel<MODE_, true>), grid, block, 0, stream, (const uint8_t*)B,             \
-                         (const half_t*)S, (const half_t*)Z, (half_t*)W, N, K, group);                             \
+    if (word_layout == LAYOUT_PLAIN) {                                                                             \
+      if (converter) DQ_DQ3(MODE_, false, true);                                                                   \
+      else DQ_DQ3(MODE_, false, false);                                                                            \
+    } else {                                                                                                       \
+      if (converter) DQ_DQ3(MODE_, true, true);                                                                    \
+      else DQ_DQ3(MODE_, true, false);                                                                             \
+    }                                                                                                              \
   } while (0)
   switch (mode) {
     case W4_UNSIGNED: DQ_DQ(W4_UNSIGNED); break;
@@ -355,9 +367,11 @@ int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int 
     case W4_USCALE: DQ_DQ(W4_USCALE); break;
     case W4_ZEROS_ORIGINAL: DQ_DQ(W4_ZEROS_ORIGINAL); break;
     case W4_ZEROS_RESCALE: DQ_DQ(W4_ZEROS_RESCALE); break;
+    case W4_ZEROS_FOLDED: DQ_DQ(W4_ZEROS_FOLDED); break;
     default: DQ_FAIL("w4 dequant: unknown mode %d", mode);
   }
 #undef DQ_DQ
+#undef DQ_DQ3
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
 }

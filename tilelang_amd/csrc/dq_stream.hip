@@ -180,8 +180,6 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   // The pipeline runs across steps: the last two slots of a step read from the NEXT stage, so the
   // workgroup barrier that publishes that stage (and releases the current one for the DMA engine)
   // sits in front of them.
-  constexpr bool kPermW = APERM && RBW < MB;   // bring the decoded weights to natural k order
-  constexpr bool kPermA = APERM && !kPermW;    // or the activations to the decoder's order
   uint4_t w_c[kU][RBW], w_n[kU][RBW], yraw[2][MB];
   half_t sc_c[kU][RBW], zp_c[kU][RBW], sc_n[kU][RBW], zp_n[kU][RBW];
   half8_t x_m[RBW], y_m[MB], x_d[RBW], y_d[MB];
@@ -193,22 +191,13 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
       for (int rb = 0; rb < RBW; ++rb) {
         w_n[ui][rb] = *reinterpret_cast<const uint4_t*>(sb + w_off[rb][ui]);
         sc_n[ui][rb] = kScale ? *reinterpret_cast<const half_t*>(sc_nxt + sc_off[rb][ui]) : (half_t)1.f;
-        zp_n[ui][rb] = kZeros ? *reinterpret_cast<const half_t*>(sc_nxt + sc_off[rb][ui] + 2048) : (half_t)0.f;
+        const half_t z = kZeros ? *reinterpret_cast<const half_t*>(sc_nxt + sc_off[rb][ui] + 2048) : (half_t)0.f;
+        zp_n[ui][rb] = w4_cvt_addend<MODE>(sc_n[ui][rb], z);  // what the decoder adds: -8 s, -z or -(z s)
       }
   };
-  auto decode = [&](uint32_t w, half_t sc, half_t zp) -> half8_t {
-    const half8_t x = decode_w4<MODE>(w, sc, zp);
-    if constexpr (kPermW) {
-      const uint4_t d = __builtin_bit_cast(uint4_t, x);  // (n0,n4) (n1,n5) (n2,n6) (n3,n7)
-      uint4_t o;
-      o[0] = __builtin_amdgcn_perm(d[1], d[0], 0x05040100u);
-      o[1] = __builtin_amdgcn_perm(d[3], d[2], 0x05040100u);
-      o[2] = __builtin_amdgcn_perm(d[1], d[0], 0x07060302u);
-      o[3] = __builtin_amdgcn_perm(d[3], d[2], 0x07060302u);
-      return __builtin_bit_cast(half8_t, o);
-    } else {
-      return x;
-    }
+  // element order 0..7 for either word layout: the activations are used as they come out of LDS
+  auto decode = [&](uint32_t w, half_t sc, half_t addend) -> half8_t {
+    return decode_w4_cvt<MODE, !APERM, true>(w, sc, addend);
   };
   // slots s_begin .. s_end-1 of a step whose stage is sb_cur; kCur: the step exists (false only
   // while the pipeline fills before step 0), kNext: so does the next one, staged at sb_nxt
@@ -233,7 +222,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
       if (s1 < kSub ? kCur : kNext) {  // D(t+1)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          y_d[mb] = __builtin_bit_cast(half8_t, kPermA ? permute_k8_16bit(yraw[s1 & 1][mb]) : yraw[s1 & 1][mb]);
+          y_d[mb] = __builtin_bit_cast(half8_t, yraw[s1 & 1][mb]);
 #pragma unroll
         for (int rb = 0; rb < RBW; ++rb) {
           if (s1 < kSub) x_d[rb] = decode(w_c[(s1 >> 2) % kU][rb][s1 & 3], sc_c[(s1 >> 2) % kU][rb], zp_c[(s1 >> 2) % kU][rb]);
@@ -371,6 +360,7 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
     case W4_USCALE: DQ_LAUNCH_MODE(W4_USCALE); break;
     case W4_ZEROS_ORIGINAL: DQ_LAUNCH_MODE(W4_ZEROS_ORIGINAL); break;
     case W4_ZEROS_RESCALE: DQ_LAUNCH_MODE(W4_ZEROS_RESCALE); break;
+    case W4_ZEROS_FOLDED: DQ_LAUNCH_MODE(W4_ZEROS_FOLDED); break;
     default: DQ_FAIL("w4a16: unknown mode %d", mode);
   }
 #undef DQ_LAUNCH_MODE

@@ -16,8 +16,9 @@ from . import _lib
 from .adapter import KernelAdapter, KernelParam
 
 # ---- enums of include/dqgemm.h -------------------------------------------------------------
-W4_UNSIGNED, W4_SIGNED, W4_OFFSET8, W4_SCALE, W4_USCALE, W4_ZEROS_ORIGINAL, W4_ZEROS_RESCALE = range(7)
+W4_UNSIGNED, W4_SIGNED, W4_OFFSET8, W4_SCALE, W4_USCALE, W4_ZEROS_ORIGINAL, W4_ZEROS_RESCALE, W4_ZEROS_FOLDED = range(8)
 LAYOUT_PLAIN, LAYOUT_INTERLEAVED, LAYOUT_FRAGMENTS = 0, 1, 2
+DECODER_CONVERTER = 4  # flag of call_dequantize_w4's layout: dump the tile with the fp8-converter decoder
 I4_UNSIGNED, I4_TWOS, I4U_INTERLEAVED, I4S_INTERLEAVED = range(4)
 
 _DTYPES = {
@@ -48,6 +49,10 @@ def _w4_mode(source_format: str, fast_decoding: bool, with_scaling: bool, with_z
             return W4_ZEROS_ORIGINAL
         if zeros_mode == "rescale":
             return W4_ZEROS_RESCALE
+        if zeros_mode == "folded":
+            # (q - z) * s as one fused multiply-add per weight, fma(q, s, -rne16(z * s)): this library's own, cheaper
+            # form of "original" (no counterpart in the reference); inside rtol = atol = 1e-2 of it
+            return W4_ZEROS_FOLDED
         raise ValueError(f"unknown zeros_mode {zeros_mode!r}")
     if with_scaling:
         return W4_SCALE if source_format == "int" else W4_USCALE
@@ -291,18 +296,23 @@ def dequantize_w4(
     storage_dtype="int8",
     _formula_fast: bool | None = None,
     qzeros_format: str = "int16",
+    decoder: str = "mask",
 ) -> KernelAdapter:
     """Dequantised weight tile ``W[N,K] fp16 = decode(B[N,K/2][, Scale[, Zeros]])``.
 
     The decode-only kernel the examples use to test a converter
     (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:36-65), here for the 4-bit
-    integer decoders.  ``W = kernel(B[, Scale[, Zeros]])``.
+    integer decoders.  ``W = kernel(B[, Scale[, Zeros]])``.  ``decoder``: which of the library's two device decoders
+    writes the tile, ``"mask"`` (nibbles OR-ed into an fp16 mantissa) or ``"converter"`` (nibbles read as fp8 by the
+    hardware converter); they agree bit for bit.
     """
+    if decoder not in ("mask", "converter"):
+        raise ValueError(f"dequantize_w4: unknown decoder {decoder!r}")
     if group_size == -1:
         group_size = K
     formula_fast = fast_decoding if _formula_fast is None else _formula_fast
     mode = _w4_mode(source_format, formula_fast, with_scaling, with_zeros, zeros_mode)
-    layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
+    layout = (LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN) | (DECODER_CONVERTER if decoder == "converter" else 0)
     groups = K // group_size
     params = [KernelParam("B", _dtype(storage_dtype), (N, K // 2), packed=True)]
     if with_scaling:
