@@ -187,7 +187,8 @@ def bench_mxfp4(torch, tl, workloads, M, N, K, steps, warmup, dev, **tk):
         return f
 
     ms, graphed = _time_launches(torch, [mk(i) for i in range(nc)], steps, warmup, **tk)
-    return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "timing": graphed}
+    return {"us": ms * 1e3, "bytes": workloads.mxfp4_bytes(M, N, K), "flops": workloads.flops(M, N, K), "timing": graphed,
+            "inputs": d, "out": out[0]}
 
 
 def bench_mxfp4_blockscaled(torch, tl, workloads, M, N, K, steps, warmup, dev, **tk):
@@ -390,6 +391,33 @@ def cpu_baselines(budget_s=16.0):
     return cpu
 
 
+def check_timed_outputs(head, mx):
+    """What the timed launches left in their output buffers against the torch-CPU ``ref_program`` (rtol = atol = 1e-2,
+    the tolerance the reference's own checks use), after the timing and outside it: every output of the headline
+    GEMV; for the MXFP4 GEMM the columns of 64 weight rows spread over N.  Returns ``(gemv, gemm)`` dictionaries
+    ``{"checked": bool, "max_abs_err": float, "compared": int}``."""
+    import torch
+
+    from oracle import ref_torch
+
+    def verdict(got, ref):
+        got, ref = got.float(), ref.float()
+        ok = bool(torch.isfinite(got).all()) and bool(torch.allclose(got, ref, rtol=1e-2, atol=1e-2))
+        return {"checked": ok, "max_abs_err": float((got - ref).abs().max()), "compared": got.numel()}
+
+    d = {k: torch.from_numpy(v) for k, v in head["inputs"].items()}
+    gemv = verdict(head["out"].cpu(), ref_torch.ref_w4a16(d["A"], d["B"], d["Scale"], d.get("Zeros")))
+    gemm = None
+    if mx is not None:
+        d = mx["inputs"]
+        n_rows = d["B"].shape[0]
+        rows = torch.arange(0, n_rows, max(1, n_rows // 64))[:64]
+        ref = ref_torch.ref_mxfp4_e2m1(torch.from_numpy(d["A"]).view(torch.bfloat16), torch.from_numpy(d["B"])[rows],
+                                       torch.from_numpy(d["Scale"])[rows], 127)
+        gemm = verdict(mx["out"].cpu()[:, rows], ref)
+    return gemv, gemm
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -436,6 +464,7 @@ def main():
         del src, dst
 
     shapes = []
+    mx_run = None
     if not args.headline_only:
         gemm = {"min_launches": 24, "max_launches": 48}  # launches of hundreds of microseconds: a replay is milliseconds
         for (m, n, kk) in [(1, 1024, 1024), (1, 11008, 4096), (1, 4096, 11008), (1, 4096, 4096)]:
@@ -453,6 +482,7 @@ def main():
         r = bench_w2a16(torch, tl, 1, 28672, 8192, S, W, dev)
         shapes.append(_row("w2a16_gemv M=1 N=28672 K=8192 (num_bits=2, interleaved words, (c-2)*s)", r, "hbm", MFMA_BF16_PEAK))
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
+        mx_run = r
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
         for m in (1, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m == 1 else gemm))
@@ -491,6 +521,13 @@ def main():
                          "algorithmic_flops": 2 * 4096 * 8192 * 8192}
     cpu = None
     if not args.no_cpu:
+        # the CPU leg also looks at what was timed: a kernel that regressed to wrong results must not print a figure
+        gemv_check, gemm_check = check_timed_outputs(head, mx_run)
+        roof.update(gemv_check)
+        if roof_gemm is not None and gemm_check is not None:
+            roof_gemm.update(gemm_check)
+        if not gemv_check["checked"] or (gemm_check is not None and not gemm_check["checked"]):
+            sys.exit(f"bench.py: the timed kernels' outputs do not match the CPU ref_program: gemv {gemv_check}, gemm {gemm_check}")
         cpu = cpu_baselines()
 
     line = {

@@ -96,9 +96,14 @@ int call_dequantize_w4(const void* B, const void* Scale, const void* Zeros, void
 
 enum dq_qzeros_format {
   DQ_QZEROS_INT16 = 0,  /* QZeros[N, groups] int16, one zero point per group: what decode_i4u_to_f16_scale_zeros_quantized
-                           reads (`int16_t zero_r`, examples/dequantize_gemm/quantize/lop3.py:339-341)                    */
-  DQ_QZEROS_PACKED4 = 1 /* QZeros[N, ceil(groups / 2)] bytes, 4-bit zero points, group g in bits 4 (g % 2) of byte g / 2:
-                           the `(qzeros >> (group_offset * 4)) & 0xf` of the _offset variant, lop3.py:381-385             */
+                           reads (`int16_t zero_r`, examples/dequantize_gemm/quantize/lop3.py:339-341).  The reference
+                           folds it as `0xe400 | zero_r`, which means -(1024 + qz) for 0 <= qz <= 1023 only: that is the
+                           range with reference parity.  Values outside it are taken as the integers they are (the
+                           reference gives them no meaning).                                                            */
+  DQ_QZEROS_PACKED4 = 1 /* QZeros[N, ceil(groups / 2)] bytes, 4-bit zero points, group g in bits 4 (g % 2) of byte g / 2.
+                           The tensor shape and the order of the groups inside a row are THIS LIBRARY'S convention: the
+                           reference shows only the device-side extraction `(qzeros >> (group_offset * 4)) & 0xf` from
+                           two storage words (the _offset variant, lop3.py:367-390) and defines no host-side tensor.    */
 };
 
 /* Zeros[N, groups] fp16 = the integer zero points of the "quantized" zeros mode.  The reference's decoder computes

@@ -83,3 +83,23 @@ def test_bitlinear_layer_with_fragment_ordered_copy(cuda):
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     assert not tl.BitLinear(1024, 768, prefill_fragments=True).prefill_fragments  # in_features the kernel cannot slice
 
+
+
+def test_bitlinear_decode_batches_stay_on_the_streaming_kernel(cuda):
+    """An 8192 x 8192 layer has 64 output tiles already at one row: a layer with the fragment-ordered copy must still
+    hand decode batches (M <= 4) the row-major words, which the streaming decode kernel reads, and give the plain
+    layer's bits."""
+    in_f = out_f = 8192
+    rng = np.random.default_rng(13)
+    W = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
+    plain = tl.BitLinear(in_f, out_f)
+    frag = tl.BitLinear(in_f, out_f, prefill_fragments=True)
+    for layer in (plain, frag):
+        layer.load_float_weight(torch.from_numpy(W))
+        layer.to(cuda)
+    assert not frag._takes_fragments(1) and not frag._takes_fragments(4) and frag._takes_fragments(5)
+    for M in (1, 4):
+        x = torch.from_numpy(rng.standard_normal((M, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
+        a, b = plain(x), frag(x)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))

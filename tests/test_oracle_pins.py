@@ -206,6 +206,14 @@ def test_w4_decoders_rounding_order_step_by_step():
             assert got.tolist() == [_rne16(Fraction(_rne16(q - fz)) * fs) for q in range(16)]
             got = orc.dequant_u4_scale_zeros(packed, S, Z, 16, "rescale")[0]
             assert got.tolist() == [_rne16(q * fs - fz) for q in range(16)]
+            # the library's folded form: z * s rounded to fp16 first, then one fused multiply-add per weight
+            got = orc.dequant_u4_scale_zeros(packed, S, Z, 16, "folded")[0]
+            fzs = Fraction(_rne16(fz * fs))
+            assert got.tolist() == [_rne16(q * fs - fzs) for q in range(16)]
+            # ... which stays within one fp16 step of z * s of the reference's "original" form
+            orig = orc.dequant_u4_scale_zeros(packed, S, Z, 16, "original")[0].astype(np.float64)
+            step = max(np.spacing(np.float16(abs(float(fz * fs)))), np.spacing(np.float16(15 * float(fs)))).astype(np.float64)
+            assert np.abs(got.astype(np.float64) - orig).max() <= 2 * step
         for qz in qz_int:
             got = orc.dequant_u4_scale_zeros(packed, S, np.array([[qz]]), 16, "quantized")[0]
             want = [_rne16((q - qz) * fs) for q in range(16)]
@@ -352,6 +360,13 @@ def test_ref_int_paths_brute_force():
     a4 = orc.decode_i4_signed(Ap).astype(np.int64)
     np.testing.assert_array_equal(orc.ref_int4xint4(Ap, B4), a4 @ w4.T)
     assert orc.ref_w4a8(A, B4).dtype == np.int32 and orc.ref_w4a8(A, B4).shape == (N, M)
+    # the fine-grained example's int8 path (unsigned nibbles) and the unscaled fp16 tiles, nibble by nibble
+    u4 = np.array([[(int(B4[n, k // 2]) >> (4 * (k % 2))) & 15 for k in range(K)] for n in range(N)], dtype=np.int64)
+    np.testing.assert_array_equal(orc.ref_u4_int8(A, B4), a @ u4.T)
+    assert orc.ref_u4_int8(A, B4).dtype == np.int32
+    np.testing.assert_array_equal(orc.dequant_u4_plain(B4, signed=False).astype(np.int64), u4)
+    np.testing.assert_array_equal(orc.dequant_u4_plain(B4, signed=True).astype(np.int64), w4)
+    assert orc.dequant_u4_plain(B4).dtype == np.float16
 
 
 def test_ref_mxfp4_exact_scaling_and_identity():

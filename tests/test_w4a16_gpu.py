@@ -389,6 +389,40 @@ def test_full_size_linearity(cuda):
 
 
 @pytest.fixture(scope="module")
+def headline_full_size():
+    """The configuration the metric is quoted on at its full size: N = 28672, K = 8192, w = (q - 8) * s, with the
+    oracle's tile over ALL weight rows."""
+    M, N, K, group = 4, 28672, 8192, 128
+    d = workloads.w4a16(M, N, K, group, seed=9, scale_range=(0.005, 0.02))
+    W = orc.dequant_u4_scale(d["B"], d["Scale"], group).astype(np.float32)
+    return d, W
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_headline_full_size_every_output(cuda, headline_full_size, M, interleaved):
+    """The headline decode GEMV (M = 1, N = 28672, K = 8192, (q - 8) * s) and its M = 2, 3, 4 siblings of the same
+    kernel family, through the library's own dispatch: EVERY one of the M x 28672 outputs against the oracle, for the
+    plain and the interleaved word layout."""
+    d, W = headline_full_size
+    N, K, group = 28672, 8192, 128
+    print(f"headline full size: M={M} interleaved={interleaved}", flush=True)
+    kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, source_format="int",
+                              with_scaling=True, fast_decoding=interleaved)
+    Bd = _dev(d["B"], cuda).view(torch.int8)
+    if interleaved:
+        Bd = tl.quantize.interleave_weight(Bd, 4, "float16")
+    A = d["A"][:M]
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(_dev(A, cuda), Bd, _dev(d["Scale"], cuda), C)
+    torch.cuda.synchronize()
+    got = C.float().cpu().numpy()
+    ref = (A.astype(np.float32) @ W.T).astype(np.float16).astype(np.float32)
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.fixture(scope="module")
 def cfg3_full_size():
     """Configuration 3 at its full size, N = 28672, K = 8192, with the oracle's tile over ALL weight rows."""
     M, N, K, group = 64, 28672, 8192, 128

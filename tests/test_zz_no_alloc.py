@@ -33,11 +33,14 @@ def _both(lib, cuda, M, N, K, split, transposed, seed):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = lib.call_dequant_gemm_fp16_fp4_splitk(_ptr(A), _ptr(B), _ptr(parts), _ptr(want), M, N, K, split, int(transposed), stream)
     assert rc == 0, lib.get_last_error().decode()
-    before = torch.cuda.memory_allocated()
+    # device-wide free memory, not torch's own counter: a hipMalloc inside the library would show here
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     rc = lib.call_dequant_gemm_fp16_fp4_splitk_static(_ptr(A), _ptr(B), _ptr(got), M, N, K, split, int(transposed), stream)
     assert rc == 0, lib.get_last_error().decode()
-    assert torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     assert torch.isfinite(got).all()
     assert torch.equal(got, want)
 
@@ -62,6 +65,43 @@ def test_static_scratch_matches_caller_buffer_twice(cuda):
     # transposed output, ragged tiles, then again a smaller one
     _both(lib, cuda, 300, 520, 768, 3, True, seed=14)
     _both(lib, cuda, 100, 72, 512, 2, True, seed=15)
+
+
+def test_static_scratch_under_graph_capture(cuda):
+    """The callers the entry point is for: captured into a graph after one eager call (an allocation during capture
+    would raise), replayed several times with eager work and synchronisations in between, every replay bit-identical
+    to the eager result."""
+    lib = _lib.get_library()
+    M, N, K, split = 256, 384, 1024, 4
+    rng = np.random.default_rng(21)
+    A = torch.from_numpy((rng.standard_normal((M, K), dtype=np.float32) * 0.5).astype(np.float16)).to(cuda)
+    B = torch.from_numpy(rng.integers(0, 256, size=(N, K // 2), dtype=np.uint8)).to(cuda)
+    eager = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.call_dequant_gemm_fp16_fp4_splitk_static(_ptr(A), _ptr(B), _ptr(eager), M, N, K, split, 0, stream)
+    assert rc == 0, lib.get_last_error().decode()
+    torch.cuda.synchronize()
+    print("no-alloc split-K: graph capture", flush=True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.call_dequant_gemm_fp16_fp4_splitk_static(_ptr(A), _ptr(B), _ptr(out), M, N, K, split, 0,
+                                                              ctypes.c_void_p(side.cuda_stream))
+    assert rc == 0, lib.get_last_error().decode()
+    torch.cuda.synchronize()
+    for i in range(3):
+        out.fill_(float("nan"))
+        # eager work between the replays, on the same scratch buffer, with another shape
+        small = torch.empty((64, 128), dtype=torch.float16, device=cuda)
+        rc = lib.call_dequant_gemm_fp16_fp4_splitk_static(_ptr(A), _ptr(B), _ptr(small), 64, 128, 512, 2, 0, stream)
+        assert rc == 0, lib.get_last_error().decode()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i} differs from the eager result"
 
 
 def test_static_scratch_rejects_what_does_not_fit(cuda):

@@ -19,7 +19,7 @@ CSRC_DIR = os.path.join(_PKG_DIR, "csrc")
 
 _lock = threading.Lock()
 _lib = None
-_initialised = False
+_initialised_devices: set = set()
 
 _vp, _i = ctypes.c_void_p, ctypes.c_int
 
@@ -80,16 +80,28 @@ def load_library() -> ctypes.CDLL:
     return _lib
 
 
-def get_library() -> ctypes.CDLL:
-    """Library ready for kernel calls: loaded and ``init()`` run once on the current device."""
-    global _initialised
+def get_library(device_index: int | None = None) -> ctypes.CDLL:
+    """Library ready for kernel calls on the CURRENT device: loaded, and ``init()`` (architecture check, LDS limit,
+    the device's copy of the static scratch buffer) run once per device.  ``device_index`` names the current device
+    when the caller knows it; ``None`` asks torch (and falls back to one ``init()`` per process when torch sees no
+    GPU runtime, in which case ``init()`` itself reports the error).
+
+    Calls through ``call_dequant_gemm_fp16_fp4_splitk_static`` share one scratch buffer per GPU: two of them that
+    overlap in time on one GPU (different streams, or two captured graphs replayed concurrently) race on it."""
     lib = load_library()
-    if not _initialised:
+    if device_index is None:
+        try:
+            import torch
+
+            device_index = torch.cuda.current_device() if torch.cuda.is_available() else -1
+        except ImportError:
+            device_index = -1
+    if device_index not in _initialised_devices:
         with _lock:
-            if not _initialised:
+            if device_index not in _initialised_devices:
                 if lib.init() != 0:
                     raise RuntimeError(f"libdqgemm init failed: {lib.get_last_error().decode()}")
-                _initialised = True
+                _initialised_devices.add(device_index)
     return lib
 
 

@@ -16,6 +16,7 @@ Mirrors the call contract of the reference's adapter for JIT kernels
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from dataclasses import dataclass
 from typing import Callable, Sequence
@@ -59,7 +60,8 @@ class KernelAdapter:
         self.result_idx = [i if i >= 0 else n + i for i in result_idx]
         # parameters the kernel uses as scratch (the reference's T.alloc_buffer globals): allocated here for every
         # call, passed to the library, never returned.  torch's caching allocator hands a freed block back to the
-        # stream it was used on only, so calls on different streams never share a scratch buffer.
+        # stream it was allocated under only (__call__ allocates under the stream it launches on), so calls on
+        # different streams never share a scratch buffer.
         self.workspace_idx = [i if i >= 0 else n + i for i in workspace_idx]
         self._launch = launch
         self._get_last_error = get_last_error
@@ -112,27 +114,39 @@ class KernelAdapter:
             raise ValueError(
                 f"Expected {n_params} inputs, got {n_in + n_out} with {n_in} inputs and {n_out} outputs"
             )
-        if stream == -1:
-            stream = current_stream_handle(self.device_type)
-
         device = None
         for t in inputs:
             if isinstance(t, torch.Tensor):
                 device = t.device
                 break
-        tensors, it = [], iter(inputs)
-        for i, p in enumerate(self.params):
-            if i in self.workspace_idx:
-                if device is None:
-                    device = torch.device(self.device_type)
-                tensors.append(torch.empty(*p.shape, dtype=p.dtype, device=device))
-            elif i in self.result_idx:
-                if device is None:
-                    device = torch.device(self.device_type)
-                tensors.append(torch.empty(*p.shape, dtype=p.dtype, device=device))
-            else:
-                tensors.append(next(it))
+        if device is None:
+            device = torch.device(self.device_type)
+        on_gpu = device.type == "cuda" and torch.cuda.is_available()
+        # the library launches on the CURRENT device: make the operands' device current for the length of the call
+        guard = contextlib.nullcontext()
+        if on_gpu and device.index is not None and device.index != torch.cuda.current_device():
+            guard = torch.cuda.device(device)
+        with guard:
+            current = current_stream_handle(self.device_type)
+            if stream == -1:
+                stream = current
+            # Outputs and scratch come from torch's caching allocator, which hands a freed block back to work on
+            # the stream it was allocated under only.  With an explicit stream= that is not torch's current one,
+            # allocate under that stream, so that a block freed while this launch still runs cannot go to an op on
+            # another stream.
+            alloc_ctx = contextlib.nullcontext()
+            if on_gpu and stream != current and (self.result_idx or self.workspace_idx):
+                alloc_ctx = torch.cuda.stream(torch.cuda.ExternalStream(stream, device=device))
+            tensors, it = [], iter(inputs)
+            with alloc_ctx:
+                for i, p in enumerate(self.params):
+                    if i in self.workspace_idx or i in self.result_idx:
+                        tensors.append(torch.empty(*p.shape, dtype=p.dtype, device=device))
+                    else:
+                        tensors.append(next(it))
+            return self._run(tensors, stream, skip_tensor_validation, n_out)
 
+    def _run(self, tensors, stream, skip_tensor_validation, n_out):
         ptrs = []
         for t in tensors:
             if isinstance(t, torch.Tensor):

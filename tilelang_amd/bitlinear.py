@@ -84,7 +84,11 @@ class BitLinear(nn.Module):
         self._kernels.clear()
 
     def _takes_fragments(self, M: int) -> bool:
-        # the shapes the library gives to the kernel that slices K over the waves (tiles of 64 x 128)
+        # the shapes the library gives to the kernel that slices K over the waves (tiles of 64 x 128), in the order
+        # call_gemm_int8xint2 decides: up to four rows go to the streaming decode kernel first, which reads the
+        # row-major words only
+        if M <= 4:
+            return False
         tiles = ((M + 63) // 64) * ((self.out_features + 127) // 128)
         return self.prefill_fragments and 64 <= tiles <= 448
 

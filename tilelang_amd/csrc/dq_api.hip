@@ -73,10 +73,19 @@ constexpr size_t kStaticScratchBytes = DQ_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 static void* g_scratch_ptr[kMaxDevices];
 
-static int scratch_of_current_device(const char* fn, void** out) {
+// `stream`: when not the null stream, it must belong to the current device (the scratch buffer handed out is the
+// current device's copy, the kernels run where the stream lives).
+static int scratch_of_current_device(const char* fn, hipStream_t stream, void** out) {
   int device = -1;
   DQ_CHECK_HIP(hipGetDevice(&device));
   if (device < 0 || device >= kMaxDevices) DQ_FAIL("%s: device index %d is beyond the %d this library tracks", fn, device, kMaxDevices);
+  if (stream) {
+    hipDevice_t stream_device = -1;
+    DQ_CHECK_HIP(hipStreamGetDevice(stream, &stream_device));
+    if ((int)stream_device != device)
+      DQ_FAIL("%s: the stream belongs to device %d but device %d is current; make the stream's device current first", fn,
+              (int)stream_device, device);
+  }
   if (!g_scratch_ptr[device]) {
     void* ptr = nullptr;
     DQ_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
@@ -122,7 +131,7 @@ extern "C" int init(void) {
   if (largest_lds_request() > max_lds)
     DQ_FAIL("Requested dynamic shared memory %d exceeds device limit %d", largest_lds_request(), max_lds);
   void* scratch_ptr = nullptr;
-  if (scratch_of_current_device("init", &scratch_ptr)) return -1;
+  if (scratch_of_current_device("init", nullptr, &scratch_ptr)) return -1;
   return 0;
 }
 
@@ -332,7 +341,7 @@ extern "C" int call_dequant_gemm_fp16_fp4_splitk_static(const void* A, const voi
     DQ_FAIL("%s: split * M * N fp16 partial results need %zu bytes, the static scratch buffer holds %zu; use "
             "call_dequant_gemm_fp16_fp4_splitk with a buffer of your own", fn, need, kStaticScratchBytes);
   void* parts = nullptr;
-  if (scratch_of_current_device(fn, &parts)) return -1;
+  if (scratch_of_current_device(fn, (hipStream_t)stream, &parts)) return -1;
   // every partial result the summing kernel reads is written by its slice's workgroups first, in stream order:
   // nothing has to start at zero, whatever the last call left behind
   return fp16_fp4_gemm_splitk(A, B, parts, C, M, N, K, split, transposed, (hipStream_t)stream);

@@ -221,9 +221,12 @@ namespace {
 // decoder folds the integer into the magic number, (0x6400 | q) + (0xe400 | qz) = q - qz exactly, then multiplies by
 // the scale once (examples/dequantize_gemm/quantize/lop3.py:339-354); fp16(qz) is exact for 0 <= qz <= 2048 and so
 // is q - fp16(qz), hence the "original" decoder fed with these zeros returns the same bits.
-// PACKED = false: one int16 per group (lop3.py:339-341 reads `int16_t zero_r = *((int16_t*)zeros)`).
-// PACKED = true: 4-bit zero points, two per byte, group g in bits 4 (g % 2) of byte g / 2 of the row
-// (lop3.py:381-385: `(qzeros >> (group_offset * 4)) & 0xf`).
+// PACKED = false: one int16 per group (lop3.py:339-341 reads `int16_t zero_r = *((int16_t*)zeros)` and folds it as
+// `0xe400 | zero_r`, which is -(1024 + qz) for 0 <= qz <= 1023 only: the range with reference parity; other values
+// are taken here as the integers they are).
+// PACKED = true: 4-bit zero points, two per byte, group g in bits 4 (g % 2) of byte g / 2 of the row.  This row
+// layout is the library's own convention: the reference shows only the extraction `(qzeros >> (group_offset * 4))
+// & 0xf` inside its device snippet (lop3.py:381-385) and no host-side tensor shape.
 template <bool PACKED>
 __global__ __launch_bounds__(256) void unpack_qzeros_kernel(const void* __restrict__ QZ, half_t* __restrict__ Z, int N,
                                                             int groups) {

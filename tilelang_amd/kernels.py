@@ -72,8 +72,11 @@ def _zeros_params(N: int, groups: int, zeros_mode: str, qzeros_format: str):
     ``"original"`` / ``"rescale"``: fp16 ``Zeros[N, groups]``.  ``"quantized"``
     (examples/dequantize_gemm/quantize/lop3.py:326-420): integer zero points, ``qzeros_format="int16"`` for
     ``Zeros[N, groups]`` int16 (the ``int16_t zero_r`` of :339-341) or ``"packed4"`` for 4-bit zero points two per
-    byte, ``Zeros[N, ceil(groups / 2)]`` (:381-385); they are unpacked to fp16 into a workspace in front of the
-    kernel, which then runs its ``(q - z) * s`` decoder: the same bits, since ``q - qz`` is exact either way.
+    byte, ``Zeros[N, ceil(groups / 2)]`` (the extraction of :381-385; the tensor shape and the order of the groups
+    inside a row are this library's convention, the reference defines no host-side tensor for them); they are
+    unpacked to fp16 into a workspace in front of the kernel, which then runs its ``(q - z) * s`` decoder: the same
+    bits, since ``q - qz`` is exact either way.  Reference parity of the int16 form holds for 0 <= qz <= 1023 (what
+    ``0xe400 | zero_r`` can express); other values are taken as the integers they are.
     """
     if zeros_mode != "quantized":
         return KernelParam("Zeros", torch.float16, (N, groups)), None, None

@@ -82,42 +82,146 @@ def torch_assert_close(a, b, rtol=1e-2, atol=1e-2, max_mismatched_ratio=0.0, bas
     return True
 
 
+def _summarise(times_ms: "torch.Tensor", quantiles, return_mode: str):
+    """One number (mean / median / min / max) or the requested quantiles of the per-call times."""
+    if quantiles is not None:
+        q = torch.quantile(times_ms, torch.tensor(list(quantiles), dtype=torch.float)).tolist()
+        return q[0] if len(q) == 1 else q
+    return getattr(torch, return_mode)(times_ms).item()
+
+
+def _time_with_events(fn, flush, n_repeat):
+    """One event pair around every call, the cache flushed in front of each."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_repeat)]
+    for begin, finish in pairs:
+        flush()
+        begin.record()
+        fn()
+        finish.record()
+    torch.cuda.synchronize()
+    return torch.tensor([b.elapsed_time(f) for b, f in pairs], dtype=torch.float)
+
+
+def _time_with_graph(fn, flush, n_repeat, replays: int = 10):
+    """``n_repeat`` calls captured back to back into one graph on a side stream (default priority), the graph
+    replayed ``replays`` times with the cache flushed in front of every replay: per-call time without the host's
+    launch cost.  The flush cannot be part of the graph, so calls after the first of a replay may hit the cache."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(n_repeat):
+                fn()
+        torch.cuda.synchronize()
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(replays)]
+        for begin, finish in pairs:
+            flush()
+            begin.record()
+            graph.replay()
+            finish.record()
+        torch.cuda.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    return torch.tensor([b.elapsed_time(f) / n_repeat for b, f in pairs], dtype=torch.float)
+
+
+_FLUSH_RANGE = "tilelang_amd::cache_flush"
+
+
+def _time_with_trace(fn, flush, n_repeat):
+    """Device time of the kernels themselves from torch's kernel trace (the reference's ``backend="cupti"``; on
+    ROCm the trace comes from the runtime's tracer): everything the GPU ran during the measured step minus what ran
+    inside the annotated flush range, divided by the number of calls.  One number: the trace has no per-call split."""
+    import warnings
+
+    from torch.profiler import ProfilerActivity, profile, record_function, schedule
+
+    with warnings.catch_warnings(), profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA], schedule=schedule(wait=1, warmup=0, active=1, repeat=1)) as prof:
+        warnings.simplefilter("ignore", UserWarning)  # "won't be using warmup", "clears events at the end of each cycle"
+        for _ in range(2):  # the first step is the schedule's wait step
+            for _ in range(n_repeat):
+                with record_function(_FLUSH_RANGE):
+                    flush()
+                fn()
+            torch.cuda.synchronize()
+            prof.step()
+    kernels_us = flush_us = 0.0
+    for ev in prof.events():
+        if getattr(getattr(ev, "device_type", None), "name", "") != "CUDA":
+            continue
+        if ev.is_user_annotation:
+            if ev.key == _FLUSH_RANGE:
+                flush_us += ev.self_device_time_total
+        else:
+            kernels_us += ev.self_device_time_total
+    return torch.tensor([(kernels_us - flush_us) / n_repeat * 1e-3], dtype=torch.float)
+
+
 def do_bench(
     fn: Callable,
     warmup: float = 25,
     rep: float = 100,
     _n_warmup: int = 0,
     _n_repeat: int = 0,
+    quantiles=None,
+    fast_flush: bool = True,
+    backend: str = "event",
     return_mode: str = "mean",
+    device=None,
     cache_size: int = 256,
-) -> float:
-    """Mean (or min/max/median) milliseconds per call, event-timed, L2 flushed before each call."""
+    early_stop_baseline: float | None = None,
+):
+    """Milliseconds per call of ``fn`` with the last-level cache flushed between calls.  Twin of ``do_bench`` of
+    tilelang/profiler/bench.py:68-272 (same arguments and result conventions).
+
+    ``warmup`` / ``rep``: target milliseconds of untimed and timed calls (the counts follow from a five-call
+    estimate; ``_n_warmup`` / ``_n_repeat`` override them).  ``backend``: ``"event"`` (an event pair per call),
+    ``"cudagraph"`` (the calls captured into one graph, replayed ten times) or ``"cupti"`` (device time from the
+    kernel trace; ``"profiler"`` is accepted as a name for it).  ``return_mode`` (mean, median, min, max) or
+    ``quantiles`` (a list of fractions; one fraction returns a float) pick the summary; ``early_stop_baseline``
+    returns the estimate at once when it already exceeds that many milliseconds.  ``device``: a device index or
+    ``torch.device`` to run on (default: the current one).
+    """
+    if return_mode not in ("min", "max", "mean", "median"):
+        raise ValueError(f"Invalid return_mode: {return_mode}")
+    if backend not in ("event", "cudagraph", "cupti", "profiler"):
+        raise ValueError(f"Unknown profiler backend: {backend}")
+    if device is not None:
+        dev = torch.device("cuda", device) if isinstance(device, int) else torch.device(device)
+        if dev.type != "cuda":
+            raise ValueError(f"do_bench device must be a CUDA device, got {dev}")
+        with torch.cuda.device(dev):
+            return do_bench(fn, warmup, rep, _n_warmup, _n_repeat, quantiles, fast_flush, backend, return_mode, None,
+                            cache_size, early_stop_baseline)
+
     fn()
     torch.cuda.synchronize()
-    cache = torch.empty(cache_size * 1024 * 1024 // 4, dtype=torch.int, device="cuda")
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
+    nbytes = cache_size * 1024 * 1024
+    cache = torch.empty(nbytes // 4 if fast_flush else nbytes, dtype=torch.int if fast_flush else torch.int8, device="cuda")
+    flush = cache.zero_
+
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    first.record()
     for _ in range(5):
-        cache.zero_()
+        flush()
         fn()
-    end.record()
+    last.record()
     torch.cuda.synchronize()
-    estimate_ms = max(start.elapsed_time(end) / 5, 1e-4)
-    n_warmup = _n_warmup if _n_warmup > 0 else max(1, int(warmup / estimate_ms))
-    n_repeat = _n_repeat if _n_repeat > 0 else max(1, int(rep / estimate_ms))
-    n_warmup, n_repeat = min(n_warmup, 1000), min(n_repeat, 1000)
+    estimate_ms = max(first.elapsed_time(last) / 5, 1e-4)
+    if early_stop_baseline is not None and estimate_ms > early_stop_baseline:
+        return [estimate_ms] * len(quantiles) if quantiles is not None else estimate_ms
+
+    n_warmup = min(_n_warmup if _n_warmup > 0 else max(1, int(warmup / estimate_ms)), 1000)
+    n_repeat = min(_n_repeat if _n_repeat > 0 else max(1, int(rep / estimate_ms)), 1000)
     for _ in range(n_warmup):
         fn()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
-    for i in range(n_repeat):
-        cache.zero_()
-        starts[i].record()
-        fn()
-        ends[i].record()
-    torch.cuda.synchronize()
-    times = torch.tensor([s.elapsed_time(e) for s, e in zip(starts, ends)], dtype=torch.float)
-    return getattr(torch, return_mode)(times).item()
+    if backend == "event":
+        times = _time_with_events(fn, flush, n_repeat)
+    elif backend == "cudagraph":
+        times = _time_with_graph(fn, flush, n_repeat)
+    else:
+        return _time_with_trace(fn, flush, n_repeat).item()
+    return _summarise(times, quantiles, return_mode)
 
 
 class Profiler:
