@@ -136,15 +136,17 @@ def _time_with_trace(fn, flush, n_repeat):
 
     from torch.profiler import ProfilerActivity, profile, record_function, schedule
 
-    with warnings.catch_warnings(), profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA], schedule=schedule(wait=1, warmup=0, active=1, repeat=1)) as prof:
+    with warnings.catch_warnings():
         warnings.simplefilter("ignore", UserWarning)  # "won't be using warmup", "clears events at the end of each cycle"
-        for _ in range(2):  # the first step is the schedule's wait step
-            for _ in range(n_repeat):
-                with record_function(_FLUSH_RANGE):
-                    flush()
-                fn()
-            torch.cuda.synchronize()
-            prof.step()
+        plan = schedule(wait=1, warmup=0, active=1, repeat=1)
+        with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA], schedule=plan) as prof:
+            for _ in range(2):  # the first step is the schedule's wait step
+                for _ in range(n_repeat):
+                    with record_function(_FLUSH_RANGE):
+                        flush()
+                    fn()
+                torch.cuda.synchronize()
+                prof.step()
     kernels_us = flush_us = 0.0
     for ev in prof.events():
         if getattr(getattr(ev, "device_type", None), "name", "") != "CUDA":
