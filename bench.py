@@ -304,6 +304,26 @@ def bench_int4(torch, tl, workloads, M, N, K, a_packed, steps, warmup, dev, **tk
     return {"us": ms * 1e3, "bytes": nbytes, "flops": workloads.flops(M, N, K), "timing": graphed}
 
 
+def bench_int8_gemv(torch, tl, M, N, K, bits, steps, warmup, dev, **tk):
+    """The integer branch of dequantize_gemv (int8 activations, int32 out) with the fast decoder: 4-bit words through
+    interleave_weight(., 4, "int8"), w = q - 7 (decode_i4s_to_i8s)."""
+    from tilelang_amd import quantize
+
+    rng = np.random.default_rng(0)
+    A = torch.from_numpy(rng.integers(-127, 128, size=(M, K), dtype=np.int8)).to(dev)
+    nbytes = N * K * bits // 8 + M * K + 4 * M * N
+    nc = _copies(nbytes)
+    Bs = []
+    for _ in range(nc):
+        b = torch.from_numpy(rng.integers(0, 256, size=(N, K * bits // 8), dtype=np.uint8)).view(torch.int8)
+        Bs.append(quantize.interleave_weight(b, bits, "int8").to(dev).contiguous())
+    C = torch.empty((M, N), dtype=torch.int32, device=dev)
+    kern = tl.dequantize_gemv(M, N, K, "int8", "int32", "int32", num_bits=bits, source_format="int", fast_decoding=True)
+    fns = [(lambda i=i: kern(A, Bs[i], C, skip_tensor_validation=True)) for i in range(nc)]
+    ms, graphed = _time_launches(torch, fns, steps, warmup, **tk)
+    return {"us": ms * 1e3, "bytes": nbytes, "flops": 2 * M * N * K, "timing": graphed}
+
+
 def _row(config, r, bound, peak):
     sec = r["us"] * 1e-6
     row = {"config": config, "us": r["us"], "us_min": r["timing"]["us_min"], "GB/s": r["bytes"] / sec / 1e9, "TFLOP/s": r["flops"] / sec / 1e12, "bound": bound}
@@ -481,6 +501,8 @@ def main():
                                r, "hbm", MFMA_BF16_PEAK))
         r = bench_w2a16(torch, tl, 1, 28672, 8192, S, W, dev)
         shapes.append(_row("w2a16_gemv M=1 N=28672 K=8192 (num_bits=2, interleaved words, (c-2)*s)", r, "hbm", MFMA_BF16_PEAK))
+        r = bench_int8_gemv(torch, tl, 1, 28672, 8192, 4, S, W, dev)
+        shapes.append(_row("w4a8_gemv M=1 N=28672 K=8192 (int8 activations, interleaved words, q - 7, int32 out)", r, "hbm", MFMA_I8_PEAK))
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
         mx_run = r
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))

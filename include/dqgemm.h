@@ -244,18 +244,37 @@ enum dq_i4_decode {
   DQ_I4_TWOS = 1,          /* w = sext4(q), plain nibbles (example_dequant_gemm_w4a8.py:10-21)                          */
   DQ_I4U_INTERLEAVED = 2,  /* w = q, words through interleave_weight(qB, 4, "int8"): decode_i4u_to_i8s,
                               examples/dequantize_gemm/quantize/lop3.py:1027-1047                                      */
-  DQ_I4S_INTERLEAVED = 3   /* w = q - 7 (the decoder's MEDIAN_NUM is 0x07070707), same words: decode_i4s_to_i8s,
+  DQ_I4S_INTERLEAVED = 3,  /* w = q - 7 (the decoder's MEDIAN_NUM is 0x07070707), same words: decode_i4s_to_i8s,
                               lop3.py:999-1025                                                                         */
+  DQ_I2_TO_I4 = 4          /* B[N,K/4] holds 2-bit codes, w = c: decode_i2u_to_i4s / decode_i2s_to_i4s, lop3.py:1049-1089
+                              (the 2-bit operand of the int4 x int4 matrix instruction; the signed decoder's adjustment
+                              is commented out in the reference, so both are w = c).  With a_packed = 1 only.          */
 };
+
+/* flag for `transposed` (tests and measurements): run the tiled GEMM also where the decode kernel would be taken */
+#define DQ_I4_KERNEL_TILED 32
 
 /* int8 x 4-bit, exact int32: C[M,N] or Ct[N,M] (transposed = 1) = A . decode(B[N,K/2])^T, `decode` a DQ_I4_* value.
  * Replaces `call(A, B, Ct)` of examples/dequantize_gemm/example_dequant_gemm_w4a8.py:109-147 (DQ_I4_TWOS), the int8
- * path of example_dequant_gemm_fine_grained.py (DQ_I4_UNSIGNED) and the int8 branch of
- * example_dequant_gemv_fp16xint4.py:47-48,113-133 with fast_decoding (the two interleaved decoders).
+ * path of example_dequant_gemm_fine_grained.py (DQ_I4_UNSIGNED) and the int8 branch (`use_dp4a`) of
+ * example_dequant_gemv_fp16xint4.py:47-54,113-133: its slow path (DQ_I4_TWOS) and, with fast_decoding, the two
+ * interleaved decoders.  M <= 4 runs as a streaming dot-product kernel (K <= 16384; 16 bytes of B per lane,
+ * v_dot4_i32_i8, the decoder's constant applied through the sum of the activations), larger M on the tiled GEMM.
  * a_packed 1: A is packed int4 too, A[M,K/2] (examples/gemm_int4/example_tilelang_gemm_int4.py:17-38), DQ_I4_TWOS
- * only, K < 131072 (both operands carry a factor 16 in the int32 accumulator).  Requires K % 128 == 0. */
+ * or DQ_I2_TO_I4, K < 131072 (the operands carry a factor 16 in the int32 accumulator).  Requires K % 128 == 0. */
 int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int decode, int a_packed,
                         int transposed, dq_stream_t stream);
+
+/* int8 x 1-bit decode GEMV, exact int32: C[M,N] = A[M,K] int8 . decode(B[N,K/8])^T for M <= 4, K <= 65536,
+ * K % 128 == 0.  `convention` (a dq_i2_convention value read for one bit): DQ_I2_UNSIGNED w = c (decode_i1u_to_i8s),
+ * DQ_I2_OFFSET w = 2 c - 1 (decode_i1s_to_i8s), DQ_I2_TWOS w = -c (the sign extension of a one-bit field, the int8
+ * branch's slow path, quantization.py:333-343).  `layout`: DQ_LAYOUT_PLAIN (bit e of a byte is code e) or
+ * DQ_LAYOUT_INTERLEAVED (32-bit words through interleave_weight(qB, 1, "int8"), utils.py:102-109, the order the
+ * reference's 16-bit decoder expects).  Replaces the int8 branch of
+ * examples/dequantize_gemm/example_dequant_gemv_fp16xint4.py:47-54,126-133 at num_bits = 1 with the decoders of
+ * examples/dequantize_gemm/quantize/lop3.py:893-948. */
+int call_gemv_int8xint1(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout,
+                        dq_stream_t stream);
 
 /* ---- plain GEMM on the same MFMA tile (no dequantise step) ----------------------------------------- */
 

@@ -289,6 +289,53 @@ def decode_i4_fast_int8(packed_interleaved: np.ndarray, signed: bool) -> np.ndar
     return fast_decode_i4_to_i8(w, signed).reshape(p.shape[0], -1)
 
 
+def fast_decode_i1_to_i8(halfwords: np.ndarray, signed: bool) -> np.ndarray:
+    """Semantics of decode_i1{u,s}_to_i8s on one uint16 (16 one-bit codes) -> 16 int8, in output order.
+
+    Follows examples/dequantize_gemm/quantize/lop3.py:893-948: ``i1b = (x & 0x0f0f) | ((x & 0xf0f0) << 12)``; for i
+    in 0..3 ``i8s[i] = (i1b >> i) & 0x01010101``; the signed form then computes ``v + v - 1`` per byte (``2 c - 1``).
+    Output element ``4 i + b`` is byte ``b`` of ``i8s[i]``.
+    """
+    x = np.asarray(halfwords).astype(np.uint32) & np.uint32(0xFFFF)
+    i1b = (x & np.uint32(0x0F0F)) | ((x & np.uint32(0xF0F0)) << np.uint32(12))
+    out = np.empty(x.shape + (16,), dtype=np.int8)
+    for i in range(4):
+        d = (i1b >> np.uint32(i)) & np.uint32(0x01010101)
+        for b in range(4):
+            v = ((d >> np.uint32(8 * b)) & 0xFF).astype(np.int16)
+            out[..., 4 * i + b] = (2 * v - 1 if signed else v).astype(np.int8)
+    return out
+
+
+def decode_i1_fast_int8(packed_interleaved: np.ndarray, signed: bool) -> np.ndarray:
+    """[N, K/8] bytes whose 32-bit words went through ``interleave_weight(., 1, "int8")`` -> int8 [N, K] as
+    decode_i1{u,s}_to_i8s yields them, 16 values per halfword (lop3.py:893-948)."""
+    p = np.ascontiguousarray(packed_interleaved).view(np.uint8)
+    h = p.view(np.uint16)
+    return fast_decode_i1_to_i8(h, signed).reshape(p.shape[0], -1)
+
+
+def fast_decode_i2_to_i4(words: np.ndarray) -> np.ndarray:
+    """Semantics of decode_i2{u,s}_to_i4s on one uint32 (16 two-bit codes) -> two uint32 of eight 4-bit fields each.
+
+    Follows examples/dequantize_gemm/quantize/lop3.py:1049-1089: with N = 16, for i in 0..1
+    ``i4s[i] = (i2b[0] >> 2 i) & 0x33333333``: nibble ``e`` of ``i4s[i]`` is code ``2 e + i``.  The reference's signed
+    form subtracts nothing (its adjustment is commented out, :1068-1073), so both decoders return the unsigned code
+    in a nibble.  Returns ``[..., 2]`` uint32.
+    """
+    w = np.asarray(words).astype(np.uint32)
+    return np.stack([(w >> np.uint32(2 * i)) & np.uint32(0x33333333) for i in range(2)], axis=-1)
+
+
+def decode_i2_fast_int4(packed: np.ndarray) -> np.ndarray:
+    """[N, K/4] bytes of 2-bit codes -> [N, K/2] bytes of 4-bit fields as decode_i2{u,s}_to_i4s writes them: word ``j``
+    of a row becomes words ``2 j`` and ``2 j + 1``; field ``e`` of output word ``2 j + i`` is code ``2 e + i`` of
+    input word ``j`` (lop3.py:1049-1089)."""
+    p = np.ascontiguousarray(packed).view(np.uint8)
+    out = fast_decode_i2_to_i4(p.view(np.uint32))  # [N, W, 2]
+    return np.ascontiguousarray(out.reshape(p.shape[0], -1)).view(np.uint8)
+
+
 def fast_decode_i4u_to_f16_zeros_quantized(words: np.ndarray, scale, qzero) -> np.ndarray:
     """Bit-level semantics of decode_i4u_to_f16_scale_zeros_quantized on one uint32 -> 8 fp16, in output order
     (examples/dequantize_gemm/quantize/lop3.py:326-363): ``h = (w >> 4i) & 0x000f000f | 0x64006400`` as two fp16,

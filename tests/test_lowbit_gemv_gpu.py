@@ -169,3 +169,135 @@ def test_dequantize_gemv_int8_exact(cuda, M, N, K, bits, fast, fmt):
     kernel(torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda), C)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), A.astype(np.int64) @ W.T)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (2, 520, 2048), (4, 300, 4096), (1, 4099, 8192), (3, 64, 11008),
+                                   (4, 96, 16384), (1, 7, 128), (2, 33, 12288)])
+@pytest.mark.parametrize("decode", ["twos", "fast_uint", "fast_int", "unsigned"])
+def test_int8xint4_decode_gemv_exact(cuda, M, N, K, decode):
+    """The streaming int8 x 4-bit decode kernel (M <= 4: v_dot4_i32_i8 over 16 bytes of B per lane, the decoder's
+    constant applied through the sum of the activations): exact int32 against the oracle's decoders, shapes that take
+    a quarter of a wave, one to four waves and two chunks per thread, ragged N; and bit for bit what the tiled GEMM
+    gives on the same operands."""
+    from tilelang_amd import _lib
+    import ctypes
+
+    rng = np.random.default_rng(M * 3 + N + K)
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    packed = _packed(N, K, 4, seed=K + len(decode))
+    if decode == "twos":
+        W, B, dec = orc.decode_i4_signed(packed).astype(np.int64), packed, 1
+    elif decode == "unsigned":
+        W, B, dec = orc.unpack_u4(packed).astype(np.int64), packed, 0
+    else:
+        B = orc.interleave_weight(packed.view(np.int8), 4, "int8").view(np.uint8)
+        W = orc.decode_i4_fast_int8(B, signed=(decode == "fast_int")).astype(np.int64)
+        dec = 3 if decode == "fast_int" else 2
+    lib = _lib.get_library()
+    Ad, Bd = torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda)
+    outs = []
+    for flag in (0, 32):  # the library's choice (the decode kernel), then the tiled GEMM by name
+        C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+        rc = lib.call_gemm_int8xint4(ctypes.c_void_p(Ad.data_ptr()), ctypes.c_void_p(Bd.data_ptr()), ctypes.c_void_p(C.data_ptr()),
+                                     M, N, K, dec, 0, flag, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.get_last_error().decode()
+        torch.cuda.synchronize()
+        outs.append(C.cpu().numpy())
+    np.testing.assert_array_equal(outs[0].astype(np.int64), A.astype(np.int64) @ W.T)
+    np.testing.assert_array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("M", [1, 4])
+@pytest.mark.parametrize("decode", ["twos", "fast_int"])
+def test_int8xint4_decode_gemv_full_size(cuda, M, decode):
+    """N = 28672, K = 8192 (117 MB of weights): every int32 output."""
+    N, K = 28672, 8192
+    print(f"int8 x int4 decode GEMV full size: M={M} decode={decode}", flush=True)
+    rng = np.random.default_rng(17 + M)
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    packed = _packed(N, K, 4, seed=23)
+    fast = decode == "fast_int"
+    if fast:
+        B = orc.interleave_weight(packed.view(np.int8), 4, "int8").view(np.uint8)
+        W = (orc.unpack_u4(packed).astype(np.int32) - 7)
+    else:
+        B, W = packed, orc.decode_i4_signed(packed).astype(np.int32)
+    kernel = tl.dequantize_gemv(M, N, K, "int8", "int32", "int32", num_bits=4, source_format="int", fast_decoding=fast)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    kernel(torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda), C)
+    torch.cuda.synchronize()
+    ref = (A.astype(np.float64) @ W.T.astype(np.float64)).astype(np.int64)  # |sum| < 2^53: exact in fp64
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (2, 520, 4096), (3, 77, 8192), (4, 300, 16384), (1, 9, 128), (1, 40, 65536),
+                                   (2, 4099, 2048)])
+@pytest.mark.parametrize("fast,fmt", [(False, "uint"), (True, "uint"), (True, "int")])
+def test_int8xint1_decode_gemv_exact(cuda, M, N, K, fast, fmt):
+    """int8 x 1-bit (decode_i1{u,s}_to_i8s, lop3.py:893-948, over interleave_weight(., 1, "int8") words; the slow path
+    sign-extends the one-bit field): exact int32."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    packed = _packed(N, K, 1, seed=5 + int(fast))
+    if fast:
+        B = orc.interleave_weight(packed.view(np.int8), 1, "int8").view(np.uint8)
+        W = orc.decode_i1_fast_int8(B, signed=(fmt == "int")).astype(np.int64)
+        assert np.array_equal(W, orc.decode_lowbit(packed, 1, "offset" if fmt == "int" else "unsigned").astype(np.int64))
+    else:
+        B, W = packed, orc.decode_lowbit(packed, 1, "twos").astype(np.int64)
+    kernel = tl.dequantize_gemv(M, N, K, "int8", "int32", "int32", num_bits=1, source_format=fmt, fast_decoding=fast)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    kernel(torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda), C)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), A.astype(np.int64) @ W.T)
+
+
+def test_int8xint1_refuses_prefill_batches(cuda):
+    with pytest.raises(ValueError, match="decode kernel"):
+        tl.dequantize_gemv(8, 64, 1024, "int8", "int32", "int32", num_bits=1)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (300, 520, 384), (1, 64, 1024), (1500, 2000, 256)])
+def test_int4xint2_gemm_exact(cuda, M, N, K):
+    """Packed int4 activations x 2-bit codes (the operands decode_i2{u,s}_to_i4s prepare for the int4 x int4 matrix
+    instruction, lop3.py:1049-1089; both decoders leave the code unsigned): exact int32."""
+    rng = np.random.default_rng(M + N)
+    Ap = rng.integers(0, 256, size=(M, K // 2), dtype=np.uint8)
+    Bp = _packed(N, K, 2, seed=9)
+    # the reference decoder's own output, read back as unsigned nibbles: nibble e of word 2 j + i is code 2 e + i of word j
+    i4 = orc.unpack_u4(orc.decode_i2_fast_int4(Bp)).reshape(N, K // 16, 2, 8)
+    codes = orc.unpack_u2(Bp).reshape(N, K // 16, 8, 2)
+    assert np.array_equal(i4.transpose(0, 1, 3, 2), codes)
+    kernel = tl.matmul_nt_int4xint2(M, N, K)
+    C = kernel(torch.from_numpy(Ap.view(np.int8)).to(cuda), torch.from_numpy(Bp.view(np.int8)).to(cuda))
+    torch.cuda.synchronize()
+    ref = orc.decode_i4_signed(Ap).astype(np.int64) @ orc.unpack_u2(Bp).astype(np.int64).T
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), ref)
+
+
+@pytest.mark.parametrize("M", [1, 4, 20])
+@pytest.mark.parametrize("qfmt", ["int16", "packed4"])
+def test_w2a16_quantized_zeros(cuda, M, qfmt):
+    """zeros_mode="quantized" for two bits (decode_i2u_to_f16_scale_zeros_quantized, lop3.py:638-677): integer zero
+    points folded into the magic number, (1024 + c) + (0xe400 | qz) = c - qz exactly, times the scale once."""
+    N, K, group = 520, 2048, 128
+    rng = np.random.default_rng(31 + M)
+    A = rng.standard_normal((M, K)).astype(np.float16)
+    packed = _packed(N, K, 2, seed=3)
+    S = rng.uniform(0.005, 0.02, size=(N, K // group)).astype(np.float16)
+    qz = rng.integers(0, 4, size=(N, K // group)).astype(np.int16)
+    Z = qz if qfmt == "int16" else (qz[:, 0::2] | (qz[:, 1::2] << 4)).astype(np.uint8)
+    B = orc.interleave_weight(packed.view(np.int8), 2, "float16").view(np.uint8)
+    kernel = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", num_bits=2, source_format="uint", fast_decoding=True,
+                                group_size=group, with_scaling=True, with_zeros=True, zeros_mode="quantized", qzeros_format=qfmt)
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kernel(torch.from_numpy(A).to(cuda), torch.from_numpy(B.view(np.int8)).to(cuda), torch.from_numpy(S).to(cuda),
+           torch.from_numpy(Z).to(cuda), C)
+    torch.cuda.synchronize()
+    # the oracle's tile with the integers as fp16 zero points: c - qz is exact either way
+    W = orc.dequant_lowbit(packed, 2, "unsigned", S, qz.astype(np.float16), group, "original").astype(np.float32)
+    ref = (A.astype(np.float32) @ W.T).astype(np.float16).astype(np.float32)
+    np.testing.assert_allclose(C.float().cpu().numpy(), ref, rtol=1e-2, atol=1e-2)
+    with pytest.raises(ValueError, match="quantized"):
+        tl.dequantize_gemv(M, N, K, num_bits=2, source_format="int", fast_decoding=True, group_size=group, with_scaling=True,
+                           with_zeros=True, zeros_mode="quantized")

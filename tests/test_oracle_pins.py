@@ -255,6 +255,53 @@ def test_i4_to_i8_fast_decode_and_interleave():
     np.testing.assert_array_equal(orc.decode_i4_fast_int8(il, signed=True), orc.unpack_u4(raw).astype(np.int8) - 7)
 
 
+def test_i1_to_i8_fast_decode_all_halfwords_and_interleave():
+    """decode_i1{u,s}_to_i8s (lop3.py:893-948) over every 16-bit input, against its bit shuffle written out bit by
+    bit: output element 4 i + b is input bit (i, 8 + i, 4 + i, 12 + i)[b]; the signed form is 2 c - 1.  Over words
+    that went through interleave_weight(., 1, "int8") (with its extra nibble shuffle, utils.py:102-109) the decoder
+    returns the codes in k order."""
+    x = np.arange(65536, dtype=np.uint32)
+    got_u = orc.fast_decode_i1_to_i8(x, signed=False)
+    got_s = orc.fast_decode_i1_to_i8(x, signed=True)
+    for i in range(4):
+        for b, bit in enumerate((i, 8 + i, 4 + i, 12 + i)):
+            c = ((x >> bit) & 1).astype(np.int8)
+            np.testing.assert_array_equal(got_u[:, 4 * i + b], c)
+            np.testing.assert_array_equal(got_s[:, 4 * i + b], 2 * c - 1)
+    rng = np.random.default_rng(14)
+    codes = rng.integers(0, 2, size=(8, 256)).astype(np.int8)
+    codes[0, :32] = np.eye(32, dtype=np.int8)[5]  # a single set bit
+    raw = orc.general_compress(codes, 1)
+    il = orc.interleave_weight(raw.view(np.int8), 1, "int8").view(np.uint8)
+    np.testing.assert_array_equal(orc.decode_i1_fast_int8(il, signed=False), codes)
+    np.testing.assert_array_equal(orc.decode_i1_fast_int8(il, signed=True), 2 * codes - 1)
+    np.testing.assert_array_equal(orc.decode_lowbit(raw, 1, "offset"), 2 * codes - 1)
+    for k in range(32):  # every bit position of a word
+        one = np.zeros((1, 32), dtype=np.int8)
+        one[0, k] = 1
+        w = orc.interleave_weight(orc.general_compress(one, 1).view(np.int8), 1, "int8").view(np.uint8)
+        assert orc.decode_i1_fast_int8(w, signed=False)[0].tolist() == one[0].tolist()
+
+
+def test_i2_to_i4_fast_decode():
+    """decode_i2{u,s}_to_i4s (lop3.py:1049-1089): (w >> 2 i) & 0x33333333 leaves code 2 e + i in nibble e of output
+    word i, for every code value at every position; nothing is subtracted (the signed adjustment is commented out in
+    the reference)."""
+    for k in range(16):
+        for c in range(4):
+            w = np.array([c << (2 * k)], dtype=np.uint32)
+            out = orc.fast_decode_i2_to_i4(w)[0]
+            want = [0, 0]
+            want[k % 2] = c << (4 * (k // 2))
+            assert out.tolist() == want
+    rng = np.random.default_rng(15)
+    codes = rng.integers(0, 4, size=(4, 128)).astype(np.int8)
+    packed = orc.general_compress(codes, 2)
+    nib = orc.unpack_u4(orc.decode_i2_fast_int4(packed))  # [4, 128] nibbles of the decoder's output
+    want = codes.reshape(4, 8, 8, 2).transpose(0, 1, 3, 2).reshape(4, 128)  # per 16 codes: the even ones, then the odd ones
+    np.testing.assert_array_equal(nib, want)
+
+
 def test_i2_conventions():
     packed = np.array([[0b11100100]], dtype=np.uint8)  # codes 0,1,2,3 low first
     assert orc.unpack_u2(packed).tolist() == [[0, 1, 2, 3]]

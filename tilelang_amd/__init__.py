@@ -21,6 +21,7 @@ from .kernels import (  # noqa: F401
     matmul_int8xint4,
     matmul,
     matmul_nt_int4,
+    matmul_nt_int4xint2,
     matmul_w4_fine_grained,
     matmul_w4a16,
     quantize_bf16_mxfp4,

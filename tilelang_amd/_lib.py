@@ -40,6 +40,7 @@ SIGNATURES = {
     "call_bitnet_activation_quant": [_vp, _vp, _vp, _i, _i, _vp],
     "call_quantize_bf16_mxfp4": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "call_gemm_int8xint4": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "call_gemv_int8xint1": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_gemm_plain": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_gemm_mxfp4_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
 }

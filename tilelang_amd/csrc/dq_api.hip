@@ -50,6 +50,8 @@ int i2_gemm_kslice(const void* A, const void* B, void* C, int M, int N, int K, i
                    float s_w, int bitnet_epilogue, int force, hipStream_t stream);
 int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int out_kind, hipStream_t stream);
+int i4_gemv(const void* A, const void* B, void* C, int M, int N, int K, int decode, hipStream_t stream);
+int i1_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, hipStream_t stream);
 int activation_quant(const void* X, void* Q, void* S, int M, int K, hipStream_t stream);
 int mxfp4_quant(const void* W, void* B, void* S, int N, int K, int scale_bias, hipStream_t stream);
 int fp16_fp4_gemm_splitk(const void* A, const void* B, void* parts, void* C, int M, int N, int K, int split,
@@ -64,6 +66,7 @@ int plain_gemm(const void* A, const void* B, void* C, void* workspace, int M, in
                int trans_A, int trans_B, hipStream_t stream);
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static int variant_bits(int transposed) { return transposed & ~1; }
 
 // ---- device-resident scratch of the entry point that allocates nothing ---------------------------------
 // One copy per GPU, held from the moment the library's code object is loaded on that GPU until the process
@@ -445,7 +448,34 @@ extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M,
                                    int a_packed, int transposed, dq_stream_t stream) {
   const char* fn = "call_gemm_int8xint4";
   if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
-  if (decode < DQ_I4_UNSIGNED || decode > DQ_I4S_INTERLEAVED) DQ_FAIL("%s: unknown decode %d", fn, decode);
-  if (a_packed && decode != DQ_I4_TWOS) DQ_FAIL("%s: a packed A goes with decode DQ_I4_TWOS only (got %d)", fn, decode);
-  return i4_gemm(A, B, C, M, N, K, decode, a_packed, transposed, (hipStream_t)stream);
+  if (decode < DQ_I4_UNSIGNED || decode > DQ_I2_TO_I4) DQ_FAIL("%s: unknown decode %d", fn, decode);
+  if (decode == DQ_I2_TO_I4 && !a_packed) DQ_FAIL("%s: decode DQ_I2_TO_I4 (2-bit codes to int4) goes with a packed int4 A", fn);
+  if (a_packed && decode != DQ_I4_TWOS && decode != DQ_I2_TO_I4)
+    DQ_FAIL("%s: a packed A goes with decode DQ_I4_TWOS or DQ_I2_TO_I4 only (got %d)", fn, decode);
+  if (a_packed && K >= 131072) DQ_FAIL("%s: K=%d is beyond the 131071 that keep the int32 accumulation of a packed A exact", fn, K);
+  // decode batches: the streaming dot-product kernel (Ct[N,1] and C[1,N] are the same bytes)
+  if (!a_packed && M <= 4 && (!transposed || M == 1) && !(variant_bits(transposed) & DQ_I4_KERNEL_TILED)) {
+    const int rc = i4_gemv(A, B, C, M, N, K, decode, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
+  return i4_gemm(A, B, C, M, N, K, decode, a_packed, transposed & 1, (hipStream_t)stream);
+}
+
+extern "C" int call_gemv_int8xint1(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout,
+                                   dq_stream_t stream) {
+  const char* fn = "call_gemv_int8xint1";
+  if (check_gemm_args(fn, A, B, C, M, N, K, 128)) return -1;
+  if (convention < I2_UNSIGNED || convention > I2_TWOS) DQ_FAIL("%s: unknown code convention %d", fn, convention);
+  if (layout != LAYOUT_PLAIN && layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
+  if (M > 4) DQ_FAIL("%s: M=%d is beyond the decode batch (4) this kernel is built for", fn, M);
+  if (K > 65536) DQ_FAIL("%s: K=%d is beyond the 65536 this kernel is built for", fn, K);
+  // the activations of two rows at a time fit a thread's registers
+  for (int m0 = 0; m0 < M; m0 += 2) {
+    const int rows = M - m0 < 2 ? M - m0 : 2;
+    const int rc = i1_gemv((const int8_t*)A + (size_t)m0 * K, B, (int32_t*)C + (size_t)m0 * N, rows, N, K, convention, layout,
+                           (hipStream_t)stream);
+    if (rc > 0) DQ_FAIL("%s: shape M=%d N=%d K=%d is not covered", fn, M, N, K);
+    if (rc < 0) return rc;
+  }
+  return 0;
 }

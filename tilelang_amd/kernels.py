@@ -19,7 +19,7 @@ from .adapter import KernelAdapter, KernelParam
 W4_UNSIGNED, W4_SIGNED, W4_OFFSET8, W4_SCALE, W4_USCALE, W4_ZEROS_ORIGINAL, W4_ZEROS_RESCALE, W4_ZEROS_FOLDED = range(8)
 LAYOUT_PLAIN, LAYOUT_INTERLEAVED, LAYOUT_FRAGMENTS = 0, 1, 2
 DECODER_CONVERTER = 4  # flag of call_dequantize_w4's layout: dump the tile with the fp8-converter decoder
-I4_UNSIGNED, I4_TWOS, I4U_INTERLEAVED, I4S_INTERLEAVED = range(4)
+I4_UNSIGNED, I4_TWOS, I4U_INTERLEAVED, I4S_INTERLEAVED, I2_TO_I4 = range(5)
 
 _DTYPES = {
     "float16": torch.float16,
@@ -149,7 +149,7 @@ def dequantize_gemv(
         raise ValueError("dequantize_gemv: storage_dtype must be int8 or uint8")
     if num_bits < 4:
         return _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fast_decoding, group_size,
-                                       with_scaling, with_zeros, zeros_mode, _formula_fast)
+                                       with_scaling, with_zeros, zeros_mode, _formula_fast, qzeros_format)
     if group_size == -1:
         group_size = K
     if K % 128 != 0:
@@ -232,13 +232,27 @@ def _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dty
         def launch(ptrs, stream):
             return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, dec, 0, 0, stream)
 
+    elif num_bits == 1:
+        # slow path: the sign extension of a one-bit field, w = -c.  Fast path: the words went through
+        # interleave_weight(B, 1, "int8") and decode as decode_i1u_to_i8s (w = c) or decode_i1s_to_i8s (w = 2 c - 1)
+        # (examples/dequantize_gemm/quantize/lop3.py:893-948)
+        if M > 4:
+            raise ValueError(f"dequantize_gemv: int8 x 1-bit is a decode kernel, M <= 4 (got {M})")
+        if K > 65536:
+            raise ValueError(f"dequantize_gemv: int8 x 1-bit is built for K <= 65536 (got {K})")
+        conv = I2_TWOS if not formula_fast else (I2_OFFSET if source_format == "int" else I2_UNSIGNED)
+        layout = LAYOUT_INTERLEAVED if fast_decoding else LAYOUT_PLAIN
+
+        def launch(ptrs, stream):
+            return _lib.get_library().call_gemv_int8xint1(ptrs[0], ptrs[1], ptrs[2], M, N, K, conv, layout, stream)
+
     else:
-        raise ValueError("dequantize_gemv: int8 activations are built for num_bits 4 and 2")
+        raise ValueError("dequantize_gemv: int8 activations are built for num_bits 4, 2 and 1")
     return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
 
 
 def _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fast_decoding, group_size, with_scaling,
-                            with_zeros, zeros_mode, _formula_fast) -> KernelAdapter:
+                            with_zeros, zeros_mode, _formula_fast, qzeros_format="int16") -> KernelAdapter:
     """The ``num_bits`` = 2 and 1 cases of :func:`dequantize_gemv`: ``B[N, K * num_bits / 8]``.
 
     Slow path: two's-complement codes whatever ``source_format`` says
@@ -246,7 +260,11 @@ def _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fas
     ``interleave_weight(B, num_bits, "float16")`` and decodes as ``c`` (``"uint"``) or as ``c - 2`` / ``2 c - 1``
     (``"int"``, two bits / one bit; examples/dequantize_gemm/quantize/lop3.py:424-463, 679-746), times
     ``Scale[N, K/group]`` with ``with_scaling``, and with ``with_zeros`` ``(w - z) * s`` (``"original"``) or
-    ``w * s - z`` (``"rescale"``) (lop3.py:564-636, 812-891).  Call surface ``kernel(A, B[, Scale[, Zeros]], C)``.
+    ``w * s - z`` (``"rescale"``) (lop3.py:564-636, 812-891).  ``zeros_mode="quantized"`` (two bits, ``"uint"``
+    codes: decode_i2u_to_f16_scale_zeros_quantized, lop3.py:638-677): integer zero points in the formats of
+    :func:`_zeros_params`; the decoder's ``(1024 + c) + (0xe400 | qz)`` is ``c - qz`` exactly, so they are unpacked to
+    fp16 in front of the kernel, which runs ``(c - z) * s``: the same bits.  Call surface
+    ``kernel(A, B[, Scale[, Zeros]], C)``.
     """
     chunk = 128 // num_bits
     if group_size == -1:
@@ -259,7 +277,11 @@ def _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fas
         raise ValueError(f"dequantize_gemv: num_bits={num_bits} is a decode kernel, M <= 64 (got {M})")
     if with_zeros and not with_scaling:
         raise ValueError("with_zeros requires with_scaling")
-    if with_zeros and zeros_mode not in ("original", "rescale"):
+    quantized = with_zeros and zeros_mode == "quantized"
+    if quantized and not (num_bits == 2 and fast_decoding and source_format == "uint"):
+        raise ValueError("dequantize_gemv: zeros_mode 'quantized' below four bits is the two-bit unsigned fast decoder's "
+                         "(num_bits=2, source_format='uint', fast_decoding=True)")
+    if with_zeros and zeros_mode not in ("original", "rescale", "quantized"):
         raise ValueError(f"dequantize_gemv: zeros_mode {zeros_mode!r} is not built for num_bits={num_bits}")
     if with_scaling and (K % group_size != 0 or group_size % chunk != 0):
         raise ValueError(f"dequantize_gemv: group_size={group_size} must divide K={K} and be a multiple of {chunk}")
@@ -274,17 +296,29 @@ def _dequantize_gemv_lowbit(M, N, K, num_bits, storage_dtype, source_format, fas
               KernelParam("B", _dtype(storage_dtype), (N, K * num_bits // 8), packed=True)]
     if with_scaling:
         params.append(KernelParam("Scale", torch.float16, (N, K // group_size)))
+    zwork, zfmt = None, None
+    groups = K // group_size
     if with_zeros:
-        params.append(KernelParam("Zeros", torch.float16, (N, K // group_size)))
+        zparam, zwork, zfmt = _zeros_params(N, groups, zeros_mode, qzeros_format)
+        params.append(zparam)
+    c_idx = len(params)
     params.append(KernelParam("C", torch.float16, (M, N)))
+    if zwork is not None:
+        params.append(zwork)
 
     def launch(ptrs, stream):
+        lib = _lib.get_library()
         s = ptrs[2] if with_scaling else None
         z = ptrs[3] if with_zeros else None
-        return _lib.get_library().call_dequantize_gemv_lowbit(ptrs[0], ptrs[1], s, z, ptrs[-1], M, N, K, group_size, num_bits,
-                                                              conv, layout, rescale, stream)
+        if zwork is not None:
+            if lib.call_unpack_qzeros(z, ptrs[-1], N, groups, zfmt, stream) != 0:
+                return -1
+            z = ptrs[-1]
+        return lib.call_dequantize_gemv_lowbit(ptrs[0], ptrs[1], s, z, ptrs[c_idx], M, N, K, group_size, num_bits,
+                                               conv, layout, rescale, stream)
 
-    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error)
+    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error,
+                         workspace_idx=[-1] if zwork is not None else [])
 
 
 def dequantize_w4(
@@ -720,6 +754,23 @@ def matmul_nt_int4(M: int, N: int, K: int, block_M: int = 128, block_N: int = 12
         return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, 1, 1, 0, stream)
 
     return KernelAdapter("matmul_nt_int4", params, [-1], launch, _lib.last_error)
+
+
+def matmul_nt_int4xint2(M: int, N: int, K: int) -> KernelAdapter:
+    """int4 x 2-bit: ``C[M,N] int32 = sext4(A[M,K/2]) @ c(B[N,K/4]).T`` with the 2-bit codes taken unsigned, the
+    operand pair that decode_i2u_to_i4s / decode_i2s_to_i4s (examples/dequantize_gemm/quantize/lop3.py:1049-1089)
+    prepare for the int4 x int4 matrix instruction of examples/gemm_int4/example_tilelang_gemm_int4.py:17-38 (the
+    signed decoder's adjustment is commented out in the reference, so both decode to ``w = c``).
+    ``C = kernel(A_packed, B_packed)``."""
+    if K % 128 != 0:
+        raise ValueError(f"matmul_nt_int4xint2: K={K} must be a multiple of 128")
+    params = [KernelParam("A", torch.int8, (M, K // 2), packed=True), KernelParam("B", torch.int8, (N, K // 4), packed=True),
+              KernelParam("C", torch.int32, (M, N))]
+
+    def launch(ptrs, stream):
+        return _lib.get_library().call_gemm_int8xint4(ptrs[0], ptrs[1], ptrs[2], M, N, K, I2_TO_I4, 1, 0, stream)
+
+    return KernelAdapter("matmul_nt_int4xint2", params, [-1], launch, _lib.last_error)
 
 
 I2_UNSIGNED, I2_OFFSET, I2_TWOS = 0, 1, 2
