@@ -181,8 +181,9 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     if (rc <= 0) return rc;
     if (variant >= 40) DQ_FAIL("%s: the register-resident kernel does not cover M=%d N=%d K=%d group=%d", fn, M, N, K, group);
   }
-  if (variant < 0 && M > 16 && M <= 48) {
-    // measured at N = 28672, K = 8192: 11-18 % faster than the streaming kernel at M = 32 and 48, equal at M = 64
+  if (variant < 0 && M > 32 && M <= 48) {
+    // measured at N = 28672, K = 8192 with zero points: 45 us against the streaming kernel's 50 at M = 48; up to
+    // 32 rows the streaming kernel with its cheaper decoder is level or ahead (38.6 against 40.0 us), at 64 rows too
     const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, 1, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
