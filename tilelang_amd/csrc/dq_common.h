@@ -270,36 +270,37 @@ __device__ __forceinline__ uint4_t split_even_odd_bytes(uint4_t d) {
   return o;
 }
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float x) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+template <int CTRL, class T>
+__device__ __forceinline__ T dpp_move(T x) {
+  static_assert(sizeof(T) == 4, "one register");
+  return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
 }
 
-// Sums N per-lane values over each DPP row of 16 lanes at once.  While more than one value is
+// Sums N per-lane values (float or int) over each DPP row of 16 lanes at once.  While more than one value is
 // left, a level lets a lane keep the value its lane bit selects and add the partner lane's copy
 // of it, which halves the number of values; afterwards a level is a plain add.  Levels: xor 1,
 // xor 2 (quad_perm), rotate by 4, rotate by 8 (row_ror).  On return lane l holds the row total
 // of value (l & (N - 1)).  N values cost about 3 (N - 1) + 4 instructions instead of 4 N.
-template <int N, int LEVEL>
+template <int N, int LEVEL, class T = float>
 struct RowReduce {
-  static __device__ __forceinline__ float run(const float* v, int lane) {
+  static __device__ __forceinline__ T run(const T* v, int lane) {
     if constexpr (LEVEL == 4) {
       return v[0];
     } else {
       constexpr int kCtrl = LEVEL == 0 ? 0xB1 : (LEVEL == 1 ? 0x4E : (LEVEL == 2 ? 0x124 : 0x128));
       if constexpr (N == 1) {
-        const float t[1] = {v[0] + dpp_move<kCtrl>(v[0])};
-        return RowReduce<1, LEVEL + 1>::run(t, lane);
+        const T t[1] = {v[0] + dpp_move<kCtrl>(v[0])};
+        return RowReduce<1, LEVEL + 1, T>::run(t, lane);
       } else {
         const bool bit = (lane >> LEVEL) & 1;
-        float t[N / 2];
+        T t[N / 2];
 #pragma unroll
         for (int i = 0; i < N / 2; ++i) {
-          const float keep = bit ? v[2 * i + 1] : v[2 * i];
-          const float give = bit ? v[2 * i] : v[2 * i + 1];
+          const T keep = bit ? v[2 * i + 1] : v[2 * i];
+          const T give = bit ? v[2 * i] : v[2 * i + 1];
           t[i] = keep + dpp_move<kCtrl>(give);
         }
-        return RowReduce<N / 2, LEVEL + 1>::run(t, lane);
+        return RowReduce<N / 2, LEVEL + 1, T>::run(t, lane);
       }
     }
   }

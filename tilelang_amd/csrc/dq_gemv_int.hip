@@ -15,22 +15,14 @@
 //   * every decoder is  w = mul c' - zsub  with c' = c ^ flip:  sum a w = mul sum a c' - zsub sum a  (exact in
 //     integers).  Unsigned: (1, 0, 0).  Two's complement: sext(c) = (c ^ top) - top.  The signed fast decoders:
 //     c - 7 (four bits: the constant of decode_i4s_to_i8s), c - 2 (two bits), 2 c - 1 (one bit);
-//   * K is reduced over the lanes with DPP row operations and over the waves of a row through LDS; integer sums,
-//     so the result is exact whatever the order.
+//   * K is reduced over each 16-lane row with DPP row operations, all values of a batch of rows together (most levels
+//     halve the number of values), and over the 16-lane rows of a weight row through LDS; integer sums, so the result
+//     is exact whatever the order.
 #include "dq_common.h"
 
 namespace dq {
 
 namespace {
-
-__device__ __forceinline__ int wave_half_reduce_i32(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);   // quad_perm(1,0,3,2)
-  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);   // quad_perm(2,3,0,1)
-  v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);  // row_half_mirror
-  v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);  // row_mirror
-  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false); // row_bcast:15 -> lanes 31 / 63 hold 32-lane sums
-  return v;
-}
 
 constexpr int kMaxRowsPerWg = 128;
 
@@ -103,7 +95,10 @@ __global__ __launch_bounds__(256) void int_gemv_kernel(const int8_t* __restrict_
   constexpr int kDwords = kCodes / 4;      // activation dwords per chunk
   constexpr int kPerWord = 8 / BITS;       // dwords a 32-bit word of weights decodes into
   constexpr uint32_t kMask = BITS == 4 ? 0x0F0F0F0Fu : (BITS == 2 ? 0x03030303u : 0x01010101u);
-  __shared__ int red[kMaxRowsPerWg * 4 * MROWS];
+  constexpr int NV = R * MROWS;  // values reduced together per batch
+  static_assert(NV <= 16 && (NV & (NV - 1)) == 0, "a power of two of at most 16 values per lane row");
+  // partial sums: [batch][16-lane row of the workgroup (16)][value]
+  __shared__ int red[kMaxRowsPerWg * 16 * MROWS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -111,7 +106,6 @@ __global__ __launch_bounds__(256) void int_gemv_kernel(const int8_t* __restrict_
   const int rpp = 256 >> tpr_shift;
   const int slot = tid >> tpr_shift;
   const int ct = tid & (tpr - 1);
-  const int wave_in_row = ct >> 6;
   const int c16 = K / kCodes;  // 16-byte chunks per row
   const int rows_per_batch = R * rpp;
   const int rows_per_wg = nb * rows_per_batch;
@@ -151,8 +145,11 @@ __global__ __launch_bounds__(256) void int_gemv_kernel(const int8_t* __restrict_
     }
   }
 
+  const bool writer = (lane & 15) < NV;
+  int* red_w = red + (tid >> 4) * NV + (lane & (NV - 1));
+
   for (int b = 0; b < nb; ++b) {
-    int acc[R][MROWS];
+    int acc[NV];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       int dot[MROWS];
@@ -176,7 +173,7 @@ __global__ __launch_bounds__(256) void int_gemv_kernel(const int8_t* __restrict_
         int zs = 0;
 #pragma unroll
         for (int p = 0; p < NP; ++p) zs += asum[p][m];
-        acc[u][m] = mul * dot[m] - zsub * zs;
+        acc[u * MROWS + m] = mul * dot[m] - zsub * zs;
       }
     }
     // every row of the batch is consumed: refill all of them (wave-uniform branch)
@@ -184,27 +181,21 @@ __global__ __launch_bounds__(256) void int_gemv_kernel(const int8_t* __restrict_
 #pragma unroll
       for (int u = 0; u < R; ++u) issue_row(u, b + 1);
     }
-#pragma unroll
-    for (int u = 0; u < R; ++u) {
-      const int rl = b * rows_per_batch + u * rpp + slot;
-#pragma unroll
-      for (int m = 0; m < MROWS; ++m) {
-        int v = wave_half_reduce_i32(acc[u][m]);
-        if (tpr >= 64) {
-          v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31
-          if (lane == 63) red[(rl * 4 + wave_in_row) * MROWS + m] = v;
-        } else {
-          if ((lane & 31) == 31) red[(rl * 4 + 0) * MROWS + m] = v;
-        }
-      }
-    }
+    // the batch's R x MROWS values are summed over each 16-lane row together; lane l then holds value l % NV
+    const int v = RowReduce<NV, 0, int>::run(acc, lane);
+    if (writer) red_w[b * 16 * NV] = v;
   }
   __syncthreads();
-  const int waves_per_row = tpr >= 64 ? (tpr >> 6) : 1;
+
+  // ---- sum of the 16-lane partials of each output (integers: exact whatever the order) ----------------
+  const int parts = tpr >> 4;  // 16-lane rows per weight row
   for (int o = tid; o < rows_per_wg * MROWS; o += 256) {
     const int rl = o / MROWS, m = o - rl * MROWS;
-    int v = red[(rl * 4 + 0) * MROWS + m];
-    for (int w = 1; w < waves_per_row; ++w) v += red[(rl * 4 + w) * MROWS + m];
+    const int b = rl / rows_per_batch, within = rl - b * rows_per_batch;
+    const int u = within >> (8 - tpr_shift), sl = within & (rpp - 1);
+    const int* src = red + (b * 16 + sl * parts) * NV + u * MROWS + m;
+    int v = src[0];
+    for (int j = 1; j < parts; ++j) v += src[j * NV];
     const int row = row0 + rl;
     if (row < N && m < M) {
       if (out_kind == 0) {
