@@ -232,7 +232,7 @@ def test_w4a16_large_m_tile_exact_through_identity(cuda, mode, interleaved, N):
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384), (1500, 2000, 256), (3590, 3580, 128),
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (1, 256, 256), (130, 300, 384), (1500, 2000, 256), (1300, 4000, 256), (3590, 3580, 128),
                                    (3590, 3580, 768)])  # the last one: direct-to-LDS kernel
 @pytest.mark.parametrize("interleaved", [True, False])
 def test_bitnet_gemm_int32_exact(cuda, convention, M, N, K, interleaved):
@@ -286,10 +286,10 @@ def test_bitlinear_config5(cuda, M):
     np.testing.assert_array_equal(acc.cpu().numpy(), d["A"].astype(np.int64) @ d["W"].astype(np.int64).T)
 
 
-@pytest.mark.parametrize("M", [256, 2048])
+@pytest.mark.parametrize("M", [256, 1024, 2048])
 @pytest.mark.parametrize("interleaved", [True, False])
 def test_bitnet_full_size_exact(cuda, M, interleaved):
-    """Configuration 5 at full size (M in {256, 2048}, N = K = 8192), in the interleaved packing the benchmark
+    """Configuration 5 at full size (M in {256, 2048}, and 1024 for the small-tile kernel in between; N = K = 8192), in the interleaved packing the benchmark
     feeds and in the plain one: EVERY int32 entry against the integer oracle.  |A . w| <= 127 * 8192 < 2^24 and so
     is every partial sum, hence an fp32 BLAS matmul on the host gives the exact integers; a sample of entries is
     recomputed in int64 to pin that, and the fused BitLinear epilogue runs on the same inputs."""

@@ -66,6 +66,9 @@ def test_many_tiles(cuda, fmt, with_bias):
     _check(cuda, 3581, 3589, 128, fmt, scale_bias=127, with_bias=with_bias)
     _check(cuda, 3584, 3584, 320, fmt, scale_bias=0, with_bias=with_bias, exp_range=(0, 4))
     _check(cuda, 1500, 2000, 192, fmt, scale_bias=127, with_bias=with_bias)
+    # too few 256 x 256 tiles, 96 of 128 x 256: the direct-to-LDS kernel on its half-height tile (ragged both ways)
+    _check(cuda, 1500, 2000, 256, fmt, scale_bias=127, with_bias=with_bias)
+    _check(cuda, 1025, 3000, 384, fmt, scale_bias=127, with_bias=with_bias)
     if not with_bias:  # direct-to-LDS kernel with 4, 6 and 10 K tiles: prologue pair, steady pairs, tail
         for K in (256, 384, 640):
             _check(cuda, 3584, 3600, K, fmt, scale_bias=127)
@@ -129,7 +132,7 @@ def test_full_size_properties(cuda):
 # ---- bf16 x fp4 without block scales (the example with kernel(A, qB)) ------------------------------------------------
 
 @pytest.mark.parametrize("fast_dequant", [True, False])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (100, 300, 192), (512, 1024, 2048)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (100, 300, 192), (512, 1024, 2048), (1500, 2000, 256)])
 def test_unscaled_bf16_fp4(cuda, fast_dequant, M, N, K):
     """examples/dequantize_gemm/example_dequant_gemm_bf16_fp4_hopper.py: main(256, 256, 256, fast_dequant) against
     ref_program_twiddling / ref_program_simple, here the oracle's restatement of them (block exponent 0)."""

@@ -906,6 +906,22 @@ bool dma_eligible(const Params& p) {
   return P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
 }
 
+// Problems with too few 256 x 256 tiles for the kernel above but at least `min_tiles` tiles of 128 x 256: the same
+// kernel on the half-height tile (two workgroups fit a CU), which keeps the operands on the direct-to-LDS path.
+// Measured at N = K = 8192 against the register-staged 128 x 128 tiles, M = 1024: MXFP4 139 -> 114 us, fp16 x uint4
+// 213 -> 158 us, int8 x 2-bit 68 -> 57 us, int8 x int4 75 -> 60 us; M = 384 (96 tiles): MXFP4 90 -> 85.5 us, fp16 x
+// uint4 139 -> 117 us.  The int8 x 2-bit policy gains from 160 tiles on only (M = 512: 43.5 us register-staged
+// against 48.8 us; M = 640: 61 against 49 us).
+constexpr int kHalfTileMin = 96;
+template <class P>
+bool dma_half_eligible(const Params& p, int min_tiles = kHalfTileMin) {
+  const long tiles = (long)((p.M + 127) / 128) * ((p.N + BN - 1) / BN) * p.split;
+  const size_t a_bytes = (size_t)p.M * (p.ldk / P::kKPerBlock) * kARowBytes;
+  const size_t b_bytes = (size_t)p.N * (p.ldk / P::kKPerBlock) * P::kBRowBytes;
+  return !dma_eligible<P>(p) && P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= min_tiles &&
+         a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
+}
+
 template <class P, int kMBW, int kNBW>
 int launch_dma_tile(Params p, hipStream_t stream) {
   constexpr int kWaves = 16 / kNBW;
@@ -926,6 +942,20 @@ int launch_dma_tile(Params p, hipStream_t stream) {
 template <class P>
 int launch_dma(const Params& p, hipStream_t stream) {
   return launch_dma_tile<P, DQ_DMA_MBW, DQ_DMA_NBW>(p, stream);
+}
+
+template <class P>
+int launch_dma_half(const Params& p, hipStream_t stream) {
+  return launch_dma_tile<P, 2, 4>(p, stream);
+}
+
+// The tile choice of every policy that can take the direct-to-LDS path: 256 x 256 tiles there when the problem has
+// enough of them, else 128 x 256 tiles there, else the register-staged kernel with the tile size launch_auto picks.
+template <class P>
+int launch_best(const Params& p, hipStream_t stream, int half_tile_min = kHalfTileMin) {
+  if (dma_eligible<P>(p)) return launch_dma<P>(p, stream);
+  if (dma_half_eligible<P>(p, half_tile_min)) return launch_dma_half<P>(p, stream);
+  return launch_auto<P>(p, stream);
 }
 
 inline Params make_params(const void* A, const void* B, const void* S, const void* Z, const void* Bias, void* C, int M,

@@ -203,14 +203,10 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
                int scale_bias, hipStream_t stream) {
   Params p = gemm::make_params(A, B, S, nullptr, Bias, C, M, N, K);
   p.p0 = 127 - scale_bias;
-#define DQ_MX(FMT_)                                                                          \
-  do {                                                                                       \
-    if (gemm::dma_eligible<MxPolicy<FMT_, false>>(p)) {                                      \
-      if (Bias) return gemm::launch_dma<MxPolicy<FMT_, true>>(p, stream);                    \
-      return gemm::launch_dma<MxPolicy<FMT_, false>>(p, stream);                             \
-    }                                                                                        \
-    if (Bias) return gemm::launch_auto<MxPolicy<FMT_, true>>(p, stream);                          \
-    return gemm::launch_auto<MxPolicy<FMT_, false>>(p, stream);                                   \
+#define DQ_MX(FMT_)                                                        \
+  do {                                                                     \
+    if (Bias) return gemm::launch_best<MxPolicy<FMT_, true>>(p, stream);   \
+    return gemm::launch_best<MxPolicy<FMT_, false>>(p, stream);            \
   } while (0)
   switch (fmt) {
     case FP4_E2M1: DQ_MX(FP4_E2M1);
@@ -223,11 +219,7 @@ int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, vo
 
 int bf16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int fmt, hipStream_t stream) {
   Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
-#define DQ_F4(FMT_)                                                                                          \
-  do {                                                                                                       \
-    if (gemm::dma_eligible<Bf16Fp4Policy<FMT_>>(p)) return gemm::launch_dma<Bf16Fp4Policy<FMT_>>(p, stream); \
-    return gemm::launch_auto<Bf16Fp4Policy<FMT_>>(p, stream);                                                \
-  } while (0)
+#define DQ_F4(FMT_) return gemm::launch_best<Bf16Fp4Policy<FMT_>>(p, stream)
   switch (fmt) {
     case FP4_E2M1: DQ_F4(FP4_E2M1);
     case FP4_SIMPLE: DQ_F4(FP4_SIMPLE);
@@ -239,12 +231,8 @@ int bf16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, in
 
 int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream) {
   Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, C, M, N, K);
-  if (gemm::dma_eligible<Fp16Fp4Policy<true>>(p)) {
-    if (transposed) return gemm::launch_dma<Fp16Fp4Policy<true>>(p, stream);
-    return gemm::launch_dma<Fp16Fp4Policy<false>>(p, stream);
-  }
-  if (transposed) return gemm::launch_auto<Fp16Fp4Policy<true>>(p, stream);
-  return gemm::launch_auto<Fp16Fp4Policy<false>>(p, stream);
+  if (transposed) return gemm::launch_best<Fp16Fp4Policy<true>>(p, stream);
+  return gemm::launch_best<Fp16Fp4Policy<false>>(p, stream);
 }
 
 namespace {
@@ -276,12 +264,7 @@ int fp16_fp4_gemm_splitk(const void* A, const void* B, void* parts, void* C, int
   Params p = gemm::make_params(A, B, nullptr, nullptr, nullptr, parts, M, N, K / split);
   p.ldk = K;
   p.split = split;
-  int rc;
-  if (gemm::dma_eligible<Fp16Fp4Policy<true>>(p)) {
-    rc = transposed ? gemm::launch_dma<Fp16Fp4Policy<true>>(p, stream) : gemm::launch_dma<Fp16Fp4Policy<false>>(p, stream);
-  } else {
-    rc = transposed ? gemm::launch_auto<Fp16Fp4Policy<true>>(p, stream) : gemm::launch_auto<Fp16Fp4Policy<false>>(p, stream);
-  }
+  const int rc = transposed ? gemm::launch_best<Fp16Fp4Policy<true>>(p, stream) : gemm::launch_best<Fp16Fp4Policy<false>>(p, stream);
   if (rc) return rc;
   const size_t count = (size_t)M * N;
   // the partial results are 16-byte aligned slice by slice only when M x N is a multiple of 8
@@ -297,14 +280,10 @@ int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void
   Params p = gemm::make_params(A, B, S, Z, nullptr, C, M, N, K);
   p.p0 = (group == K) ? 31 : (31 - __builtin_clz(group));
   p.p1 = K / group;
-#define DQ_W4(MODE_)                                                                        \
-  do {                                                                                      \
-    if (layout == LAYOUT_PLAIN) {                                                           \
-      if (gemm::dma_eligible<W4F16Policy<MODE_, false>>(p)) return gemm::launch_dma<W4F16Policy<MODE_, false>>(p, stream); \
-      return gemm::launch_auto<W4F16Policy<MODE_, false>>(p, stream);                       \
-    }                                                                                       \
-    if (gemm::dma_eligible<W4F16Policy<MODE_, true>>(p)) return gemm::launch_dma<W4F16Policy<MODE_, true>>(p, stream); \
-    return gemm::launch_auto<W4F16Policy<MODE_, true>>(p, stream);                          \
+#define DQ_W4(MODE_)                                                                                \
+  do {                                                                                              \
+    if (layout == LAYOUT_PLAIN) return gemm::launch_best<W4F16Policy<MODE_, false>>(p, stream);     \
+    return gemm::launch_best<W4F16Policy<MODE_, true>>(p, stream);                                  \
   } while (0)
   switch (mode) {
     case W4_UNSIGNED: DQ_W4(W4_UNSIGNED);

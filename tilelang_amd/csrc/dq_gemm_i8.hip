@@ -178,14 +178,10 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int bitnet_epilogue, hipStream_t stream) {
   Params p = gemm::make_params(A, B, s_a, nullptr, nullptr, C, M, N, K);
   p.f0 = s_w;
-#define DQ_I2P(POL_BITNET_, POL_INT32_)                                                         \
-  do {                                                                                          \
-    if (gemm::dma_eligible<POL_BITNET_>(p)) {                                                   \
-      if (bitnet_epilogue) return gemm::launch_dma<POL_BITNET_>(p, stream);                     \
-      return gemm::launch_dma<POL_INT32_>(p, stream);                                           \
-    }                                                                                           \
-    if (bitnet_epilogue) return gemm::launch_auto<POL_BITNET_>(p, stream);                      \
-    return gemm::launch_auto<POL_INT32_>(p, stream);                                            \
+#define DQ_I2P(POL_BITNET_, POL_INT32_)                                            \
+  do {                                                                             \
+    if (bitnet_epilogue) return gemm::launch_best<POL_BITNET_>(p, stream, 160);    \
+    return gemm::launch_best<POL_INT32_>(p, stream, 160);                          \
   } while (0)
 #define DQ_I2L(CONV_, IL_)                                                                            \
   do {                                                                                                \
@@ -232,8 +228,7 @@ int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int deco
 #define DQ_I4(DEC_, SHIFT_, TRANS_)                                           \
   do {                                                                        \
     using Pol = I4Policy<DEC_, false, Int32Out<SHIFT_, TRANS_>>;              \
-    if (gemm::dma_eligible<Pol>(p)) return gemm::launch_dma<Pol>(p, stream);  \
-    return gemm::launch_auto<Pol>(p, stream);                                 \
+    return gemm::launch_best<Pol>(p, stream);                                 \
   } while (0)
 #define DQ_I4T(DEC_, SHIFT_)                  \
   do {                                        \
