@@ -66,8 +66,9 @@ enum dq_w4_layout {
                                instruction; its BitBLAS permutation inside a tile is third-party and not reproduced.
                                call_gemm_int8xint2 takes the flag too, with the order of the 32x32x32 int8 instruction:
                                B[(N+31)/32][K/128][64][16 bytes], entry 32 h + r of a 128-k chunk = bytes 16 h .. + 15
-                               of that chunk (32 bytes) of row r of the block of 32, rows past N zero; the K-sliced
-                               kernel is the one that reads it (K % 4096 == 0).                                      */
+                               of that chunk (32 bytes) of row r of the block of 32, rows past N zero; read by the
+                               decode kernel (M <= 4, M * K <= 32768), the K-sliced kernel (K % 4096 == 0) and the
+                               direct-to-LDS tiled kernel (from 160 tiles of 128 x 256 on).                          */
 };
 
 /* Flag for the `layout` of call_dequantize_w4 only: decode with the fp8-converter decoder (a nibble in a byte read as
@@ -204,7 +205,8 @@ enum dq_i2_convention {
  * Replaces `call(A, B, C, stream)` of tilelang_bitnet_158_int8xint2_prefill.py:188-296 and
  * tilelang_bitnet_158_int8xint2_decode.py:66-175.  Requires K % 128 == 0.
  * The library picks the kernel by shape (M <= 4: a streaming dot-product kernel; a few hundred rows on a long K:
- * K sliced over the waves of a workgroup; else the tiled GEMM).  For tests and measurements out_kind may carry one
+ * K sliced over the waves of a workgroup; else the tiled GEMM).  All three read DQ_LAYOUT_FRAGMENTS; where the
+ * tiled GEMM does not take a fragment-ordered problem (too few tiles) the K-sliced kernel runs it whatever its size.  For tests and measurements out_kind may carry one
  * of the flags below, which names the kernel instead; all kernels return the same bits. */
 enum dq_i2_kernel {
   DQ_I2_KERNEL_KSLICED = 16, /* needs K % 4096 == 0, K < 131072; -1 where it cannot run */

@@ -52,11 +52,11 @@ def test_bitlinear_forward(cuda, interleave, batch):
     np.testing.assert_allclose(out.float().cpu().numpy().reshape(-1, out_f), ref, rtol=1e-2, atol=1e-2)
 
 
-def test_bitlinear_layer_with_fragment_ordered_copy(cuda):
-    """``prefill_fragments=True``: the layer keeps a second, fragment-ordered copy of its weights and hands it to the
-    K-sliced kernel at the batch sizes that kernel serves (here 256 rows: 64 tiles), the row-major copy elsewhere
-    (8 rows); both layers must give the same bits at both sizes."""
-    in_f, out_f = 4096, 2048
+def test_bitlinear_layer_on_fragment_ordered_weights(cuda):
+    """``prefill_fragments=True``: the layer holds its weights in the matrix instruction's operand order ONLY (one
+    packed copy) and every batch size reads it: the decode kernel (1 and 4 rows), the K-sliced kernel (8 and 256 rows),
+    the tiled kernel (1300 rows); each must give the bits of the row-major layer."""
+    in_f, out_f = 4096, 4096
     rng = np.random.default_rng(11)
     W = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
     plain = tl.BitLinear(in_f, out_f)
@@ -64,31 +64,34 @@ def test_bitlinear_layer_with_fragment_ordered_copy(cuda):
     for layer in (plain, frag):
         layer.load_float_weight(torch.from_numpy(W))
         layer.to(cuda)
-    assert frag._takes_fragments(256) and not frag._takes_fragments(8) and not plain._takes_fragments(256)
-    for M in (256, 8):
+    assert frag.prefill_fragments and frag.qweight.shape == (out_f // 32, in_f // 128, 64, 16) and frag.qweight.is_cuda
+    assert plain.qweight.shape == (out_f, in_f // 4)
+    assert sum(b.numel() for b in frag.buffers()) == sum(b.numel() for b in plain.buffers())  # one copy, same bytes
+    assert torch.equal(frag.rowmajor_weight(), plain.qweight)
+    for M in (1, 4, 8, 256, 1300):
+        print(f"BitLinear on fragments: M={M}", flush=True)
         x = torch.from_numpy(rng.standard_normal((M, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
         a, b = plain(x), frag(x)
         torch.cuda.synchronize()
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
-    assert frag.qweight_fragments is not None and frag.qweight_fragments.is_cuda and plain.qweight_fragments is None
-    # weights replaced through the state dict: the fragment copy follows
+    # weights replaced through the state dict of another fragment-ordered layer
     W2 = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
-    plain.load_float_weight(torch.from_numpy(W2))
-    plain.to(cuda)
-    frag.load_state_dict(plain.state_dict())
-    assert frag._sw_value == plain._sw_value
+    other = tl.BitLinear(in_f, out_f, prefill_fragments=True)
+    other.load_float_weight(torch.from_numpy(W2))
+    other.to(cuda)
+    frag.load_state_dict(other.state_dict())
+    plain.load_packed_weight(other.rowmajor_weight(), other.sw)
+    assert frag._sw_value == plain._sw_value == other._sw_value
     x = torch.from_numpy(rng.standard_normal((256, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
     a, b = plain(x), frag(x)
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
-    assert not tl.BitLinear(1024, 768, prefill_fragments=True).prefill_fragments  # in_features the kernel cannot slice
+    assert not tl.BitLinear(1024, 768, prefill_fragments=True).prefill_fragments  # in_features the kernels cannot slice
 
 
-
-def test_bitlinear_decode_batches_stay_on_the_streaming_kernel(cuda):
-    """An 8192 x 8192 layer has 64 output tiles already at one row: a layer with the fragment-ordered copy must still
-    hand decode batches (M <= 4) the row-major words, which the streaming decode kernel reads, and give the plain
-    layer's bits."""
+def test_bitlinear_decode_batches_on_a_large_layer(cuda):
+    """An 8192 x 8192 layer on fragment-ordered weights at decode batches: the decode kernel reads the fragment order
+    (M * K <= 32768: one to four rows at K = 8192) and gives the plain layer's bits."""
     in_f = out_f = 8192
     rng = np.random.default_rng(13)
     W = (rng.standard_normal((out_f, in_f), dtype=np.float32) * 0.02).astype(np.float32)
@@ -97,8 +100,7 @@ def test_bitlinear_decode_batches_stay_on_the_streaming_kernel(cuda):
     for layer in (plain, frag):
         layer.load_float_weight(torch.from_numpy(W))
         layer.to(cuda)
-    assert not frag._takes_fragments(1) and not frag._takes_fragments(4) and frag._takes_fragments(5)
-    for M in (1, 4):
+    for M in (1, 2, 4):
         x = torch.from_numpy(rng.standard_normal((M, in_f), dtype=np.float32).astype(np.float16)).to(cuda)
         a, b = plain(x), frag(x)
         torch.cuda.synchronize()

@@ -377,12 +377,17 @@ def test_bitnet_k_sliced_kernel_exact(cuda, convention, M, N, K, interleaved):
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
-@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288)])
+@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288),
+                                   # decode kernel on fragments: one to four rows, one to eight blocks per wave, ragged N
+                                   (1, 128, 4096), (1, 1001, 8192), (2, 300, 16384), (3, 77, 8192), (4, 4100, 8192), (1, 40, 32768),
+                                   # direct-to-LDS tiled kernel on fragments: 256 x 256 and 128 x 256 tiles, ragged edges
+                                   (3590, 3580, 4096), (1300, 4000, 4096)])
 @pytest.mark.parametrize("interleaved", [True, False])
 def test_bitnet_fragment_ordered_weights_exact(cuda, convention, M, N, K, interleaved):
     """Weights re-ordered offline into the matrix instruction's operand order (``prepack_i2_fragments``; N ragged, so
-    the last block of 32 rows is padded): every int32 entry against the integer oracle, and the fused BitLinear
-    epilogue against the bits of the row-major path."""
+    the last block of 32 rows is padded) through whichever kernel the library picks for the shape (decode kernel,
+    K-sliced kernel, direct-to-LDS tiled kernel): every int32 entry against the integer oracle, and the fused
+    BitLinear epilogue against the bits of the row-major path."""
     rng = np.random.default_rng(M + K + 1)
     A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
     B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
@@ -397,23 +402,30 @@ def test_bitnet_fragment_ordered_weights_exact(cuda, convention, M, N, K, interl
     print(f"bitnet fragments: M={M} N={N} K={K} {convention} interleaved={interleaved}", flush=True)
     tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention=convention, weight_fragments=True)(_dev(A, cuda), Bfrag, C)
     out = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, weight_fragments=True)(_dev(A, cuda), Bfrag, s_a)
-    out_rows = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="ksliced")(_dev(A, cuda), Bdev, s_a)
+    out_rows = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved)(_dev(A, cuda), Bdev, s_a)
     torch.cuda.synchronize()
-    np.testing.assert_array_equal(C.cpu().numpy(), orc.ref_bitnet_int(A, B, convention))
+    # every product is at most 128 * 3 and every partial sum below 2^53 (2^24 when K * 384 < 2^24): a BLAS product in
+    # floating point is exact, whatever its summation order, and far faster than an int64 one
+    ft = np.float32 if K * 384 < (1 << 24) else np.float64
+    ref = (A.astype(ft) @ orc.decode_i2(B, convention).astype(ft).T).astype(np.int64)
+    rows, cols = np.arange(0, M, max(1, M // 7)), np.arange(0, N, max(1, N // 11))
+    np.testing.assert_array_equal(ref[np.ix_(rows, cols)], A[rows].astype(np.int64) @ orc.decode_i2(B[cols], convention).astype(np.int64).T)
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), ref)
     assert torch.equal(out.view(torch.int16), out_rows.view(torch.int16))
 
 
-def test_bitnet_fragment_ordered_weights_need_the_k_sliced_kernel(cuda):
-    """Through the C-ABI: a K the K-sliced kernel cannot slice, and the tiled kernel named together with the flag."""
+def test_bitnet_fragment_ordered_weights_where_no_kernel_reads_them(cuda):
+    """Through the C-ABI: a K that neither the K-sliced nor (for want of tiles) the tiled kernel takes, and the tiled
+    kernel named on a problem with too few tiles for it."""
     lib = tl._lib.get_library()
     A = torch.zeros((64, 2048), dtype=torch.int8, device=cuda)
-    B = torch.zeros((4, 16, 64, 16), dtype=torch.int8, device=cuda)
+    B = torch.zeros((4, 32, 64, 16), dtype=torch.int8, device=cuda)
     C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
     stream = torch.cuda.current_stream().cuda_stream
     assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 2048, 1, 2, None, 1.0, 0, stream) == -1
-    assert "K-sliced kernel needs" in tl._lib.last_error()
+    assert "no kernel takes" in tl._lib.last_error()
     assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 4096, 1, 2, None, 1.0, 32, stream) == -1
-    assert "K-sliced kernel only" in tl._lib.last_error()
+    assert "the tiled kernel reads fragment-ordered weights from" in tl._lib.last_error()
 
 
 def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):

@@ -333,6 +333,29 @@ def test_fragment_prepack_matches_the_oracle_and_inverts():
 
 
 
+def test_i2_fragment_addresses_of_the_decode_and_tiled_kernels():
+    """The byte offsets the decode kernel and the direct-to-LDS tiled kernel compute for fragment-ordered 2-bit
+    weights (block (nb, kb) at ((nb * K/128) + kb) * 1024, lane 32 h + r at + 16 lane) against the prepack itself:
+    lane (h, r) of block (nb, kb) must hold bytes 32 kb + 16 h .. + 15 of row 32 nb + r, for a ragged N."""
+    from tilelang_amd import quantize
+
+    N, K = 70, 1024
+    rng = np.random.default_rng(3)
+    B = torch.from_numpy(rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8))
+    flat = quantize.prepack_i2_fragments(B).reshape(-1).numpy()
+    KB, row_blocks = K // 128, (N + 31) // 32
+    for nb in range(row_blocks):
+        for kb in range(KB):
+            for lane in range(64):
+                h, r = lane >> 5, lane & 31
+                off = (nb * KB + kb) * 1024 + lane * 16  # dq_gemv_int.hip: issue(); dq_gemm_core.h: b_voff + kb * 1024
+                got = flat[off:off + 16]
+                row = 32 * nb + r
+                want = B[row, 32 * kb + 16 * h:32 * kb + 16 * h + 16].numpy() if row < N else np.zeros(16, np.uint8)
+                assert np.array_equal(got, want), (nb, kb, lane)
+    assert flat.size == row_blocks * KB * 1024
+
+
 def test_i2_fragment_prepack_matches_the_oracle_and_inverts():
     """quantize.prepack_i2_fragments against the oracle's index formula (N ragged: the last block of 32 rows is padded
     with zeros), its inverse, and the factories' shape rules."""
@@ -352,5 +375,5 @@ def test_i2_fragment_prepack_matches_the_oracle_and_inverts():
     assert tl.bitlinear_int8xint2(256, 128, 4096, 1.0, weight_fragments=True).params[1].shape == (4, 32, 64, 16)
     with pytest.raises(ValueError, match="K % 4096 == 0"):
         tl.bitnet_158_int8xint2_prefill(256, 128, 2048, weight_fragments=True)
-    with pytest.raises(ValueError, match="K-sliced kernel only"):
-        tl.bitlinear_int8xint2(256, 128, 4096, 1.0, kernel="tiled", weight_fragments=True)
+    # the tiled kernel may be named together with the flag: the library decides whether the problem has tiles enough
+    assert tl.bitlinear_int8xint2(256, 128, 4096, 1.0, kernel="tiled", weight_fragments=True).params[1].shape == (4, 32, 64, 16)

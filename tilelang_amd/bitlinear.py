@@ -36,10 +36,11 @@ class BitLinear(nn.Module):
 
     def __init__(self, in_features: int, out_features: int, weight_bits: int = 1, input_bits: int = 8, interleave: bool = True,
                  prefill_fragments: bool = False):
-        """``prefill_fragments``: keep a second copy of the packed weights in the matrix instruction's operand order
-        (``quantize.prepack_i2_fragments``, a quarter byte per weight more) and use it for the batch sizes that the
-        library runs on its K-sliced kernel (64 to 448 output tiles of 64 x 128; in_features a multiple of 4096), which
-        is about 12 % faster on that order.  Same results bit for bit."""
+        """``prefill_fragments``: hold the packed weights in the matrix instruction's operand order
+        (``quantize.prepack_i2_fragments``: ``[ceil(out/32), in/128, 64, 16]`` bytes) INSTEAD of row-major: one copy,
+        read at every batch size (decode kernel, K-sliced kernel, tiled kernel), about 10 % faster at a few hundred
+        rows.  Needs ``in_features % 4096 == 0``; otherwise the layer keeps the row-major words.  Same results bit for
+        bit."""
         super().__init__()
         if input_bits != 8:
             raise ValueError("BitLinear: only 8-bit activations are built")
@@ -49,9 +50,8 @@ class BitLinear(nn.Module):
         self.weight_bits, self.input_bits = weight_bits, input_bits
         self.interleave = interleave
         self.prefill_fragments = bool(prefill_fragments) and in_features % 4096 == 0 and in_features < 131072
-        self.qweight_fragments = None  # built on first use from qweight, rebuilt when qweight is replaced or moved
-        self._fragments_of = None
-        self.register_buffer("qweight", torch.zeros((out_features, in_features // 4), dtype=torch.int8))
+        shape = ((out_features + 31) // 32, in_features // 128, 64, 16) if self.prefill_fragments else (out_features, in_features // 4)
+        self.register_buffer("qweight", torch.zeros(shape, dtype=torch.int8))
         self.register_buffer("sw", torch.ones((), dtype=torch.float32))
         self._sw_value = 1.0
         self.bias = None
@@ -71,11 +71,25 @@ class BitLinear(nn.Module):
         packed = quantize.general_compress(codes.cpu(), source_bits=2)
         if self.interleave:
             packed = quantize.interleave_weight(packed, 2, "int8")
+        self.load_packed_weight(packed, sw, bias)
+
+    def load_packed_weight(self, packed_rowmajor: torch.Tensor, sw, bias: torch.Tensor | None = None) -> None:
+        """Row-major packed words ``[out, in/4]`` (interleaved or not, as the layer was built) and the weight scale;
+        stored in the layer's own order."""
+        packed = packed_rowmajor.contiguous()
+        if self.prefill_fragments:
+            packed = quantize.prepack_i2_fragments(packed)
         self.qweight = packed.to(self.qweight.device).contiguous()
-        self.sw = sw.to(torch.float32).to(self.sw.device)
+        self.sw = torch.as_tensor(sw, dtype=torch.float32).to(self.sw.device)
         self._sw_value = float(self.sw)
         self.bias = None if bias is None else bias.detach().to(self.qweight.device)
         self._kernels.clear()
+
+    def rowmajor_weight(self) -> torch.Tensor:
+        """The packed words ``[out, in/4]`` whatever order the layer holds them in."""
+        if self.prefill_fragments:
+            return quantize.unpack_i2_fragments(self.qweight, self.out_features)
+        return self.qweight
 
     def _load_from_state_dict(self, *args, **kwargs):
         super()._load_from_state_dict(*args, **kwargs)
@@ -83,32 +97,14 @@ class BitLinear(nn.Module):
         self._sw_value = float(self.sw)
         self._kernels.clear()
 
-    def _takes_fragments(self, M: int) -> bool:
-        # the shapes the library gives to the kernel that slices K over the waves (tiles of 64 x 128), in the order
-        # call_gemm_int8xint2 decides: up to four rows go to the streaming decode kernel first, which reads the
-        # row-major words only
-        if M <= 4:
-            return False
-        tiles = ((M + 63) // 64) * ((self.out_features + 127) // 128)
-        return self.prefill_fragments and 64 <= tiles <= 448
-
-    def _fragments(self) -> torch.Tensor:
-        """The fragment-ordered copy of ``qweight`` (not part of the state dict: it follows whatever ``qweight`` holds)."""
-        key = (self.qweight.data_ptr(), self.qweight._version, str(self.qweight.device))
-        if self._fragments_of != key:
-            self.qweight_fragments = quantize.prepack_i2_fragments(self.qweight)
-            self._fragments_of = key
-        return self.qweight_fragments
-
     def _get_kernels(self, M: int):
         k = self._kernels.get(M)
         if k is None:
             k = (kernels.bitnet_activation_quant(M, self.in_features),
                  kernels.bitlinear_int8xint2(M, self.out_features, self.in_features, self._sw_value, convention="offset",
-                                             interleaved=self.interleave, weight_fragments=self._takes_fragments(M)))
+                                             interleaved=self.interleave, weight_fragments=self.prefill_fragments))
             self._kernels[M] = k
         return k
-
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         x = input.reshape(-1, self.in_features)
@@ -116,7 +112,7 @@ class BitLinear(nn.Module):
             x = x.to(torch.float16)
         quant, gemm = self._get_kernels(x.shape[0])
         x_q, s_a = quant(x.contiguous())
-        out = gemm(x_q, self._fragments() if self._takes_fragments(x.shape[0]) else self.qweight, s_a)
+        out = gemm(x_q, self.qweight, s_a)
         if self.bias is not None:
             out += self.bias.view(1, -1).expand_as(out)
         return out.reshape(*input.shape[:-1], self.out_features)

@@ -369,20 +369,17 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   // bits 4 and 5 of out_kind name a kernel (tests and measurements): K sliced over the waves / the tiled GEMM
   int kernel_choice = out_kind & (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
   out_kind &= ~(DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
-  if (layout & LAYOUT_FRAGMENTS) {  // only the K-sliced kernel reads the fragment order
-    if (kernel_choice == DQ_I2_KERNEL_TILED) DQ_FAIL("%s: fragment-ordered weights are read by the K-sliced kernel only", fn);
-    kernel_choice = DQ_I2_KERNEL_KSLICED;
-  }
   if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
   if (kernel_choice == (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED)) DQ_FAIL("%s: out_kind names two kernels", fn);
   if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);
   if (out_kind == 1 && !(s_w != 0.f)) DQ_FAIL("%s: s_w must be non-zero", fn);
+  const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
   if (kernel_choice == DQ_I2_KERNEL_KSLICED) {
     const int rc = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 1, (hipStream_t)stream);
     if (rc > 0) DQ_FAIL("%s: the K-sliced kernel needs K %% 4096 == 0, K < 131072 and operands below 4 GiB (got M=%d N=%d K=%d)", fn, M, N, K);
     return rc;
   }
-  if (M <= 4 && !kernel_choice) {  // decode: the streaming dot4 kernel
+  if (M <= 4 && !kernel_choice) {  // decode: the streaming dot4 kernel (row-major or fragment-ordered weights)
     const int rc = i2_gemv(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
@@ -390,7 +387,17 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
     const int rc = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 0, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
-  return i2_gemm(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+  const int rc = i2_gemm(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+  if (rc <= 0 || !frag) return rc;
+  // Fragment-ordered weights are read by the decode kernel, the K-sliced kernel and the direct-to-LDS tiled kernel;
+  // a shape the tiled one does not take (too few tiles) goes to the K-sliced kernel whatever its size.
+  if (kernel_choice == DQ_I2_KERNEL_TILED)
+    DQ_FAIL("%s: the tiled kernel reads fragment-ordered weights from 160 tiles of 128 x 256 on and K %% 256 == 0 (got M=%d N=%d K=%d)", fn, M, N, K);
+  const int rck = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 1, (hipStream_t)stream);
+  if (rck > 0)
+    DQ_FAIL("%s: fragment-ordered weights: no kernel takes M=%d N=%d K=%d (decode: M <= 4 and M * K <= 32768; K-sliced: K %% 4096 == 0; "
+            "tiled: 160 tiles of 128 x 256 and K %% 256 == 0)", fn, M, N, K);
+  return rck;
 }
 
 extern "C" int call_bitnet_activation_quant(const void* X, void* Q, void* S, int M, int K, dq_stream_t stream) {

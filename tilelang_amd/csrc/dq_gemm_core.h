@@ -456,6 +456,15 @@ __global__ __launch_bounds__(kThreads * kKSplit, 1) void gemm_kernel(const Param
   }
 }
 
+// A policy may declare `static constexpr bool kBFragments = true`: its packed B was re-ordered offline into the
+// matrix instruction's operand order, B[(N + 31) / 32][K / kKPerBlock][64 lanes][16 bytes] (lane 32 h + r of a
+// block: bytes 16 h .. 16 h + 15 of that k-block of row r of the block of 32; 32-byte B rows only).  Read by the
+// direct-to-LDS kernel: a B load is then 1 KiB contiguous and lands in LDS as the operand it is.
+template <class P, class = void>
+struct BFragments : std::false_type {};
+template <class P>
+struct BFragments<P, std::void_t<decltype(P::kBFragments)>> : std::integral_constant<bool, P::kBFragments> {};
+
 // ---- direct-to-LDS variant ---------------------------------------------------------------------
 // For policies whose A needs no transform on its way to LDS (any per-fragment transform is P::fix_a,
 // applied after the fragment is read) and whose scales are absent, one byte per 32 k or one fp16 (plus
@@ -524,6 +533,8 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   constexpr int kRing = kPairB ? kStages * kAStage + 4 * kBStage : kStages * kStage;
   constexpr int kSOps = P::kScaleDma == 0 ? 0 : (P::kScaleDma == 3 ? 2 : 1);  // scale DMA instructions per wave per tile
   constexpr int kBWords = P::kBRowBytes / 8;   // dwords per lane and 32-row block: 4 or 8
+  constexpr bool kBFrag = BFragments<P>::value;
+  static_assert(!kBFrag || (P::kBRowBytes == 32 && kNBW == 4), "fragment-ordered B: 32-byte rows, four waves across the tile");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -553,6 +564,11 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     // LDS position (piece + rotation) % pieces holds source piece `piece`
     b_voff[i] = (unsigned)min(n0 + row, N - 1) * (unsigned)(p.ldk * P::kBRowBytes / P::kKPerBlock) +
                 (unsigned)(((pp - (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);
+    if constexpr (kBFrag) {
+      // instruction (wave, i) brings the 32-row block wave * kBOps + i of the tile: 1 KiB as stored, lane-linear
+      const int blk = min((n0 >> 5) + wave * kBOps + i, ((N + 31) >> 5) - 1);
+      b_voff[i] = (unsigned)blk * (unsigned)(p.ldk / P::kKPerBlock) * 1024u + (unsigned)lane * 16u;
+    }
   }
   const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(P::kScaleDma == 1 ? (K >> 5) : (K >> 6));  // waves 4..7 repeat 0..3
 
@@ -577,7 +593,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
       dma16(sbase + (wave * kAOps + i) * 1024, a_voff[i], (const unsigned char*)p.A + (size_t)kb * 128);
     } else {
       const int i = op - kSOps - kAOps;
-      dma16(bbase + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * P::kBRowBytes);
+      dma16(bbase + (wave * kBOps + i) * 1024, b_voff[i], (const unsigned char*)p.B + (size_t)kb * (kBFrag ? 1024 : P::kBRowBytes));
     }
   };
   constexpr int kWaitOps = kTileOps;  // outstanding DMA instructions of one tile
@@ -597,6 +613,8 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     for (int h = 0; h < kBPiecesPerRow / 2; ++h) {
       const int piece = g * (kBPiecesPerRow / 2) + h;
       b_off[nb][h] = row * P::kBRowBytes + (((piece + (row >> kBRot)) & (kBPiecesPerRow - 1)) << 4);  // in its B slot
+      // fragment order: block row / 32 of the tile, then the lanes as the matrix instruction numbers them
+      if constexpr (kBFrag) b_off[nb][h] = (row >> 5) * 1024 + lane * 16;
     }
     s_off[nb] = kRing + row * 4 + (P::kScaleDma == 1 ? g : 0);
   }

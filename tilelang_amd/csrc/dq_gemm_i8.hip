@@ -54,10 +54,13 @@ using BitnetOut = BitnetOutS<0>;
 // TOP (signed conventions, K < 131072): the codes are shifted to the top two bits of their byte instead, where the
 // int8 reading of the byte is 64 sext2(c) (offset binary: c - 2 = sext2(c ^ 2), the flip in the same three-input bit
 // operation as the mask): two instructions per dword instead of three, and the epilogue shifts the sum back by 6.
-template <int CONV, class EPI, bool INTERLEAVED, bool TOP = false>
+// FRAG: B re-ordered offline by prepack_i2_fragments (whole 16-byte pieces move, so the decode is the same); the
+// direct-to-LDS kernel only.
+template <int CONV, class EPI, bool INTERLEAVED, bool TOP = false, bool FRAG = false>
 struct I2Policy : I8Mfma, gemm::NoScale, EPI {
   static_assert(!TOP || CONV != I2_UNSIGNED, "unsigned codes are masked in place");
   static constexpr int kBRowBytes = 32;
+  static constexpr bool kBFragments = FRAG;
   static constexpr bool kAPacked = false;
   __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : transpose4x4_bytes(v); }
   __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
@@ -178,25 +181,50 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
             float s_w, int bitnet_epilogue, hipStream_t stream) {
   Params p = gemm::make_params(A, B, s_a, nullptr, nullptr, C, M, N, K);
   p.f0 = s_w;
+  // LAYOUT_FRAGMENTS: returns 1 where the direct-to-LDS kernel does not take the shape (no other tiled kernel reads
+  // that order)
+  const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
+  const int word_layout = layout & ~LAYOUT_FRAGMENTS;
 #define DQ_I2P(POL_BITNET_, POL_INT32_)                                            \
   do {                                                                             \
     if (bitnet_epilogue) return gemm::launch_best<POL_BITNET_>(p, stream, 160);    \
     return gemm::launch_best<POL_INT32_>(p, stream, 160);                          \
   } while (0)
+// fragment-ordered weights: the direct-to-LDS kernel on either tile height, or 1 (not this kernel's shape)
+#define DQ_I2F(POL_BITNET_, POL_INT32_)                                                                     \
+  do {                                                                                                      \
+    if (gemm::dma_eligible<POL_BITNET_>(p)) {                                                               \
+      if (bitnet_epilogue) return gemm::launch_dma<POL_BITNET_>(p, stream);                                 \
+      return gemm::launch_dma<POL_INT32_>(p, stream);                                                       \
+    }                                                                                                       \
+    if (gemm::dma_half_eligible<POL_BITNET_>(p, 160)) {                                                     \
+      if (bitnet_epilogue) return gemm::launch_dma_half<POL_BITNET_>(p, stream);                            \
+      return gemm::launch_dma_half<POL_INT32_>(p, stream);                                                  \
+    }                                                                                                       \
+    return 1;                                                                                               \
+  } while (0)
 #define DQ_I2L(CONV_, IL_)                                                                            \
   do {                                                                                                \
     using PlainB = I2Policy<CONV_, BitnetOut, IL_>;                                                   \
     using PlainI = I2Policy<CONV_, Int32Out<0, false>, IL_>;                                          \
+    using FragB = I2Policy<CONV_, BitnetOut, IL_, false, true>;                                       \
+    using FragI = I2Policy<CONV_, Int32Out<0, false>, IL_, false, true>;                              \
     if constexpr (CONV_ != I2_UNSIGNED) {                                                             \
       using TopB = I2Policy<CONV_, BitnetOutS<6>, IL_, true>;                                         \
       using TopI = I2Policy<CONV_, Int32Out<6, false>, IL_, true>;                                    \
-      if (K < 131072) DQ_I2P(TopB, TopI); /* 128 x 128 x K stays below 2^31 */                          \
+      using TopFragB = I2Policy<CONV_, BitnetOutS<6>, IL_, true, true>;                               \
+      using TopFragI = I2Policy<CONV_, Int32Out<6, false>, IL_, true, true>;                          \
+      if (K < 131072) { /* 128 x 128 x K stays below 2^31 */                                          \
+        if (frag) DQ_I2F(TopFragB, TopFragI);                                                         \
+        DQ_I2P(TopB, TopI);                                                                           \
+      }                                                                                               \
     }                                                                                                 \
+    if (frag) DQ_I2F(FragB, FragI);                                                                   \
     DQ_I2P(PlainB, PlainI);                                                                           \
   } while (0)
 #define DQ_I2(CONV_)                                        \
   do {                                                      \
-    if (layout == LAYOUT_INTERLEAVED) DQ_I2L(CONV_, true);  \
+    if (word_layout == LAYOUT_INTERLEAVED) DQ_I2L(CONV_, true);  \
     DQ_I2L(CONV_, false);                                   \
   } while (0)
   switch (convention) {
@@ -207,6 +235,7 @@ int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int conv
   }
 #undef DQ_I2
 #undef DQ_I2L
+#undef DQ_I2F
 #undef DQ_I2P
 }
 

@@ -264,6 +264,128 @@ int int_gemv(const void* A, const void* B, void* C, int M, int N, int K, Decoder
   return 1;
 }
 
+// ---- two-bit weights in fragment order (prepack_i2_fragments) ------------------------------------------------
+// B[(N + 31) / 32][K / 128][64 lanes][16 bytes]: lane 32 h + r of block (nb, kb) holds the 64 codes
+// k = 128 kb + 64 h .. + 63 of row 32 nb + r.  In that order the pieces of one K chunk of 32 consecutive rows are
+// contiguous, so here a wave instruction reads one block (1 KiB) and the rows run over the lanes: lane (h, r) adds up
+// row r's products over the wave's K blocks.  Its activations change from block to block, so they live in LDS, staged
+// once per workgroup in decoder order, and every read of them is a broadcast (the 32 lanes of a half share a chunk).
+// A workgroup is 16 waves; wave w takes blocks kb = w, w + 16, ... of a row block, the 32 partial sums of a row (16
+// waves x 2 halves) meet in LDS.  Integer sums: exact in any order.
+constexpr int kFragWaves = 16;
+constexpr int kFragActBytes = 32768;  // staged activations: MROWS * K bytes
+
+template <int MROWS, int NP>
+__global__ __launch_bounds__(64 * kFragWaves) void i2_gemv_frag_kernel(const int8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                                       void* __restrict__ C, const float* __restrict__ s_a,
+                                                                       float s_w, int out_kind, int M, int N, int K,
+                                                                       uint32_t flip_mask, int mul, int zsub, int interleaved) {
+  __shared__ __align__(16) int8_t act[kFragActBytes];
+  __shared__ int red[kFragWaves * 64 * MROWS];
+  __shared__ int asum[MROWS];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = lane >> 5;
+  const int KB = K >> 7;                 // blocks of 128 k per row
+  const int row_blocks = (N + 31) >> 5;
+
+  // ---- the first row block's weights go out before anything else ---------------------------------------------
+  uint4_t wq[NP];
+  auto issue = [&](int nb) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int kb = min(wave + kFragWaves * p, KB - 1);  // past the end: the last block again, unused
+      wq[p] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(B + ((size_t)nb * KB + kb) * 1024 + lane * 16));
+    }
+  };
+  int nb = blockIdx.x;
+  if (nb < row_blocks) issue(nb);
+
+  // ---- activations into LDS in decoder order, and their sums ---------------------------------------------------
+  if (tid < MROWS) asum[tid] = 0;
+  __syncthreads();
+  const int pieces = K >> 4;  // 16-byte pieces per activation row
+#pragma unroll
+  for (int m = 0; m < MROWS; ++m) {
+    const int8_t* ap = A + (size_t)min(m, M - 1) * K;
+    int s = 0;
+    for (int q = tid; q < pieces; q += 64 * kFragWaves) {
+      uint4_t d = *reinterpret_cast<const uint4_t*>(ap + q * 16);
+      if (!interleaved) d = transpose4x4_bytes(d);  // plain words decode to elements (i, 4 + i, 8 + i, 12 + i)
+      *reinterpret_cast<uint4_t*>(act + m * K + q * 16) = d;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s = __builtin_amdgcn_sdot4((int)d[i], 0x01010101, s, false);
+    }
+    const int one[1] = {s};
+    s = RowReduce<1, 0, int>::run(one, lane);
+    if ((lane & 15) == 0 && s != 0) atomicAdd(&asum[m], s);
+  }
+  __syncthreads();
+
+  for (; nb < row_blocks; nb += gridDim.x) {
+    int acc[MROWS];
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) acc[m] = 0;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int kb = wave + kFragWaves * p;
+      if (kb < KB) {  // wave-uniform
+        const int8_t* chunk = act + (2 * kb + h) * 64;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t w = wq[p][j] ^ flip_mask;
+          uint4_t a[MROWS];
+#pragma unroll
+          for (int m = 0; m < MROWS; ++m) a[m] = *reinterpret_cast<const uint4_t*>(chunk + m * K + j * 16);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int d = (int)((w >> (2 * i)) & 0x03030303u);
+#pragma unroll
+            for (int m = 0; m < MROWS; ++m) acc[m] = __builtin_amdgcn_sdot4((int)a[m][i], d, acc[m], false);
+          }
+        }
+      }
+    }
+    // the next row block's weights travel while this one's sums meet
+    const int nb_next = nb + gridDim.x;
+    if (nb_next < row_blocks) issue(nb_next);
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) red[(wave * 64 + lane) * MROWS + m] = acc[m];
+    __syncthreads();
+    if (tid < 32 * MROWS) {
+      const int r = tid / MROWS, m = tid - r * MROWS;
+      int v = 0;
+#pragma unroll
+      for (int w = 0; w < kFragWaves; ++w) v += red[(w * 64 + r) * MROWS + m] + red[(w * 64 + 32 + r) * MROWS + m];
+      v = mul * v - zsub * asum[m];
+      const int row = nb * 32 + r;
+      if (row < N && m < M) {
+        if (out_kind == 0) {
+          ((int32_t*)C)[(size_t)m * N + row] = v;
+        } else {
+          float f = (float)v;
+          f = f / s_a[m];
+          f = f / s_w;
+          ((half_t*)C)[(size_t)m * N + row] = (half_t)f;
+        }
+      }
+    }
+    __syncthreads();  // the sums are read: the next round may overwrite them
+  }
+}
+
+template <int MROWS, int NP>
+int launch_i2_gemv_frag(const void* A, const void* B, void* C, const void* s_a, float s_w, int out_kind, int M, int N, int K,
+                        Decoder dec, int interleaved, hipStream_t stream) {
+  const int row_blocks = (N + 31) / 32;
+  const int grid = row_blocks < 512 ? row_blocks : 512;
+  hipLaunchKernelGGL((i2_gemv_frag_kernel<MROWS, NP>), dim3(grid), dim3(64 * kFragWaves), 0, stream, (const int8_t*)A,
+                     (const uint8_t*)B, C, (const float*)s_a, s_w, out_kind, M, N, K, dec.flip, dec.mul, dec.zsub, interleaved);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 }  // namespace
 
 // Each returns 1 when the streaming kernel does not cover the shape (the caller then uses the MFMA GEMM): M <= 4,
@@ -275,7 +397,29 @@ int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int conv
   Decoder dec{0u, 1, 0};
   if (convention == I2_OFFSET) dec = Decoder{0u, 1, 2};
   else if (convention == I2_TWOS) dec = Decoder{0xAAAAAAAAu, 1, 2};  // sext2(c) = (c ^ 2) - 2
-  return int_gemv<2>(A, B, C, M, N, K, dec, layout == LAYOUT_INTERLEAVED, s_a, s_w, out_kind, stream);
+  const int interleaved = (layout & ~LAYOUT_FRAGMENTS) == LAYOUT_INTERLEAVED;
+  if (layout & LAYOUT_FRAGMENTS) {
+    // the activations of the batch stay in LDS; a wave walks up to eight blocks of 128 k
+    if (M < 1 || M > 4 || K % 128 != 0) return 1;
+    const int mrows = M == 1 ? 1 : (M == 2 ? 2 : 4);
+    const int np = ((K >> 7) + kFragWaves - 1) / kFragWaves;
+    if ((size_t)mrows * K > (size_t)kFragActBytes || np > 8) return 1;
+    if ((size_t)((N + 31) / 32) * (size_t)(K >> 7) * 1024 >= (1ull << 40)) return 1;
+#define DQ_GO(MR_, NP_) return launch_i2_gemv_frag<MR_, NP_>(A, B, C, s_a, s_w, out_kind, M, N, K, dec, interleaved, stream)
+#define DQ_NP(MR_)              \
+  do {                          \
+    if (np <= 1) DQ_GO(MR_, 1); \
+    if (np <= 2) DQ_GO(MR_, 2); \
+    if (np <= 4) DQ_GO(MR_, 4); \
+    DQ_GO(MR_, 8);              \
+  } while (0)
+    if (mrows == 1) DQ_NP(1);
+    if (mrows == 2) DQ_NP(2);
+    DQ_NP(4);
+#undef DQ_NP
+#undef DQ_GO
+  }
+  return int_gemv<2>(A, B, C, M, N, K, dec, interleaved, s_a, s_w, out_kind, stream);
 }
 
 // decode: the values of call_gemm_int8xint4 (0 unsigned nibbles, 1 two's complement, 2 / 3 the words of
