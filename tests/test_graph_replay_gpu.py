@@ -73,7 +73,7 @@ def test_graph_replays_match_eager(cuda):
 def test_graph_replays_match_eager_batch_kernels(cuda):
     """The K-sliced batch kernel (a voting barrier and 159 KiB of dynamic LDS), the register-resident kernel on
     fragment-ordered weights, the unscaled bf16 x fp4 GEMM and the K-sliced BitNet GEMM under capture."""
-    M1, N1, K1 = 32, 16 * 1400, 2048
+    M1, N1, K1 = 40, 16 * 1400, 2048
     d1 = workloads.w4a16(M1, N1, K1, 128, seed=5, zeros_range=(6, 10))
     ks = tl.dequantize_gemv(M1, N1, K1, group_size=128, source_format="uint", with_scaling=True, with_zeros=True)
     A1, B1, S1, Z1 = _dev(d1["A"], cuda), _dev(d1["B"], cuda).view(torch.int8), _dev(d1["Scale"], cuda), _dev(d1["Zeros"], cuda)
@@ -119,3 +119,71 @@ def test_graph_replays_match_eager_batch_kernels(cuda):
         torch.cuda.synchronize()
         for got, want in zip([C1, C2, c3_g, c5_g], eager):
             assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_graph_replays_match_eager_decode_and_half_tile_kernels(cuda):
+    """The integer decode GEMVs (4-bit and 1-bit weights; 2-bit weights in fragment order, whose kernel stages the
+    activations in LDS), the streaming batch kernel with the folded zero point, the direct-to-LDS GEMM on its
+    half-height tile (MXFP4) and on fragment-ordered BitNet weights, under capture."""
+    from tilelang_amd import quantize
+
+    rng = np.random.default_rng(21)
+    M1, N1, K1 = 2, 1000, 4096
+    A1 = _dev(rng.integers(-128, 128, size=(M1, K1), dtype=np.int8), cuda)
+    B1 = _dev(rng.integers(0, 256, size=(N1, K1 // 2), dtype=np.uint8), cuda).view(torch.int8)
+    g4 = tl.dequantize_gemv(M1, N1, K1, "int8", "int32", "int32", num_bits=4, source_format="int")
+    C1 = torch.empty((M1, N1), dtype=torch.int32, device=cuda)
+    B1b = _dev(rng.integers(0, 256, size=(N1, K1 // 8), dtype=np.uint8), cuda).view(torch.int8)
+    g1 = tl.dequantize_gemv(M1, N1, K1, "int8", "int32", "int32", num_bits=1, source_format="int", fast_decoding=True)
+    C1b = torch.empty((M1, N1), dtype=torch.int32, device=cuda)
+
+    M2, N2, K2 = 2, 1001, 8192
+    A2 = _dev(rng.integers(-128, 128, size=(M2, K2), dtype=np.int8), cuda)
+    B2 = quantize.prepack_i2_fragments(_dev(rng.integers(0, 256, size=(N2, K2 // 4), dtype=np.uint8), cuda).view(torch.int8))
+    gf = tl.bitnet_158_int8xint2_prefill(M2, N2, K2, fast_decoding=False, convention="offset", weight_fragments=True)
+    C2 = torch.empty((M2, N2), dtype=torch.int32, device=cuda)
+
+    M3, N3, K3 = 64, 300, 1536
+    d3 = workloads.w4a16(M3, N3, K3, 128, seed=9, zeros_range=(6, 10))
+    st = tl.dequantize_gemv(M3, N3, K3, group_size=128, source_format="uint", with_scaling=True, with_zeros=True)
+    A3, B3, S3, Z3 = _dev(d3["A"], cuda), _dev(d3["B"], cuda).view(torch.int8), _dev(d3["Scale"], cuda), _dev(d3["Zeros"], cuda)
+    C3 = torch.empty((M3, N3), dtype=torch.float16, device=cuda)
+
+    M4, N4, K4 = 1500, 2000, 256  # 96 tiles of 128 x 256
+    d4 = workloads.mxfp4(M4, N4, K4, seed=10, scale_bias=127)
+    mx = tl.matmul_bf16_mxfp4(M4, N4, K4, weight_format="e2m1", scale_bias=127)
+    A4, B4, S4 = _dev(d4["A"], cuda).view(torch.bfloat16), _dev(d4["B"], cuda), _dev(d4["Scale"], cuda)
+    bias = torch.empty((M4, N4), dtype=torch.bfloat16, device=cuda)
+
+    M5, N5, K5 = 1300, 4000, 4096  # 176 tiles of 128 x 256, fragment-ordered weights
+    A5 = _dev(rng.integers(-128, 128, size=(M5, K5), dtype=np.int8), cuda)
+    B5 = quantize.prepack_i2_fragments(_dev(rng.integers(0, 256, size=(N5, K5 // 4), dtype=np.uint8), cuda).view(torch.int8))
+    tf = tl.bitnet_158_int8xint2_prefill(M5, N5, K5, fast_decoding=True, convention="offset", weight_fragments=True)
+    C5 = torch.empty((M5, N5), dtype=torch.int32, device=cuda)
+
+    def run():
+        g4(A1, B1, C1)
+        g1(A1, B1b, C1b)
+        gf(A2, B2, C2)
+        st(A3, B3, S3, Z3, C3)
+        tf(A5, B5, C5)
+        return mx(A4, B4, S4, bias)
+
+    c4_e = run()
+    torch.cuda.synchronize()
+    outs = [C1, C1b, C2, C3, C5]
+    eager = [t.clone() for t in outs] + [c4_e.clone()]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            c4_g = run()
+    for _ in range(3):
+        for t in outs:
+            t.fill_(-7)
+        c4_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs + [c4_g], eager):
+            assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
