@@ -1,95 +1,12 @@
-// int8-MFMA policies of the LDS-staged dequantize GEMM (dq_gemm_core.h): BitNet W2A8
-// (int8 x 2-bit), W4A8 (int8 x int4), int4 x int4 and int8 x uint4.  Accumulation is int32 and
-// exact; the epilogue is either the raw int32 (optionally transposed) or BitLinear's
-// out = (float(acc) / s_a[m]) / s_w -> fp16.
-#include "dq_gemm_core.h"
+// int8 x 4-bit (W4A8, int8 x uint4), int4 x int4 and int4 x 2-bit policies of the LDS-staged dequantize GEMM: see
+// dq_gemm_i8.h for the matrix instruction and the epilogues.
+#include "dq_gemm_i8.h"
 
 namespace dq {
 
 namespace {
 
 using gemm::Params;
-
-struct I8Mfma {
-  static constexpr int kKPerBlock = 128;
-  using frag_t = int4_t;
-  using acc_t = int16_t_;
-  __device__ static __forceinline__ acc_t mfma(frag_t a, frag_t b, acc_t c) {
-    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-  }
-};
-
-// ---- epilogues --------------------------------------------------------------------------------------
-template <int SHIFT, bool TRANSPOSED>
-struct Int32Out {
-  static constexpr bool kTransposed = TRANSPOSED;
-  using out_t = int32_t;
-  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params&, int, int) {
-    return (int32_t)raw >> SHIFT;  // operands were decoded as 16 x value: exact
-  }
-};
-
-// BitLinear: out = (float(acc) / s_a[m]) / s_w -> fp16, two fp32 divides in that order
-// (examples/bitnet-1.58b/utils_quant.py:165-170).  p.S = s_a (float[M]), p.f0 = s_w.
-template <int SHIFT>
-struct BitnetOutS {
-  static constexpr bool kTransposed = false;
-  using out_t = half_t;
-  __device__ static __forceinline__ out_t finish(uint32_t raw, const Params& p, int m, int) {
-    float v = (float)((int32_t)raw >> SHIFT);  // operands decoded as 2^SHIFT x value: exact
-    v = v / ((const float*)p.S)[m];
-    v = v / p.f0;
-    return (half_t)v;
-  }
-};
-using BitnetOut = BitnetOutS<0>;
-
-// ---- int8 x 2-bit ---------------------------------------------------------------------------------
-// Plain layout: packed byte j of a row holds codes 4j..4j+3 at bits 0, 2, 4, 6; (w >> 2i) & 0x03030303
-// then yields elements (i, 4+i, 8+i, 12+i) of a 16-code word, and A is transposed to match.
-// INTERLEAVED: words pre-permuted by interleave_weight(qw, 2, "int8") (examples/bitnet-1.58b/
-// kernel_benchmark/tilelang_bitnet_158_int8xint2_decode.py:196-234: element e at byte e % 4, slot
-// e / 4), the layout the reference's kernels consume; the same shift-and-mask yields elements
-// 4i..4i+3 in natural order and A needs no transform.
-// TOP (signed conventions, K < 131072): the codes are shifted to the top two bits of their byte instead, where the
-// int8 reading of the byte is 64 sext2(c) (offset binary: c - 2 = sext2(c ^ 2), the flip in the same three-input bit
-// operation as the mask): two instructions per dword instead of three, and the epilogue shifts the sum back by 6.
-// FRAG: B re-ordered offline by prepack_i2_fragments (whole 16-byte pieces move, so the decode is the same); the
-// direct-to-LDS kernel only.
-template <int CONV, class EPI, bool INTERLEAVED, bool TOP = false, bool FRAG = false>
-struct I2Policy : I8Mfma, gemm::NoScale, EPI {
-  static_assert(!TOP || CONV != I2_UNSIGNED, "unsigned codes are masked in place");
-  static constexpr int kBRowBytes = 32;
-  static constexpr bool kBFragments = FRAG;
-  static constexpr bool kAPacked = false;
-  __device__ static __forceinline__ uint4_t stage_a(uint4_t v) { return INTERLEAVED ? v : transpose4x4_bytes(v); }
-  __device__ static __forceinline__ void expand_a(uint4_t, uint4_t&, uint4_t&) {}
-  // direct-to-LDS kernel: A lands in LDS untouched and each 16-byte fragment is transposed after the read
-  __device__ static __forceinline__ Scale prep_scale(int, const Params&) { return {}; }
-  using gemm::NoScale::prep_scale;
-  __device__ static __forceinline__ frag_t fix_a(frag_t f) {
-    return INTERLEAVED ? f : __builtin_bit_cast(frag_t, transpose4x4_bytes(__builtin_bit_cast(uint4_t, f)));
-  }
-  __device__ static __forceinline__ frag_t decode(const uint32_t* w, int j, const Scale&) {
-    frag_t o;
-    if constexpr (TOP) {
-      constexpr uint32_t flip = CONV == I2_OFFSET ? 0x80808080u : 0u;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = (int)(((w[j] << (6 - 2 * i)) & 0xC0C0C0C0u) ^ flip);
-      return o;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint32_t d = (w[j] >> (2 * i)) & 0x03030303u;
-      // each byte of d is a code 0..3: as the selector of v_perm_b32 it picks the code's int8 value out of a
-      // four-byte table (offset binary: c - 2; two's complement: sext2(c)), one instruction per dword
-      if constexpr (CONV == I2_OFFSET) d = __builtin_amdgcn_perm(0u, 0x0100FFFEu, d);
-      else if constexpr (CONV == I2_TWOS) d = __builtin_amdgcn_perm(0u, 0xFFFE0100u, d);
-      o[i] = (int)d;
-    }
-    return o;
-  }
-};
 
 // ---- int8 x 4-bit ---------------------------------------------------------------------------------
 // DEC = I4_TWOS: nibbles are two's complement; they are decoded as 16 x value (nibble in the top of the
@@ -176,68 +93,6 @@ struct I4xI2Policy : I8Mfma, gemm::NoScale, EPI {
 };
 
 }  // namespace
-
-int i2_gemm(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
-            float s_w, int bitnet_epilogue, hipStream_t stream) {
-  Params p = gemm::make_params(A, B, s_a, nullptr, nullptr, C, M, N, K);
-  p.f0 = s_w;
-  // LAYOUT_FRAGMENTS: returns 1 where the direct-to-LDS kernel does not take the shape (no other tiled kernel reads
-  // that order)
-  const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
-  const int word_layout = layout & ~LAYOUT_FRAGMENTS;
-#define DQ_I2P(POL_BITNET_, POL_INT32_)                                            \
-  do {                                                                             \
-    if (bitnet_epilogue) return gemm::launch_best<POL_BITNET_>(p, stream, 160);    \
-    return gemm::launch_best<POL_INT32_>(p, stream, 160);                          \
-  } while (0)
-// fragment-ordered weights: the direct-to-LDS kernel on either tile height, or 1 (not this kernel's shape)
-#define DQ_I2F(POL_BITNET_, POL_INT32_)                                                                     \
-  do {                                                                                                      \
-    if (gemm::dma_eligible<POL_BITNET_>(p)) {                                                               \
-      if (bitnet_epilogue) return gemm::launch_dma<POL_BITNET_>(p, stream);                                 \
-      return gemm::launch_dma<POL_INT32_>(p, stream);                                                       \
-    }                                                                                                       \
-    if (gemm::dma_half_eligible<POL_BITNET_>(p, 160)) {                                                     \
-      if (bitnet_epilogue) return gemm::launch_dma_half<POL_BITNET_>(p, stream);                            \
-      return gemm::launch_dma_half<POL_INT32_>(p, stream);                                                  \
-    }                                                                                                       \
-    return 1;                                                                                               \
-  } while (0)
-#define DQ_I2L(CONV_, IL_)                                                                            \
-  do {                                                                                                \
-    using PlainB = I2Policy<CONV_, BitnetOut, IL_>;                                                   \
-    using PlainI = I2Policy<CONV_, Int32Out<0, false>, IL_>;                                          \
-    using FragB = I2Policy<CONV_, BitnetOut, IL_, false, true>;                                       \
-    using FragI = I2Policy<CONV_, Int32Out<0, false>, IL_, false, true>;                              \
-    if constexpr (CONV_ != I2_UNSIGNED) {                                                             \
-      using TopB = I2Policy<CONV_, BitnetOutS<6>, IL_, true>;                                         \
-      using TopI = I2Policy<CONV_, Int32Out<6, false>, IL_, true>;                                    \
-      using TopFragB = I2Policy<CONV_, BitnetOutS<6>, IL_, true, true>;                               \
-      using TopFragI = I2Policy<CONV_, Int32Out<6, false>, IL_, true, true>;                          \
-      if (K < 131072) { /* 128 x 128 x K stays below 2^31 */                                          \
-        if (frag) DQ_I2F(TopFragB, TopFragI);                                                         \
-        DQ_I2P(TopB, TopI);                                                                           \
-      }                                                                                               \
-    }                                                                                                 \
-    if (frag) DQ_I2F(FragB, FragI);                                                                   \
-    DQ_I2P(PlainB, PlainI);                                                                           \
-  } while (0)
-#define DQ_I2(CONV_)                                        \
-  do {                                                      \
-    if (word_layout == LAYOUT_INTERLEAVED) DQ_I2L(CONV_, true);  \
-    DQ_I2L(CONV_, false);                                   \
-  } while (0)
-  switch (convention) {
-    case I2_UNSIGNED: DQ_I2(I2_UNSIGNED);
-    case I2_OFFSET: DQ_I2(I2_OFFSET);
-    case I2_TWOS: DQ_I2(I2_TWOS);
-    default: DQ_FAIL("int2 gemm: unknown code convention %d", convention);
-  }
-#undef DQ_I2
-#undef DQ_I2L
-#undef DQ_I2F
-#undef DQ_I2P
-}
 
 int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int decode, int a_packed, int transposed,
             hipStream_t stream) {
