@@ -498,20 +498,26 @@ __device__ __forceinline__ void dma4(unsigned lds_addr, unsigned voff, const voi
 // problem (410 us against 393 us), also a build option only (-DDQ_DMA_NBW=2).  Eight waves of 64 x 128
 // (four along the rows, which keeps the LDS traffic of the four-wave form) measured the same 410 us: a
 // second wave per SIMD does not buy MFMA issue slots here.
-template <class P, int kMBW, int kNBW>
-__global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel_dma(const Params p_in) {
+//
+// kWavesM = 1 (with kMBW = 8, kNBW = 2): the same 256 x 256 tile on four waves side by side, each 256 rows x 64
+// columns.  A wave then decodes only the 64 weight rows it alone multiplies (with two rows of waves every packed
+// word is decoded twice per workgroup) and reads every A fragment of the tile instead: half the decode
+// instructions, twice the LDS reads of A.  For policies whose decode keeps a lone wave's instruction issue busier
+// than its matrix pipe (P::kTallWaves).
+template <class P, int kMBW, int kNBW, int kWavesM = 2>
+__global__ __launch_bounds__(64 * kWavesM * (8 / kNBW), 32 * kMBW * kWavesM == 128 ? 2 : 1) void gemm_kernel_dma(const Params p_in) {
   Params p = p_in;
   int bid = blockIdx.x;
   take_k_slice<P>(p, bid);
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(P::kBRowBytes == 32 || P::kBRowBytes == 64, "direct-to-LDS variant: 32 or 64 packed bytes per weight row per tile");
-  static_assert(kMBW == 2 || kMBW == 4, "wave tile of 64 or 128 rows");
+  static_assert(kWavesM == 2 ? (kMBW == 2 || kMBW == 4) : (kWavesM == 1 && kMBW == 8 && kNBW == 2), "wave tile of 64, 128 or 256 rows");
   static_assert(kNBW == 2 || kNBW == 4, "wave tile of 64 or 128 columns");
   constexpr int kWavesN = 8 / kNBW;            // waves across the 256 tile columns
-  constexpr int kWaves = 2 * kWavesN;          // 4, or 8 (two per SIMD)
-  constexpr int BM = 64 * kMBW;                // shadows the 256-row default
+  constexpr int kWaves = kWavesM * kWavesN;    // 4, or 8 (two per SIMD)
+  constexpr int BM = 32 * kMBW * kWavesM;      // shadows the 256-row default
   constexpr int kAStage = BM * kARowBytes;     // 32 or 16 KiB
-  constexpr int kAOps = 8 * kMBW / kWaves;     // A DMA instructions per wave per tile
+  constexpr int kAOps = BM / 8 / kWaves;       // A DMA instructions per wave per tile
   constexpr int kBPiecesPerRow = P::kBRowBytes / 16;          // 2 or 4
   constexpr int kBRot = kBPiecesPerRow == 2 ? 3 : 2;          // piece rotation advances every 8 or 4 rows
   constexpr int kBOps = BN * kBPiecesPerRow / 64 / kWaves;    // packed-B DMA instructions per wave per tile
@@ -523,7 +529,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   // which halves the lines the B stream asks the L2 for.  Tile t + 1 then lands three iterations before it is
   // read, which takes a fourth B slot, so B gets a ring of its own behind the three A stages: kPairB.  Policies
   // with 64-byte rows keep A and B side by side in three stages (a fourth 16 KiB slot would not fit).
-  constexpr bool kPairB = P::kBRowBytes == 32 && kMBW == 4 && kNBW == 4;
+  constexpr bool kPairB = P::kBRowBytes == 32 && BM == 256 && kWaves == 4;
   constexpr int kBRing = kPairB ? kStages * kAStage : kAStage;       // where B of slot 0 starts
   constexpr int kBSlot = kPairB ? kBStage : kStage;                  // distance between B slots
   constexpr int kAStride = kPairB ? kAStage : kStage;                // distance between A stages
@@ -534,7 +540,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
   constexpr int kSOps = P::kScaleDma == 0 ? 0 : (P::kScaleDma == 3 ? 2 : 1);  // scale DMA instructions per wave per tile
   constexpr int kBWords = P::kBRowBytes / 8;   // dwords per lane and 32-row block: 4 or 8
   constexpr bool kBFrag = BFragments<P>::value;
-  static_assert(!kBFrag || (P::kBRowBytes == 32 && kNBW == 4), "fragment-ordered B: 32-byte rows, four waves across the tile");
+  static_assert(!kBFrag || (P::kBRowBytes == 32 && kWaves == 4), "fragment-ordered B: 32-byte rows, four waves");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -722,7 +728,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
     const unsigned char* base = smem + stage * kAStride;
     const unsigned char* bbase = smem + kBRing + (kPairB ? (kb & 3) : stage) * kBSlot;
     constexpr int kIterOps = !kPairB ? kTileOps : (odd ? kAOps : kSOps + kAOps + 2 * kBOps);  // issued per iteration
-    if constexpr (kMBW == 4 && kNBW == 4) {
+    if constexpr ((kMBW == 4 && kNBW == 4) || kWavesM == 1) {
       using DoMfma = std::integral_constant<bool, !first>;
       auto dma = [&](int chunk) {
         if constexpr (!kPairB) {
@@ -747,6 +753,72 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
         if constexpr (P::kScaleDma < 2) sc_c[nb] = P::prep_scale(sc_byte[nb], p);
       };
       auto nothing = [] {};
+      if constexpr (kWavesM == 1) {
+        // Eight matrix instructions (four A fragments against the wave's two B fragments) and their side work per
+        // scheduling region, as a pipeline of one matrix instruction, at most one LDS read and a few vector
+        // instructions.  Skewed by one step like the 2 x 2 form below.
+        constexpr int kValu = 3;
+        auto region = [&](int q0, auto do_mfma_tag, auto&& side) {
+          if constexpr (decltype(do_mfma_tag)::value) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int nb = 0; nb < 2; ++nb) acc[q0 + q][nb] = P::mfma(af_c[q0 + q], bf_c[nb], acc[q0 + q][nb]);
+          }
+          side();
+#define DQ_SPREAD_GROUP                                  \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     \
+  __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     \
+  __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+          DQ_SPREAD_GROUP DQ_SPREAD_GROUP DQ_SPREAD_GROUP DQ_SPREAD_GROUP
+          DQ_SPREAD_GROUP DQ_SPREAD_GROUP DQ_SPREAD_GROUP DQ_SPREAD_GROUP
+#undef DQ_SPREAD_GROUP
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        region(0, DoMfma{}, [&] {
+          fetch_b(0);
+          fetch_b(1);
+          dma(0);
+          dma(1);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) af_n[q] = read_a1(base, 0, q);
+        });
+        region(4, DoMfma{}, [&] {
+#pragma unroll
+          for (int q = 4; q < 8; ++q) af_n[q] = read_a1(base, 0, q);
+          finish_scale(0);
+          finish_scale(1);
+          dma(2);
+          dma(3);
+          bf_n[0] = P::decode(bw_c[0], 0, sc_c[0]);
+          bf_n[1] = P::decode(bw_c[1], 0, sc_c[1]);
+        });
+#pragma unroll
+        for (int q = 0; q < 8; ++q) af_c[q] = af_n[q];
+        bf_c[0] = bf_n[0];
+        bf_c[1] = bf_n[1];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          region(0, std::true_type{}, [&] {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) af_n[q] = read_a1(base, j + 1, q);
+            dma(4 + 4 * j);
+            dma(5 + 4 * j);
+            bf_n[0] = P::decode(bw_c[0], j + 1, sc_c[0]);
+          });
+          region(4, std::true_type{}, [&] {
+#pragma unroll
+            for (int q = 4; q < 8; ++q) af_n[q] = read_a1(base, j + 1, q);
+            dma(6 + 4 * j);
+            dma(7 + 4 * j);
+            bf_n[1] = P::decode(bw_c[1], j + 1, sc_c[1]);
+          });
+#pragma unroll
+          for (int q = 0; q < 8; ++q) af_c[q] = af_n[q];
+          bf_c[0] = bf_n[0];
+          bf_c[1] = bf_n[1];
+        }
+      } else {
       chunk4(0, DoMfma{}, [&] { fetch_b(0); fetch_b(1); }, [&] { dma(0); }, [&] { fetch_b(2); fetch_b(3); },
              [&] { af_n[0] = read_a1(base, 0, 0); });
       chunk4(1, DoMfma{}, [&] { af_n[1] = read_a1(base, 0, 1); finish_scale(0); }, [&] { dma(1); },
@@ -771,6 +843,7 @@ __global__ __launch_bounds__(64 * 16 / kNBW, kMBW == 2 ? 2 : 1) void gemm_kernel
           af_c[q] = af_n[q];
           bf_c[q] = bf_n[q];
         }
+      }
       }
     } else {
 #pragma unroll
@@ -940,16 +1013,17 @@ bool dma_half_eligible(const Params& p, int min_tiles = kHalfTileMin) {
          a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
 }
 
-template <class P, int kMBW, int kNBW>
+template <class P, int kMBW, int kNBW, int kWavesM = 2>
 int launch_dma_tile(Params p, hipStream_t stream) {
-  constexpr int kWaves = 16 / kNBW;
-  constexpr bool kPairB = P::kBRowBytes == 32 && kMBW == 4 && kNBW == 4;  // as in the kernel: a fourth B slot
-  constexpr int kPipe = 3 * (64 * kMBW * kARowBytes + BN * P::kBRowBytes) + (kPairB ? BN * P::kBRowBytes : 0) + 8 * 1024;
+  constexpr int kWaves = kWavesM * (8 / kNBW);
+  constexpr int kTileM = 32 * kMBW * kWavesM;
+  constexpr bool kPairB = P::kBRowBytes == 32 && kTileM == 256 && kWaves == 4;  // as in the kernel: a fourth B slot
+  constexpr int kPipe = 3 * (kTileM * kARowBytes + BN * P::kBRowBytes) + (kPairB ? BN * P::kBRowBytes : 0) + 8 * 1024;
   constexpr int kSlabs = kWaves * 32 * (32 * kNBW + 4) * 4;  // epilogue staging
   constexpr int kLds = kPipe > kSlabs ? kPipe : kSlabs;
-  p.tiles_m = (p.M + 64 * kMBW - 1) / (64 * kMBW);
+  p.tiles_m = (p.M + kTileM - 1) / kTileM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  auto kern = gemm_kernel_dma<P, kMBW, kNBW>;
+  auto kern = gemm_kernel_dma<P, kMBW, kNBW, kWavesM>;
   static bool lds_limit_raised[kMaxDevices];
   if (raise_lds_limit<kLds>(kern, lds_limit_raised)) return -1;
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n * p.split), dim3(64 * kWaves), kLds, stream, p);
@@ -957,9 +1031,16 @@ int launch_dma_tile(Params p, hipStream_t stream) {
   return 0;
 }
 
+// P::kTallWaves: the four waves side by side (see the kernel)
+template <class P, class = void>
+struct TallWaves : std::false_type {};
+template <class P>
+struct TallWaves<P, std::void_t<decltype(P::kTallWaves)>> : std::integral_constant<bool, P::kTallWaves> {};
+
 template <class P>
 int launch_dma(const Params& p, hipStream_t stream) {
-  return launch_dma_tile<P, DQ_DMA_MBW, DQ_DMA_NBW>(p, stream);
+  if constexpr (TallWaves<P>::value) return launch_dma_tile<P, 8, 2, 1>(p, stream);
+  else return launch_dma_tile<P, DQ_DMA_MBW, DQ_DMA_NBW>(p, stream);
 }
 
 template <class P>

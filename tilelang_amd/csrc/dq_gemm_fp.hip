@@ -160,6 +160,9 @@ struct W4F16Policy : F16Mfma {
   static constexpr int kBRowBytes = 32;
   static constexpr bool kTransposed = false;
   static constexpr bool kAPacked = false;
+  // 9 to 17 vector instructions per decoded operand: with two rows of waves a lone wave's instruction issue is
+  // busier than its matrix pipe (fp16 x uint4 at M = 4096, N = K = 8192: 467 us; 427 us with the waves side by side)
+  static constexpr bool kTallWaves = true;
   using out_t = half_t;
   struct ScaleRaw { half_t s, z; };
   struct Scale { half_t s, addend; };  // what the decoder multiplies by and adds (w4_cvt_addend)
