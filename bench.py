@@ -545,6 +545,18 @@ def main():
                          "frac": row["frac"], "us": row["us"], "kernel": "gemm_kernel_dma<MxPolicy<e2m1>,4,4>",
                          "workload": "A bf16 [4096,8192] x e2m1 [8192,8192] with e8m0 scales per 32, bf16 out",
                          "algorithmic_flops": 2 * 4096 * 8192 * 8192}
+    # What the matrix pipe sustains on random operands with nothing beside it, measured now on this device: the
+    # published peak assumes the top clock, which operands that toggle like real data do not hold.
+    from tilelang_amd import profiler as tl_profiler
+
+    sustained = {}
+    for dt in ("bfloat16", "float16", "int8"):
+        m = tl_profiler.mfma_sustained_rate(dt, device=dev)
+        sustained[dt] = {"T(FL)OP/s": m["ops_per_s"] / 1e12, "ms_per_launch": m["ms_per_launch"],
+                         "frac_of_published_peak": m["ops_per_s"] / (MFMA_I8_PEAK if dt == "int8" else MFMA_BF16_PEAK)}
+    if roof_gemm is not None:
+        roof_gemm["sustained_mfma_only"] = sustained["bfloat16"]["T(FL)OP/s"]
+        roof_gemm["frac_of_sustained"] = roof_gemm["achieved"] / sustained["bfloat16"]["T(FL)OP/s"]
     cpu = None
     if not args.no_cpu:
         # the CPU leg also looks at what was timed: a kernel that regressed to wrong results must not print a figure
@@ -575,6 +587,9 @@ def main():
                      f" after {head['timing']['settle_replays']} untimed replays (at least 50 ms)"},
         "roofline": roof,
         "roofline_gemm": roof_gemm,
+        "mfma_sustained": {"what": "call_mfma_rate: 16 matrix instructions of a 128 x 128 wave tile in a loop on random operands, one "
+                                   "workgroup of four waves per CU, no memory / LDS / decode work; median of 8 launches of about 5 ms "
+                                   "after 60 ms of untimed launches", **sustained},
         "cpu_baseline": cpu,
         "shapes": shapes,
     }

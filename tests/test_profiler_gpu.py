@@ -78,3 +78,25 @@ def test_explicit_stream_gets_its_own_outputs(cuda):
     for o in outs:
         assert torch.equal(o, expect)
     assert len({o.data_ptr() for o in outs}) == 4
+
+
+@pytest.mark.parametrize("dtype, peak", [("bfloat16", 2.5e15), ("float16", 2.5e15), ("int8", 5.0e15)])
+def test_mfma_sustained_rate_is_a_plausible_ceiling(cuda, dtype, peak):
+    """``call_mfma_rate`` through ``profiler.mfma_sustained_rate``: the matrix pipe alone, on random operands, runs at
+    a sizeable fraction of the published peak and never above it (the count of operations per launch is right)."""
+    m = profiler.mfma_sustained_rate(dtype, launch_ms=1.0, settle_ms=5.0, launches=3, device=cuda)
+    assert 0.35 * peak < m["ops_per_s"] < 1.02 * peak, m
+
+
+def test_mfma_rate_rejects_what_it_cannot_run(cuda):
+    from tilelang_amd import _lib
+
+    lib = _lib.get_library()
+    buf = torch.zeros(65536, dtype=torch.int8, device=cuda)
+    sink = torch.zeros(256, dtype=torch.float32, device=cuda)
+    assert lib.call_mfma_rate(buf.data_ptr(), sink.data_ptr(), 3, 1, 1, None) == -1
+    assert "in_dtype" in _lib.last_error()
+    assert lib.call_mfma_rate(None, sink.data_ptr(), 1, 1, 1, None) == -1
+    assert "non-NULL" in _lib.last_error()
+    assert lib.call_mfma_rate(buf.data_ptr(), sink.data_ptr(), 1, 0, 1, None) == -1
+    assert "workgroups" in _lib.last_error()

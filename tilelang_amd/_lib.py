@@ -42,6 +42,7 @@ SIGNATURES = {
     "call_gemm_int8xint4": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "call_gemv_int8xint1": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "call_gemm_plain": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "call_mfma_rate": [_vp, _vp, _i, _i, _i, _vp],
     "call_gemm_mxfp4_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
 }
 

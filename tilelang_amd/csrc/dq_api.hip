@@ -62,6 +62,7 @@ int i4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int deco
             hipStream_t stream);
 
 int unpack_qzeros(const void* QZ, void* Z, int N, int groups, int packed, hipStream_t stream);
+int mfma_rate(const void* operands, void* out, int dtype, int workgroups, int iters, hipStream_t stream);
 int plain_gemm(const void* A, const void* B, void* C, void* workspace, int M, int N, int K, int in_dtype, int out_dtype,
                int trans_A, int trans_B, hipStream_t stream);
 
@@ -450,6 +451,16 @@ extern "C" int call_gemm_plain(const void* A, const void* B, void* C, void* Work
   if ((trans_A || !trans_B) && !Workspace) DQ_FAIL("%s: Workspace is expected to have non-NULL data pointer when trans_A or not trans_B", fn);
   if (Workspace && !aligned16(Workspace)) DQ_FAIL("%s: Workspace must be 16-byte aligned", fn);
   return plain_gemm(A, B, C, Workspace, M, N, K, in_dtype, out_dtype, trans_A != 0, trans_B != 0, (hipStream_t)stream);
+}
+
+extern "C" int call_mfma_rate(const void* Operands, void* Out, int in_dtype, int workgroups, int iters, dq_stream_t stream) {
+  const char* fn = "call_mfma_rate";
+  if (!Operands || !Out) DQ_FAIL("%s: Operands and Out are expected to have non-NULL data pointers", fn);
+  if (!aligned16(Operands) || !aligned16(Out)) DQ_FAIL("%s: Operands and Out must be 16-byte aligned", fn);
+  if (in_dtype != DQ_DT_F16 && in_dtype != DQ_DT_BF16 && in_dtype != DQ_DT_I8)
+    DQ_FAIL("%s: in_dtype must be DQ_DT_F16, DQ_DT_BF16 or DQ_DT_I8 (got %d)", fn, in_dtype);
+  if (workgroups < 1 || workgroups > 65536 || iters < 1) DQ_FAIL("%s: workgroups=%d (1..65536) and iters=%d (>= 1) out of range", fn, workgroups, iters);
+  return mfma_rate(Operands, Out, in_dtype, workgroups, iters, (hipStream_t)stream);
 }
 
 extern "C" int call_gemm_int8xint4(const void* A, const void* B, void* C, int M, int N, int K, int decode,

@@ -269,3 +269,56 @@ class Profiler:
         ins = self._get_inputs() if input_tensors is None else input_tensors
         fn = (lambda: func(*ins)) if func is not None else (lambda: self.adapter(*ins))
         return do_bench(fn, warmup=warmup, rep=rep, **kw)
+
+
+_MFMA_RATE_DTYPES = {"float16": (0, 16), "bfloat16": (1, 16), "int8": (2, 32)}
+
+
+def mfma_sustained_rate(dtype: str = "bfloat16", launch_ms: float = 5.0, settle_ms: float = 60.0, launches: int = 8,
+                        device=None) -> dict:
+    """Operations per second the matrix pipe of the device sustains on random operands, with nothing else running
+    beside the matrix instructions (``call_mfma_rate``): one workgroup of four waves per compute unit, each issuing
+    the 16 instructions of a 128 x 128 wave tile over and over.  The published peak assumes the top clock; operands
+    that toggle like real data hold the chip at its power limit below it, so this is the rate a GEMM kernel on this
+    device can approach.  Untimed launches for ``settle_ms`` first (the clock settles), then the median of
+    ``launches`` launches of about ``launch_ms`` each, timed with events on the current stream.
+
+    No counterpart in the reference (its benchmarks quote the vendor's peak)."""
+    from . import _lib
+
+    code, k = _MFMA_RATE_DTYPES[dtype]
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        lib = _lib.get_library(dev.index)
+        gen = torch.Generator(device="cpu").manual_seed(0)
+        if dtype == "int8":
+            operands = torch.randint(-128, 128, (65536,), generator=gen, dtype=torch.int8).to(dev)
+        else:
+            operands = torch.randn(32768, generator=gen).to(getattr(torch, dtype)).to(dev)
+        workgroups = torch.cuda.get_device_properties(dev).multi_processor_count
+        sink = torch.empty(workgroups * 256, dtype=torch.float32, device=dev)
+        ops_per_iter = workgroups * 4 * 16 * 2 * 32 * 32 * k
+        stream = torch.cuda.current_stream(dev)
+
+        def launch(iters):
+            if lib.call_mfma_rate(operands.data_ptr(), sink.data_ptr(), code, workgroups, iters, stream.cuda_stream) != 0:
+                raise RuntimeError(_lib.last_error())
+
+        def timed(iters):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            launch(iters)
+            b.record(stream)
+            b.synchronize()
+            return a.elapsed_time(b)
+
+        iters = 2000
+        ms = timed(iters)
+        iters = max(1000, int(iters * launch_ms / max(ms, 1e-3)))
+        spent = 0.0
+        while spent < settle_ms:
+            spent += timed(iters)
+        times = sorted(timed(iters) for _ in range(launches))
+        ms = times[len(times) // 2]
+    return {"ops_per_s": ops_per_iter * iters / (ms * 1e-3), "ms_per_launch": ms, "iters": iters,
+            "workgroups": workgroups, "dtype": dtype}
