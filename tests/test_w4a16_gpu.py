@@ -215,7 +215,7 @@ def test_kernel_variants(cuda, variant):
     _run_gemv(cuda, 1, 1000, 2048 + 128, 128, "original", variant=variant)
 
 
-@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35, 36, 70, 72, 74, 76])
+@pytest.mark.parametrize("variant", [30, 31, 32, 33, 34, 35, 36, 37, 70, 72, 74, 76, 77])
 @pytest.mark.parametrize("mode", ["unsigned", "signed", "offset8", "scale", "uscale", "original", "rescale"])
 def test_streaming_small_batch_kernel(cuda, variant, mode):
     """The direct-to-LDS kernel: ragged M and N, a single K step, fewer steps than ring stages, many steps,
@@ -276,27 +276,15 @@ def test_register_resident_kernel(cuda, M, mode, variant):
     _run_gemv(cuda, M, 16 * 600, 2048, 128, mode, variant=variant)  # more row blocks than workgroups
 
 
-@pytest.mark.parametrize("mode", ["scale", "uscale", "original", "rescale"])
-@pytest.mark.parametrize("variant", [60, 61])
-def test_k_sliced_batch_kernel(cuda, variant, mode):
-    """17 to 64 rows with K sliced over the eight waves of one workgroup per CU (needs 1400 row blocks or more):
-    two, three and four blocks of activation rows, the smallest K (two slabs per K quarter) and a larger one, a last
-    workgroup with three of its seven row blocks, both layouts, and zero points that are not integers (those take
-    the copy of the loop that subtracts bias and zero point separately)."""
-    _run_gemv(cuda, 17, 16 * 1400, 2048, 128, mode, variant=variant)
-    _run_gemv(cuda, 64, 16 * 1403, 2048, 128, mode, variant=variant, interleaved=(mode in ("scale", "original")))
-    _run_gemv(cuda, 40, 16 * 1400, 3072, 128, mode, variant=variant, seed=3, zeros_offset=0.37)
-    if variant == 60 and mode == "original":
-        _run_gemv(cuda, 33, 16 * 1401, 4096, 128, mode, variant=variant, seed=4)
-
-
-@pytest.mark.parametrize("variant", [60, 61])
+@pytest.mark.parametrize("variant", [36, 37, 76, 77])
 @pytest.mark.parametrize("M", [48, 64])
-def test_k_sliced_batch_kernel_full_size(cuda, cfg3_full_size, M, variant):
-    """The K-sliced kernel at N = 28672, K = 8192 with (q - z) * s: every output against the oracle."""
+def test_streaming_small_batch_kernel_full_size(cuda, cfg3_full_size, M, variant):
+    """The eight-wave streaming kernel on three and on four blocks of activation rows at N = 28672, K = 8192 with
+    (q - z) * s, tile-exact (36, 37) and folded (76, 77); 64 rows on three blocks take two passes: every output
+    against the oracle."""
     d, W = cfg3_full_size
     N, K, group = 28672, 8192, 128
-    print(f"cfg3 full size, K-sliced kernel: M={M} variant={variant}", flush=True)
+    print(f"cfg3 full size, streaming kernel: M={M} variant={variant}", flush=True)
     kern = tl.dequantize_gemv(M, N, K, "float16", "float16", "float32", group_size=group, source_format="uint",
                               with_scaling=True, with_zeros=True, zeros_mode="original", variant=variant)
     C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
@@ -431,9 +419,9 @@ def cfg3_full_size():
     return d, W
 
 
-@pytest.mark.parametrize("M", [4, 16, 64])
+@pytest.mark.parametrize("M", [4, 16, 40, 64])
 def test_small_batch_full_size_default_dispatch(cuda, cfg3_full_size, M):
-    """Configuration 3 as the benchmark runs it: M in {4, 16, 64}, N = 28672, K = 8192, (q - z) * s with zeros 6..10,
+    """Configuration 3 as the benchmark runs it: M in {4, 16, 40, 64}, N = 28672, K = 8192, (q - z) * s with zeros 6..10,
     the library's own choice of kernel (variant = -1), every output against the oracle; and the kernel is linear in A."""
     d, W = cfg3_full_size
     N, K, group = 28672, 8192, 128

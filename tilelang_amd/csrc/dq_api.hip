@@ -26,8 +26,6 @@ int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, voi
                  int mode, int layout, int fast, hipStream_t stream);
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, hipStream_t stream);
-int w4a16_kslice(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
-                 int mode, int layout, int deep, hipStream_t stream);
 int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int variant, hipStream_t stream);
 int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
@@ -182,19 +180,7 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     if (rc <= 0) return rc;
     if (variant >= 40) DQ_FAIL("%s: the register-resident kernel does not cover M=%d N=%d K=%d group=%d", fn, M, N, K, group);
   }
-  if (variant < 0 && M > 32 && M <= 48) {
-    // measured at N = 28672, K = 8192 with zero points: 45 us against the streaming kernel's 50 at M = 48; up to
-    // 32 rows the streaming kernel with its cheaper decoder is level or ahead (38.6 against 40.0 us), at 64 rows too
-    const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, 1, (hipStream_t)stream);
-    if (rc <= 0) return rc;
-  }
-  if (variant == 60 || variant == 61) {
-    // 17 to 64 rows on a matrix with enough row blocks for every CU: K sliced over the waves of one workgroup per CU
-    const int rc = w4a16_kslice(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant - 60, (hipStream_t)stream);
-    if (rc > 0) DQ_FAIL("%s: the K-sliced batch kernel does not cover M=%d N=%d K=%d group=%d mode=%d", fn, M, N, K, group, mode);
-    return rc;
-  }
-  // 70..76: as 30..36 with the zero point folded into one fused multiply-add per weight pair (only "original"
+  // 70..77: as 30..37 with the zero point folded into one fused multiply-add per weight pair (only "original"
   // differs from the tile-exact form: RNE16(q s - RNE16(z s)) instead of RNE16(RNE16(q - z) s)); the default
   // above 16 rows
   const int folded_mode = mode == W4_ZEROS_ORIGINAL ? W4_ZEROS_FOLDED : mode;
@@ -217,7 +203,8 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   if (variant < 0 && M > 4) {
     // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
     const bool wide = N >= 128 * 200;
-    const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : 6);
+    // 33 to 48 rows: three blocks of 16 activation rows (40.9 us at N = 28672, K = 8192 against 45.3 us with four)
+    const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : (M <= 48 ? 7 : 6));
     const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, folded_mode, layout, config, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }

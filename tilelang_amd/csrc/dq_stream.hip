@@ -133,21 +133,27 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
     return smem + kRing + (g4 % kScaleSlots) * G::kScaleSlot + (step * 4 - scale_src_off(g4));
   };
 
-  auto issue_stage = [&](int step, int slot) {
+  // DMA instruction `op` of the stage of `step`, into ring slot `slot`: the weights, the activations, and (op == kOps,
+  // every fourth step) the scales / zeros of four steps
+  auto issue_op = [&](int op, int step, int slot) __attribute__((always_inline)) {
     const unsigned sb = lds0 + slot * G::kStage;
-#pragma unroll
-    for (int i = 0; i < kWOps; ++i) dma16(sb + (wave * kWOps + i) * 1024, w_voff[i], B + (size_t)step * (kStepK / 2));
-#pragma unroll
-    for (int i = 0; i < kAOps; ++i)
+    if (op < kWOps) {
+      dma16(sb + (wave * kWOps + op) * 1024, w_voff[op], B + (size_t)step * (kStepK / 2));
+    } else if (op < kOps) {
+      const int i = op - kWOps;
       dma16(sb + kWBytes + (wave * kAOps + i) * 1024, a_voff[i],
             reinterpret_cast<const unsigned char*>(A) + (size_t)step * (kStepK * 2));
-    if constexpr (kScale) {
+    } else if constexpr (kScale) {
       if ((step & 3) == 0) {
         const int g4 = step >> 2;
         dma16(lds0 + kRing + (g4 % kScaleSlots) * G::kScaleSlot + (wn >= 2 ? 2048 : 0) + (wn & 1) * 1024, s_voff,
               s_src + scale_src_off(g4));
       }
     }
+  };
+  auto issue_stage = [&](int step, int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int op = 0; op <= kOps; ++op) issue_op(op, step, slot);
   };
 
   // ---- fragment read offsets inside a stage (ui: the wave's ui-th half of a step) -----------------
@@ -201,12 +207,22 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   };
   // slots s_begin .. s_end-1 of a step whose stage is sb_cur; kCur: the step exists (false only
   // while the pipeline fills before step 0), kNext: so does the next one, staged at sb_nxt
+  // dma_tag: the slots also carry the DMA instructions of stage dma_step (ring slot dma_slot), which the barrier in
+  // front of slot kSub - 2 has released: kOpsPerSlot a slot, from that slot on round to slot kSub - 3 of the next
+  // step, so that all of them are out before the next step's wait and the waits count as if a stage went out at once
+  constexpr int kOpsPerSlot = (kOps + 1 + kSub - 1) / kSub;
   auto run_slots = [&](auto s_begin, auto s_end, const unsigned char* sb_cur, const unsigned char* sb_nxt, auto cur_tag,
-                       auto next_tag) {
-    constexpr bool kCur = decltype(cur_tag)::value, kNext = decltype(next_tag)::value;
+                       auto next_tag, auto dma_tag, int dma_step, int dma_slot) __attribute__((always_inline)) {
+    constexpr bool kCur = decltype(cur_tag)::value, kNext = decltype(next_tag)::value, kDma = decltype(dma_tag)::value;
 #pragma unroll
     for (int s = decltype(s_begin)::value; s < decltype(s_end)::value; ++s) {
       const int s2 = s + 2, s1 = s + 1;
+      if constexpr (kDma) {
+        const int rel = s >= kSub - 2 ? s - (kSub - 2) : s + 2;  // slots since the barrier that released the stage
+#pragma unroll
+        for (int o = 0; o < kOpsPerSlot; ++o)
+          if (rel * kOpsPerSlot + o <= kOps) issue_op(rel * kOpsPerSlot + o, dma_step, dma_slot);
+      }
       if (s2 < kSub) {  // R(t+2)
         if constexpr (kCur) {
 #pragma unroll
@@ -236,6 +252,19 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
           for (int mb = 0; mb < MB; ++mb)
             acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x_m[rb], y_m[mb], acc[rb][mb], 0, 0, 0);
       }
+#ifndef DQ_STREAM_SPREAD
+#define DQ_STREAM_SPREAD 4
+#endif
+      if constexpr (DQ_STREAM_SPREAD > 0) {
+        // one matrix instruction, at most one LDS read, a few vector instructions, RBW x MB times: left to itself
+        // the scheduler issues the slot's matrix instructions back to back and the decode in one piece
+#pragma unroll
+        for (int i = 0; i < RBW * MB; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, DQ_STREAM_SPREAD, 0);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb) x_m[rb] = x_d[rb];
@@ -264,29 +293,40 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   if (KS >= NST) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * kOps) : "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  run_slots(SlotNext{}, SlotEnd{}, smem, smem, std::false_type{}, std::true_type{});
+  using T = std::true_type;
+  using F = std::false_type;
+  run_slots(SlotNext{}, SlotEnd{}, smem, smem, F{}, T{}, F{}, 0, 0);
   next_weights_become_current();
 
   // Step `step` multiplies out of slot step % NST.  Before its last two slots the next stage must
   // have landed: the stages younger than it are the NST - 2 issued last (kWaitOps instructions), or, in
   // the tail where fewer are in flight, the wave simply drains its counter.  After the barrier no wave
   // reads stage `step` any more (the barrier also waits for the LDS reads in flight), so the DMA of
-  // step + NST goes there.
+  // step + NST goes there: spread over the slots from there to the next step's wait.
   int slot = 0;
-  for (int step = 0; step + 1 < KS; ++step) {
+  auto one_step = [&](int step, auto dma_before_tag, auto dma_after_tag) __attribute__((always_inline)) {
     const int slot1 = slot + 1 == NST ? 0 : slot + 1;
+    const int slot_prev = slot == 0 ? NST - 1 : slot - 1;
     const unsigned char* sb_cur = smem + slot * G::kStage;
-    run_slots(SlotFirst{}, SlotNext{}, sb_cur, sb_cur, std::true_type{}, std::true_type{});
+    run_slots(SlotFirst{}, SlotNext{}, sb_cur, sb_cur, T{}, T{}, dma_before_tag, step - 1 + NST, slot_prev);
     if (step + NST - 1 < KS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWaitOps) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (step + NST < KS) issue_stage(step + NST, slot);
     sc_nxt = scale_base(step + 1);
-    run_slots(SlotNext{}, SlotEnd{}, sb_cur, smem + slot1 * G::kStage, std::true_type{}, std::true_type{});
+    run_slots(SlotNext{}, SlotEnd{}, sb_cur, smem + slot1 * G::kStage, T{}, T{}, dma_after_tag, step + NST, slot);
     next_weights_become_current();
     slot = slot1;
+  };
+  // steps whose stage step + NST exists; then the tail, which only finishes the stage begun in the step before it
+  int step = 0;
+  if (KS > NST) {
+    one_step(0, F{}, T{});
+    for (step = 1; step + NST < KS; ++step) one_step(step, T{}, T{});
+    one_step(step, T{}, F{});
+    ++step;
   }
-  run_slots(SlotFirst{}, SlotEnd{}, smem + slot * G::kStage, smem, std::true_type{}, std::false_type{});
+  for (; step + 1 < KS; ++step) one_step(step, F{}, F{});
+  run_slots(SlotFirst{}, SlotEnd{}, smem + slot * G::kStage, smem, T{}, F{}, F{}, 0, 0);
 
   if constexpr (KSPLIT == 2) {
     // waves 4..7 hand their half of the K sum to waves 0..3: [wn][rb][mb][lane] float4
@@ -391,6 +431,7 @@ int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, voi
     case 4: return launch_stream<2, 1, 3, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
     case 5: return launch_stream<1, 1, 6, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
     case 6: return launch_stream<4, 2, 3, 2>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 7: return launch_stream<3, 2, 3, 2>(A, B, S, Z, C, M, N, K, mode, layout, stream);
     default: DQ_FAIL("w4a16 stream kernel: unknown configuration %d", config);
   }
 }
