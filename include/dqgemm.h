@@ -67,7 +67,7 @@ enum dq_w4_layout {
                                call_gemm_int8xint2 takes the flag too, with the order of the 32x32x32 int8 instruction:
                                B[(N+31)/32][K/128][64][16 bytes], entry 32 h + r of a 128-k chunk = bytes 16 h .. + 15
                                of that chunk (32 bytes) of row r of the block of 32, rows past N zero; read by the
-                               decode kernel (M <= 4, M * K <= 32768), the K-sliced kernel (K % 4096 == 0) and the
+                               decode kernel (M <= 4, M * K <= 32768), the K-sliced kernel (K % 2048 == 0) and the
                                direct-to-LDS tiled kernel (from 160 tiles of 128 x 256 on).                          */
 };
 
@@ -209,7 +209,7 @@ enum dq_i2_convention {
  * tiled GEMM does not take a fragment-ordered problem (too few tiles) the K-sliced kernel runs it whatever its size.  For tests and measurements out_kind may carry one
  * of the flags below, which names the kernel instead; all kernels return the same bits. */
 enum dq_i2_kernel {
-  DQ_I2_KERNEL_KSLICED = 16, /* needs K % 4096 == 0, K < 131072; -1 where it cannot run */
+  DQ_I2_KERNEL_KSLICED = 16, /* needs K % 2048 == 0, K < 131072; -1 where it cannot run */
   DQ_I2_KERNEL_TILED = 32
 };
 int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout,

@@ -353,7 +353,9 @@ def test_bitnet_decode_full_size(cuda):
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
-@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288), (1, 8, 4096)])
+@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288), (1, 8, 4096),
+                                   # an odd number of block pairs per wave: one, three, seven
+                                   (64, 130, 2048), (100, 257, 6144), (33, 128, 14336)])
 @pytest.mark.parametrize("interleaved", [True, False])
 def test_bitnet_k_sliced_kernel_exact(cuda, convention, M, N, K, interleaved):
     """The kernel that slices K over the waves of a workgroup (the library's choice at a few hundred rows), named
@@ -377,7 +379,7 @@ def test_bitnet_k_sliced_kernel_exact(cuda, convention, M, N, K, interleaved):
 
 
 @pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
-@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288),
+@pytest.mark.parametrize("M,N,K", [(64, 128, 4096), (130, 300, 4096), (256, 384, 8192), (70, 1001, 12288), (90, 200, 6144),
                                    # decode kernel on fragments: one to four rows, one to eight blocks per wave, ragged N
                                    (1, 128, 4096), (1, 1001, 8192), (2, 300, 16384), (3, 77, 8192), (4, 4100, 8192), (1, 40, 32768),
                                    # direct-to-LDS tiled kernel on fragments: 256 x 256 and 128 x 256 tiles, ragged edges
@@ -418,22 +420,22 @@ def test_bitnet_fragment_ordered_weights_where_no_kernel_reads_them(cuda):
     """Through the C-ABI: a K that neither the K-sliced nor (for want of tiles) the tiled kernel takes, and the tiled
     kernel named on a problem with too few tiles for it."""
     lib = tl._lib.get_library()
-    A = torch.zeros((64, 2048), dtype=torch.int8, device=cuda)
+    A = torch.zeros((64, 4096), dtype=torch.int8, device=cuda)
     B = torch.zeros((4, 32, 64, 16), dtype=torch.int8, device=cuda)
     C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
     stream = torch.cuda.current_stream().cuda_stream
-    assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 2048, 1, 2, None, 1.0, 0, stream) == -1
+    assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 1024, 1, 2, None, 1.0, 0, stream) == -1
     assert "no kernel takes" in tl._lib.last_error()
     assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 4096, 1, 2, None, 1.0, 32, stream) == -1
     assert "the tiled kernel reads fragment-ordered weights from" in tl._lib.last_error()
 
 
 def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):
-    A = torch.zeros((64, 2048), dtype=torch.int8, device=cuda)
-    B = torch.zeros((128, 512), dtype=torch.int8, device=cuda)
+    A = torch.zeros((64, 1024), dtype=torch.int8, device=cuda)
+    B = torch.zeros((128, 256), dtype=torch.int8, device=cuda)
     C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
     with pytest.raises(RuntimeError, match="K-sliced kernel needs"):
-        tl.bitnet_158_int8xint2_prefill(64, 128, 2048, convention="offset", kernel="ksliced")(A, B, C)
+        tl.bitnet_158_int8xint2_prefill(64, 128, 1024, convention="offset", kernel="ksliced")(A, B, C)
 
 
 @pytest.mark.parametrize("interleaved", [True, False])

@@ -39,7 +39,7 @@ class BitLinear(nn.Module):
         """``prefill_fragments``: hold the packed weights in the matrix instruction's operand order
         (``quantize.prepack_i2_fragments``: ``[ceil(out/32), in/128, 64, 16]`` bytes) INSTEAD of row-major: one copy,
         read at every batch size (decode kernel, K-sliced kernel, tiled kernel), about 10 % faster at a few hundred
-        rows.  Needs ``in_features % 4096 == 0``; otherwise the layer keeps the row-major words.  Same results bit for
+        rows.  Needs ``in_features % 2048 == 0``; otherwise the layer keeps the row-major words.  Same results bit for
         bit."""
         super().__init__()
         if input_bits != 8:
@@ -49,7 +49,7 @@ class BitLinear(nn.Module):
         self.in_features, self.out_features = in_features, out_features
         self.weight_bits, self.input_bits = weight_bits, input_bits
         self.interleave = interleave
-        self.prefill_fragments = bool(prefill_fragments) and in_features % 4096 == 0 and in_features < 131072
+        self.prefill_fragments = bool(prefill_fragments) and in_features % 2048 == 0 and in_features < 131072
         shape = ((out_features + 31) // 32, in_features // 128, 64, 16) if self.prefill_fragments else (out_features, in_features // 4)
         self.register_buffer("qweight", torch.zeros(shape, dtype=torch.int8))
         self.register_buffer("sw", torch.ones((), dtype=torch.float32))

@@ -364,7 +364,7 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
   if (kernel_choice == DQ_I2_KERNEL_KSLICED) {
     const int rc = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 1, (hipStream_t)stream);
-    if (rc > 0) DQ_FAIL("%s: the K-sliced kernel needs K %% 4096 == 0, K < 131072 and operands below 4 GiB (got M=%d N=%d K=%d)", fn, M, N, K);
+    if (rc > 0) DQ_FAIL("%s: the K-sliced kernel needs K %% 2048 == 0, K < 131072 and operands below 4 GiB (got M=%d N=%d K=%d)", fn, M, N, K);
     return rc;
   }
   if (M <= 4 && !kernel_choice) {  // decode: the streaming dot4 kernel (row-major or fragment-ordered weights)
@@ -383,7 +383,7 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
     DQ_FAIL("%s: the tiled kernel reads fragment-ordered weights from 160 tiles of 128 x 256 on and K %% 256 == 0 (got M=%d N=%d K=%d)", fn, M, N, K);
   const int rck = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 1, (hipStream_t)stream);
   if (rck > 0)
-    DQ_FAIL("%s: fragment-ordered weights: no kernel takes M=%d N=%d K=%d (decode: M <= 4 and M * K <= 32768; K-sliced: K %% 4096 == 0; "
+    DQ_FAIL("%s: fragment-ordered weights: no kernel takes M=%d N=%d K=%d (decode: M <= 4 and M * K <= 32768; K-sliced: K %% 2048 == 0; "
             "tiled: 160 tiles of 128 x 256 and K %% 256 == 0)", fn, M, N, K);
   return rck;
 }

@@ -235,10 +235,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
   for (int i = 0; i < kAOps; ++i) load_a(1, i);
   static_for<kNB>([&](auto nb) { load_w(std::integral_constant<int, 1>{}, std::integral_constant<int, 2 * decltype(nb)::value>{}, 1); });
 
-  for (int p0 = 0; p0 < npair; p0 += 2) {
-    static_for<2>([&](auto q_tag) {
+  // pair `pair` of blocks out of the weight registers w_raw[q], q = pair % 2
+  auto do_pair = [&](auto q_tag, int pair) __attribute__((always_inline)) {
       constexpr int q = decltype(q_tag)::value;
-      const int pair = p0 + q;
       static_for<2>([&](auto b_tag) {
         constexpr int b = decltype(b_tag)::value;
         const int t = 2 * pair + b;
@@ -273,7 +272,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t*
           }
         });
       });
-    });
+  };
+  for (int p0 = 0; p0 < npair; p0 += 2) {
+    do_pair(std::integral_constant<int, 0>{}, p0);
+    if (p0 + 1 < npair) do_pair(std::integral_constant<int, 1>{}, p0 + 1);  // an odd number of pairs: K % 4096 == 2048
   }
   // The loads past the end of the slice still write the stages and their registers.
   wait_loads<0>(w_raw);
@@ -350,8 +352,8 @@ int launch_i2_kslice(const void* A, const void* B, void* C, int M, int N, int K,
 // force: take every shape the kernel can compute, whether or not it is expected to be the faster one.
 int i2_gemm_kslice(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
                    float s_w, int bitnet_epilogue, int force, hipStream_t stream) {
-  // two pairs of blocks of 128 k per wave and loop turn; with signed codes the accumulators hold 64 x the sum
-  if (K % (kWaves * 512) != 0 || K >= 131072) return 1;
+  // whole pairs of blocks of 128 k per wave; with signed codes the accumulators hold 64 x the sum
+  if (K % (kWaves * 256) != 0 || K >= 131072) return 1;
   // 32-bit lane offsets
   if ((uint64_t)(M + kTileM) * (uint64_t)K >= (1ull << 32) || (uint64_t)(N + kTileN) * (uint64_t)(K >> 2) >= (1ull << 32)) return 1;
   const long tiles = (long)((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);

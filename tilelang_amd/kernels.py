@@ -803,7 +803,7 @@ def bitnet_158_int8xint2_prefill(
     ``"offset"`` (``w = c - 2``, ternary weights stored as ``w + 2``) or ``"twos"``.  ``kernel`` (tests and
     measurements): ``"ksliced"`` or ``"tiled"`` instead of the library's choice by shape; same bits either way.
     ``weight_fragments=True``: B went through ``quantize.prepack_i2_fragments`` (after ``interleave_weight`` when
-    ``fast_decoding``) and has the shape ``[ceil(N/32), K/128, 64, 16]`` (K % 4096 == 0); every batch size has a kernel
+    ``fast_decoding``) and has the shape ``[ceil(N/32), K/128, 64, 16]`` (K % 2048 == 0); every batch size has a kernel
     that reads it: the decode kernel (M <= 4), the K-sliced kernel, the direct-to-LDS tiled kernel.
     """
     if _dtype(in_dtype) != torch.int8 or _dtype(out_dtype) != torch.int32:
@@ -831,10 +831,10 @@ _I2_KERNELS = {None: 0, "ksliced": 16, "tiled": 32}  # DQ_I2_KERNEL_* of include
 
 
 def _i2_fragments_ok(fn: str, K: int, kernel: str | None) -> None:
-    # with K a multiple of 4096 the K-sliced kernel takes every shape, so some kernel always reads the order (the
+    # with K a multiple of 2048 the K-sliced kernel takes every shape, so some kernel always reads the order (the
     # decode kernel at M <= 4, the direct-to-LDS tiled kernel where the problem has enough tiles, else the K-sliced one)
-    if K % 4096 != 0 or K >= 131072:
-        raise ValueError(f"{fn}: weight_fragments needs K % 4096 == 0 and K < 131072 (got K={K})")
+    if K % 2048 != 0 or K >= 131072:
+        raise ValueError(f"{fn}: weight_fragments needs K % 2048 == 0 and K < 131072 (got K={K})")
 
 
 def _i2_kernel_choice(fn: str, kernel: str | None) -> int:
