@@ -550,10 +550,16 @@ def main():
     from tilelang_amd import profiler as tl_profiler
 
     sustained = {}
-    for dt in ("bfloat16", "float16", "int8"):
+    for dt in ("bfloat16", "float16", "int8", "fp4"):
         m = tl_profiler.mfma_sustained_rate(dt, device=dev)
         sustained[dt] = {"T(FL)OP/s": m["ops_per_s"] / 1e12, "ms_per_launch": m["ms_per_launch"],
-                         "frac_of_published_peak": m["ops_per_s"] / (MFMA_I8_PEAK if dt == "int8" else MFMA_BF16_PEAK)}
+                         "frac_of_published_peak": m["ops_per_s"] / {"int8": MFMA_I8_PEAK, "fp4": MFMA_FP4_PEAK}.get(dt, MFMA_BF16_PEAK)}
+    for row in shapes:  # every matrix-pipe row also against the matrix-only rate of its operand type
+        if row.get("bound") == "mfma" and "TFLOP/s" in row:
+            cfg = row["config"]
+            dt = ("fp4" if cfg.startswith("mxfp4_x_mxfp4") else "bfloat16" if cfg.startswith("mxfp4_gemm") else
+                  "float16" if cfg.startswith("w4a16") else "int8")
+            row["frac_of_sustained"] = row["TFLOP/s"] / sustained[dt]["T(FL)OP/s"]
     if roof_gemm is not None:
         roof_gemm["sustained_mfma_only"] = sustained["bfloat16"]["T(FL)OP/s"]
         roof_gemm["frac_of_sustained"] = roof_gemm["achieved"] / sustained["bfloat16"]["T(FL)OP/s"]

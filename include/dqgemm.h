@@ -280,7 +280,8 @@ int call_gemv_int8xint1(const void* A, const void* B, void* C, int M, int N, int
 
 /* ---- plain GEMM on the same MFMA tile (no dequantise step) ----------------------------------------- */
 
-enum dq_dtype { DQ_DT_F16 = 0, DQ_DT_BF16 = 1, DQ_DT_I8 = 2, DQ_DT_F32 = 3, DQ_DT_I32 = 4 };
+enum dq_dtype { DQ_DT_F16 = 0, DQ_DT_BF16 = 1, DQ_DT_I8 = 2, DQ_DT_F32 = 3, DQ_DT_I32 = 4,
+                DQ_DT_FP4 = 5 /* packed e2m1 codes: call_mfma_rate only */ };
 
 /* C[M,N] = op(A) . op(B), both operands at the compute type, fp32 / int32 accumulation on the tile the dequantize
  * GEMMs share.  Replaces `call(A, B, C, stream)` of the kernel built by `matmul(M, N, K, ..., trans_A, trans_B,
@@ -298,8 +299,9 @@ int call_gemm_plain(const void* A, const void* B, void* C, void* Workspace, int 
 /* The rate the matrix pipe sustains on the caller's operands, with no memory, LDS or decode work beside it: every
  * wave of `workgroups` workgroups of four loads four A and four B fragments from Operands (64 KiB, read as they
  * are: fill them with random values of `in_dtype`) and issues `iters` rounds of the 16 matrix instructions of a
- * 128 x 128 wave tile (32x32x16 for DQ_DT_F16 / DQ_DT_BF16, 32x32x32 for DQ_DT_I8); Out takes workgroups * 256
- * floats that mean nothing.  Operations = workgroups * 4 * iters * 16 * 2 * 32 * 32 * (16 or 32); time it with
+ * 128 x 128 wave tile (32x32x16 for DQ_DT_F16 / DQ_DT_BF16, 32x32x32 for DQ_DT_I8, the block-scaled 32x32x64 for
+ * DQ_DT_FP4 with both scales 1.0); Out takes workgroups * 256 floats that mean nothing.  Operations = workgroups * 4 *
+ * iters * 16 * 2 * 32 * 32 * (16, 32 or 64); time it with
  * events.  It has no counterpart in the reference: bench.py reports it beside the GEMM rows, because random
  * operands hold this chip below the clock its published peak assumes, and the figure says by how much. */
 int call_mfma_rate(const void* Operands, void* Out, int in_dtype, int workgroups, int iters, dq_stream_t stream);

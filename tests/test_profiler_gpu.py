@@ -80,7 +80,7 @@ def test_explicit_stream_gets_its_own_outputs(cuda):
     assert len({o.data_ptr() for o in outs}) == 4
 
 
-@pytest.mark.parametrize("dtype, peak", [("bfloat16", 2.5e15), ("float16", 2.5e15), ("int8", 5.0e15)])
+@pytest.mark.parametrize("dtype, peak", [("bfloat16", 2.5e15), ("float16", 2.5e15), ("int8", 5.0e15), ("fp4", 10.1e15)])
 def test_mfma_sustained_rate_is_a_plausible_ceiling(cuda, dtype, peak):
     """``call_mfma_rate`` through ``profiler.mfma_sustained_rate``: the matrix pipe alone, on random operands, runs at
     a sizeable fraction of the published peak and never above it (the count of operations per launch is right)."""

@@ -444,8 +444,8 @@ extern "C" int call_mfma_rate(const void* Operands, void* Out, int in_dtype, int
   const char* fn = "call_mfma_rate";
   if (!Operands || !Out) DQ_FAIL("%s: Operands and Out are expected to have non-NULL data pointers", fn);
   if (!aligned16(Operands) || !aligned16(Out)) DQ_FAIL("%s: Operands and Out must be 16-byte aligned", fn);
-  if (in_dtype != DQ_DT_F16 && in_dtype != DQ_DT_BF16 && in_dtype != DQ_DT_I8)
-    DQ_FAIL("%s: in_dtype must be DQ_DT_F16, DQ_DT_BF16 or DQ_DT_I8 (got %d)", fn, in_dtype);
+  if (in_dtype != DQ_DT_F16 && in_dtype != DQ_DT_BF16 && in_dtype != DQ_DT_I8 && in_dtype != DQ_DT_FP4)
+    DQ_FAIL("%s: in_dtype must be DQ_DT_F16, DQ_DT_BF16, DQ_DT_I8 or DQ_DT_FP4 (got %d)", fn, in_dtype);
   if (workgroups < 1 || workgroups > 65536 || iters < 1) DQ_FAIL("%s: workgroups=%d (1..65536) and iters=%d (>= 1) out of range", fn, workgroups, iters);
   return mfma_rate(Operands, Out, in_dtype, workgroups, iters, (hipStream_t)stream);
 }

@@ -271,7 +271,7 @@ class Profiler:
         return do_bench(fn, warmup=warmup, rep=rep, **kw)
 
 
-_MFMA_RATE_DTYPES = {"float16": (0, 16), "bfloat16": (1, 16), "int8": (2, 32)}
+_MFMA_RATE_DTYPES = {"float16": (0, 16), "bfloat16": (1, 16), "int8": (2, 32), "fp4": (5, 64)}
 
 
 def mfma_sustained_rate(dtype: str = "bfloat16", launch_ms: float = 5.0, settle_ms: float = 60.0, launches: int = 8,
@@ -291,7 +291,7 @@ def mfma_sustained_rate(dtype: str = "bfloat16", launch_ms: float = 5.0, settle_
     with torch.cuda.device(dev):
         lib = _lib.get_library(dev.index)
         gen = torch.Generator(device="cpu").manual_seed(0)
-        if dtype == "int8":
+        if dtype in ("int8", "fp4"):  # every byte is a valid operand: an int8, or two e2m1 codes
             operands = torch.randint(-128, 128, (65536,), generator=gen, dtype=torch.int8).to(dev)
         else:
             operands = torch.randn(32768, generator=gen).to(getattr(torch, dtype)).to(dev)
