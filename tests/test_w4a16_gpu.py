@@ -145,7 +145,7 @@ def test_gemv_quantized_zeros(cuda, M, qfmt):
 
 
 def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False, scale_range=(0.005, 0.02),
-              zeros_offset=0.0, fragments=False):
+              zeros_offset=0.0, fragments=False, oracle_mode=None):
     d = workloads.w4a16(M, N, K, group, seed=seed, scale_range=scale_range, zeros_range=(6, 10))
     if zeros_offset:  # zero points that are not integers
         d["Zeros"] = (d["Zeros"].astype(np.float32) + np.float32(zeros_offset)).astype(np.float16)
@@ -166,7 +166,7 @@ def _run_gemv(cuda, M, N, K, group, mode, seed=0, variant=-1, interleaved=False,
     C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
     kern(*args, C)
     torch.cuda.synchronize()
-    W = _oracle_tile(mode, d["B"], d["Scale"], d["Zeros"], group)
+    W = _oracle_tile(oracle_mode or mode, d["B"], d["Scale"], d["Zeros"], group)
     ref = (d["A"].astype(np.float32) @ W.astype(np.float32).T).astype(np.float16)
     got = C.cpu().numpy()
     assert np.isfinite(got).all()
@@ -228,6 +228,38 @@ def test_streaming_small_batch_kernel(cuda, variant, mode):
     _run_gemv(cuda, 5, 64, 256 * 9, 128, mode, variant=variant, interleaved=True)
     _run_gemv(cuda, 16, 256, 4096, 128, mode, variant=variant)
     _run_gemv(cuda, 20, 300, 11008, 128, mode, variant=variant)
+
+
+@pytest.mark.parametrize("variant", [31, 34, 36, 37, 71, 76])
+@pytest.mark.parametrize("mode", ["scale", "original"])
+@pytest.mark.parametrize("group", [32, 64, 256, 512, 1024, -1])
+def test_streaming_small_batch_kernel_group_sizes(cuda, variant, mode, group):
+    """Group sizes other than 128 (-1: one group per row): a row's 16 bytes of scales then cover one step (32), two
+    (64), eight (256) ... or, for rows of fewer than eight groups, the whole of K (one chunk that runs into the next
+    rows' scales and, for the last rows, is moved back to end with the array).  Ragged N around those last rows, K
+    with fewer steps than ring stages and with many, a K whose scales do not fill the last 16 bytes."""
+    for (M, N, K) in ((37, 16 * 13 + 3, 2048), (64, 130, 1024), (20, 300, 7168), (33, 7, 4096), (17, 129, 512)):
+        g = K if group == -1 else group
+        if g > K or K % g != 0:
+            continue
+        if N * (K // g) * 2 < 16:  # a scale array shorter than one 16-byte chunk: not this kernel's (the default
+            continue               # dispatch then takes the general kernel: test_default_dispatch_group_sizes)
+        # 70..77 fold the zero point: the rounding of z * s is then shared by a whole group, and with groups of
+        # thousands of k the sum can leave the tolerance around the exact tile (which is why the library's own choice
+        # folds up to group 128 only); they are held to the oracle's folded tile instead
+        folded = variant >= 70 and mode == "original"
+        _run_gemv(cuda, M, N, K, g, mode, variant=variant, seed=K + g, oracle_mode="folded" if folded else None)
+
+
+@pytest.mark.parametrize("M", [8, 16, 40, 64, 100])
+@pytest.mark.parametrize("group", [32, 64, 1024, -1])
+def test_default_dispatch_group_sizes(cuda, M, group):
+    """The library's own choice at group sizes other than 128 (the streaming kernel's 32-row form below 17 rows)."""
+    N, K = 1000, 2048
+    g = K if group == -1 else group
+    _run_gemv(cuda, M, N, K, g, "original", seed=M + g)
+    _run_gemv(cuda, M, N, K, g, "scale", seed=M + g + 1, interleaved=True)
+    _run_gemv(cuda, M, 7, 4096, 4096 if group == -1 else group, "original", seed=M + g + 2)
 
 
 @pytest.mark.parametrize("variant,mode", [(32, "original"), (36, "original"), (31, "scale"), (36, "rescale"), (33, "signed"),

@@ -204,9 +204,18 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
     // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
     const bool wide = N >= 128 * 200;
     // 33 to 48 rows: three blocks of 16 activation rows (40.9 us at N = 28672, K = 8192 against 45.3 us with four)
-    const int config = M <= 16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : (M <= 48 ? 7 : 6));
-    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, folded_mode, layout, config, (hipStream_t)stream);
+    // up to 16 rows with another group size than 128: the 32-row form (the six-stage ring of the 16-row form leaves
+    // no room for the scale slots of small groups)
+    const bool rows16 = M <= 16 && (group == 128 || mode < W4_SCALE);
+    const int config = rows16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : (M <= 48 ? 7 : 6));
+    // the folded zero point shares one rounding of z * s among a group's weights: up to 128 k per group the sum stays
+    // well inside the tolerance around the reference's tile, with groups of thousands it need not
+    const int stream_mode = group <= 128 ? folded_mode : asked_mode;
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, stream_mode, layout, config, (hipStream_t)stream);
     if (rc <= 0) return rc;
+    // a shape the streaming kernel does not take (K % 256, a group size that is no power of two ...): from 64 rows on
+    // the tiled GEMM is ahead of the general fallback (N = 28672, K = 8192, group 64: 142 against 285 us at M = 128)
+    if (M >= 64 && K % 64 == 0) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, (hipStream_t)stream);
   }
   return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
 }

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
                                                                      const uint8_t* __restrict__ B,
                                                                      const half_t* __restrict__ S,
                                                                      const half_t* __restrict__ Z, half_t* __restrict__ C,
-                                                                     int M, int N, int K) {
+                                                                     int M, int N, int K, int gshift, int pshift, int scale_slot_mask) {
   extern __shared__ __align__(16) unsigned char smem[];
   using G = StreamGeom<MB, RBW>;
   static_assert(KSPLIT == 1 || KSPLIT == 2, "one or two waves per SIMD");
@@ -82,7 +82,6 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   // DMA instructions per wave per stage; every fourth stage carries one more, the scales / zeros of four steps,
   // which the waits below do not count (they then wait for one instruction more than they must)
   constexpr int kOps = kWOps + kAOps;
-  constexpr int kScaleSlots = NST <= 4 ? 2 : 3;         // groups of four steps alive at a time, plus the one landing
   constexpr int kRing = NST * G::kStage;
   constexpr int kWaitOps = (NST - 2) * kOps;            // younger instructions when the next stage must have landed
   static_assert((NST - 1) * kOps <= 63, "vmcnt is a 6-bit counter");
@@ -100,7 +99,9 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   const int m0 = blockIdx.y * (16 * MB);
   const int mrows = min(M - m0, 16 * MB);
   const int KS = K / kStepK;
-  const int groups_per_row = K >> 7;
+  // Group size 2^gshift (32 .. K): a row's 16 bytes of scales (eight groups) cover 2^pshift steps of 256 k, travel
+  // once per that many steps and live in a ring of scale_slot_mask + 1 slots (the launcher sizes it).
+  const int groups_per_row = max(K >> gshift, 1);  // one group per row: any shift that maps every k to group 0
   const unsigned lds0 = (unsigned)(size_t)smem;
 
   // ---- per-lane source offsets of the DMA instructions ------------------------------------------
@@ -122,15 +123,21 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   // DMA instructions; with 64 rows per workgroup the second half is simply not read.
   // A dword of scales per row and step would ask for 64 different cache lines per instruction, and for the same
   // line 32 steps in a row: instead a row's 16 bytes (four steps) travel at once, every fourth step.
-  const int row_bytes = groups_per_row * 2;  // >= 16: K >= 1024 is checked by the launcher
-  const unsigned s_voff = (unsigned)min(n0 + (wn & 1) * 64 + lane, N - 1) * (unsigned)row_bytes;
+  const int row_bytes = groups_per_row * 2;
+  // Rows of fewer than eight groups (row_bytes < 16; the launcher then made the period cover all of K): the 16 bytes
+  // of a row start at the row's first scale and run into the next rows', except at the end of the array, where
+  // they end with it; lane_shift() is how far behind their start a row's own scales then lie.
+  const bool short_rows = row_bytes < 16;
+  auto chunk_start = [&](int n) { return short_rows ? min(n * row_bytes, N * row_bytes - 16) : n * row_bytes; };
+  const int s_row = min(n0 + (wn & 1) * 64 + lane, N - 1);
+  const unsigned s_voff = (unsigned)chunk_start(s_row);
   const unsigned char* s_src = reinterpret_cast<const unsigned char*>((wn >= 2 && kZeros) ? Z : S);
-  // the last group of a row whose K is not a multiple of 1024 reads the row's last 16 bytes instead of running
-  // past its end, and the readers shift their offset by the same amount
-  auto scale_src_off = [&](int g4) { return min(g4 * 16, row_bytes - 16); };
+  // the last chunk of a row whose scales are not a multiple of 16 bytes reads the row's last 16 bytes instead of
+  // running past its end, and the readers shift their offset by the same amount
+  auto scale_src_off = [&](int g4) { return short_rows ? 0 : min(g4 * 16, row_bytes - 16); };
   auto scale_base = [&](int step) -> const unsigned char* {
-    const int g4 = step >> 2;
-    return smem + kRing + (g4 % kScaleSlots) * G::kScaleSlot + (step * 4 - scale_src_off(g4));
+    const int g4 = step >> pshift;
+    return smem + kRing + (g4 & scale_slot_mask) * G::kScaleSlot + ((((step * 256) >> gshift) << 1) - scale_src_off(g4));
   };
 
   // DMA instruction `op` of the stage of `step`, into ring slot `slot`: the weights, the activations, and (op == kOps,
@@ -144,9 +151,9 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
       dma16(sb + kWBytes + (wave * kAOps + i) * 1024, a_voff[i],
             reinterpret_cast<const unsigned char*>(A) + (size_t)step * (kStepK * 2));
     } else if constexpr (kScale) {
-      if ((step & 3) == 0) {
-        const int g4 = step >> 2;
-        dma16(lds0 + kRing + (g4 % kScaleSlots) * G::kScaleSlot + (wn >= 2 ? 2048 : 0) + (wn & 1) * 1024, s_voff,
+      if ((step & ((1 << pshift) - 1)) == 0) {
+        const int g4 = step >> pshift;
+        dma16(lds0 + kRing + (g4 & scale_slot_mask) * G::kScaleSlot + (wn >= 2 ? 2048 : 0) + (wn & 1) * 1024, s_voff,
               s_src + scale_src_off(g4));
       }
     }
@@ -164,7 +171,10 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
 #pragma unroll
     for (int rb = 0; rb < RBW; ++rb) {
       const int row = wn * (16 * RBW) + rb * 16 + r;
-      sc_off[rb][ui] = row * 16 + u * 2;  // from scale_base(step)
+      // from scale_base(step): the row's 16 bytes, the group of this lane's 32 k inside the step, and for short rows
+      // the distance of the row's scales from the start of its 16 bytes
+      const int n_abs = min(n0 + row, N - 1);
+      sc_off[rb][ui] = row * 16 + ((((u << 7) + (g << 5)) >> gshift) << 1) + (n_abs * row_bytes - chunk_start(n_abs));
       w_off[rb][ui] = row * 128 + ((((u << 2) + g) ^ ((row >> 1) & 7)) << 4);
     }
 #pragma unroll
@@ -372,20 +382,40 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
 }
 
 template <int MB, int RBW, int NST, int KSPLIT>
-int launch_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int mode,
+int launch_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group, int mode,
                   int layout, hipStream_t stream) {
-  constexpr int kLds = NST * StreamGeom<MB, RBW>::kStage + (NST <= 4 ? 2 : 3) * StreamGeom<MB, RBW>::kScaleSlot;
+  constexpr int kRingBytes = NST * StreamGeom<MB, RBW>::kStage;
   constexpr int kRowsPerWg = StreamGeom<MB, RBW>::kRowsPerWg;
-  static_assert(kLds <= 160 * 1024, "LDS budget");
+  constexpr int kMaxLds = 160 * 1024;
+  static_assert(kRingBytes + 2 * StreamGeom<MB, RBW>::kScaleSlot <= kMaxLds, "LDS budget");
+  // Scales: 16 bytes of a row (eight groups) cover `period` steps of 256 k; a chunk is issued with the first stage it
+  // serves, NST - 1 steps ahead, and read until the last: ceil((NST + period - 1) / period) chunks are alive at a
+  // time; the ring takes the next power of two.  Rows of fewer than eight groups: one chunk for the whole of K.
+  int gshift = 7, pshift = 2, mask = 1;
+  if (mode >= W4_SCALE) {
+    gshift = group == K ? 32 - __builtin_clz((unsigned)(K - 1)) : 31 - __builtin_clz((unsigned)group);
+    pshift = gshift - 5;
+    if (K / group < 8) {  // short rows: one chunk, issued with stage 0, serves every step
+      if ((size_t)N * (K / group) * 2 < 16) return 1;
+      while ((K / kStepK) > (1 << pshift)) ++pshift;
+    }
+    const int period = 1 << pshift;
+    const int alive = (NST + period - 1 + period - 1) / period;
+    int slots = 2;
+    while (slots < alive) slots *= 2;
+    if (kRingBytes + slots * StreamGeom<MB, RBW>::kScaleSlot > kMaxLds) return 1;
+    mask = slots - 1;
+  }
+  const int lds = kRingBytes + (mask + 1) * StreamGeom<MB, RBW>::kScaleSlot;
   const dim3 grid((N + kRowsPerWg - 1) / kRowsPerWg, (M + 16 * MB - 1) / (16 * MB));
   const dim3 block(256 * KSPLIT);
 #define DQ_LAUNCH2(MODE_, APERM_)                                                                                    \
   do {                                                                                                               \
-    auto kern = w4a16_stream_kernel<MB, RBW, NST, KSPLIT, MODE_, APERM_>;                                                         \
+    auto kern = w4a16_stream_kernel<MB, RBW, NST, KSPLIT, MODE_, APERM_>;                                            \
     static bool lds_limit_raised[kMaxDevices];                                                                       \
-    if (raise_lds_limit<kLds>(kern, lds_limit_raised)) return -1;                                                    \
-    hipLaunchKernelGGL(kern, grid, block, kLds, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,       \
-                       (const half_t*)Z, (half_t*)C, M, N, K);                                                       \
+    if (raise_lds_limit<kMaxLds>(kern, lds_limit_raised)) return -1;                                                 \
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,        \
+                       (const half_t*)Z, (half_t*)C, M, N, K, gshift, pshift, mask);                                         \
   } while (0)
 #define DQ_LAUNCH_MODE(MODE_)                              \
   do {                                                     \
@@ -421,17 +451,18 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, hipStream_t stream) {
   if (K % kStepK != 0 || N < 1 || M < 1) return 1;
-  if (mode >= W4_SCALE && (group != 128 || K < 1024)) return 1;  // scales travel 16 bytes (1024 k) per row at a time
+  // scales travel 16 bytes of a row at a time: group sizes 32, 64, ... (powers of two that divide K), or one group per row
+  if (mode >= W4_SCALE && group != K && (group < 32 || group > K || (group & (group - 1)) != 0 || K % group != 0)) return 1;
   if ((size_t)N * K / 2 >= (1ull << 32) || (size_t)M * K * 2 >= (1ull << 32)) return 1;
   switch (config) {
-    case 0: return launch_stream<1, 2, 6, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 1: return launch_stream<2, 2, 4, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 2: return launch_stream<4, 2, 3, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 3: return launch_stream<1, 1, 4, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 4: return launch_stream<2, 1, 3, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 5: return launch_stream<1, 1, 6, 1>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 6: return launch_stream<4, 2, 3, 2>(A, B, S, Z, C, M, N, K, mode, layout, stream);
-    case 7: return launch_stream<3, 2, 3, 2>(A, B, S, Z, C, M, N, K, mode, layout, stream);
+    case 0: return launch_stream<1, 2, 6, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 1: return launch_stream<2, 2, 4, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 2: return launch_stream<4, 2, 3, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 3: return launch_stream<1, 1, 4, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 4: return launch_stream<2, 1, 3, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 5: return launch_stream<1, 1, 6, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 6: return launch_stream<4, 2, 3, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 7: return launch_stream<3, 2, 3, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
     default: DQ_FAIL("w4a16 stream kernel: unknown configuration %d", config);
   }
 }
