@@ -199,6 +199,34 @@ def test_w4a16_large_m(cuda, mode, interleaved, M, N, K):
     np.testing.assert_allclose(C.float().cpu().numpy(), ref.astype(np.float32), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("group", [32, 64, 256, 512, -1])
+@pytest.mark.parametrize("mode", ["scale", "original"])
+@pytest.mark.parametrize("M,N", [(3584, 3584), (1100, 3500), (300, 320)])  # direct-to-LDS 256 x 256, 128 x 256; staged
+def test_w4a16_large_m_group_sizes_tile_exact_through_identity(cuda, group, mode, M, N):
+    """Group sizes other than 128 through the GEMM: the direct-to-LDS kernel brings a dword of scales per row (two
+    groups) per the tiles it serves (one tile of 64 k at group 32, on the 128 x 256 tile only; eight tiles at 256); one group per row (-1) and odd
+    group counts stay on the register-staged kernel.  Identity rows for A: C[k, n] = W[n, k], every bit."""
+    K = 1024
+    g = K if group == -1 else group
+    d = workloads.w4a16(1, N, K, g, seed=13 + g, scale_range=(0.002, 0.02), zeros_range=(6, 10))
+    B, S, Z = d["B"], d["Scale"], d["Zeros"]
+    B[1, :] = np.arange(K // 2, dtype=np.uint8)
+    Z[3, :] = Z[3, :] - np.float16(0.25)
+    kw = {"scale": dict(source_format="int"), "original": dict(source_format="uint", with_zeros=True)}[mode]
+    W = orc.dequant_u4_scale(B, S, g) if mode == "scale" else orc.dequant_u4_scale_zeros(B, S, Z, g, mode)
+    rows = min(M, K)
+    A = np.zeros((M, K), dtype=np.float16)
+    A[np.arange(rows), np.arange(rows)] = 1.0
+    kern = tl.matmul_w4a16(M, N, K, group_size=g, **kw)
+    args = [_dev(A, cuda), _dev(B, cuda).view(torch.int8), _dev(S, cuda)] + ([_dev(Z, cuda)] if kw.get("with_zeros") else [])
+    C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+    kern(*args, C)
+    torch.cuda.synchronize()
+    got = C.cpu().numpy()
+    np.testing.assert_array_equal(got[:rows].view(np.uint16), np.ascontiguousarray(W.T[:rows]).view(np.uint16))
+    assert not got[rows:].any()
+
+
 @pytest.mark.parametrize("mode", ["scale", "original", "rescale", "folded"])
 @pytest.mark.parametrize("interleaved", [False, True])
 @pytest.mark.parametrize("N", [300, 3584])  # register-staged tiles / the direct-to-LDS kernel

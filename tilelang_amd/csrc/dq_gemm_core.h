@@ -534,7 +534,8 @@ __global__ __launch_bounds__(64 * kWavesM * (8 / kNBW), 32 * kMBW * kWavesM == 1
   constexpr int kBSlot = kPairB ? kBStage : kStage;                  // distance between B slots
   constexpr int kAStride = kPairB ? kAStage : kStage;                // distance between A stages
   // Scales that travel by DMA (P::kScaleDma): 1 = one byte per 32 k (a dword per row covers a pair of tiles),
-  // 2 = one fp16 per 128 k (a dword per row covers four tiles), 3 = the same for scales and for zeros.
+  // 2 = one fp16 per group of 64 .. 4096 k (a dword per row covers two groups: four tiles at group 128), 3 = the same
+  // for scales and for zeros.
   // Ring: 4 slots x 1 KiB (256 rows x one dword), a second ring for the zeros.
   constexpr int kRing = kPairB ? kStages * kAStage + 4 * kBStage : kStages * kStage;
   constexpr int kSOps = P::kScaleDma == 0 ? 0 : (P::kScaleDma == 3 ? 2 : 1);  // scale DMA instructions per wave per tile
@@ -576,7 +577,12 @@ __global__ __launch_bounds__(64 * kWavesM * (8 / kNBW), 32 * kMBW * kWavesM == 1
       b_voff[i] = (unsigned)blk * (unsigned)(p.ldk / P::kKPerBlock) * 1024u + (unsigned)lane * 16u;
     }
   }
-  const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(P::kScaleDma == 1 ? (K >> 5) : (K >> 6));  // waves 4..7 repeat 0..3
+  // fp16 scales (kScaleDma >= 2): one per 2^p0 k (p.p0 = 5 .. 12, the policy's dma_ok checks it), so a dword of a row
+  // serves 2^s_ps tiles of 64 k.  Groups of 32 k (one tile per dword, the two k halves of a tile in different groups)
+  // need the scales issued with every tile: not the kPairB form, which dma_eligible keeps them away from
+  const int s_gshift = P::kScaleDma >= 2 ? p.p0 : 7;
+  const int s_ps = s_gshift - 5;
+  const unsigned s_voff = (unsigned)min(n0 + (tid & 255), N - 1) * (unsigned)(P::kScaleDma == 1 ? (K >> 5) : ((K >> s_gshift) << 1));  // waves 4..7 repeat 0..3
 
   // One tile = kSOps + kAOps + kBOps DMA instructions per thread: first the scale dword(s) (row tid; issued
   // with every tile although a dword serves two or four, which keeps the loop branch-free), then the A
@@ -590,7 +596,7 @@ __global__ __launch_bounds__(64 * kWavesM * (8 / kNBW), 32 * kMBW * kWavesM == 1
         const int pair = kb >> 1;
         dma4(lds0 + kRing + (pair & 3) * 1024 + (wave & 3) * 256, s_voff, (const unsigned char*)p.S + (size_t)pair * 4);
       } else if constexpr (P::kScaleDma >= 2) {
-        const int quad = kb >> 2;
+        const int quad = kb >> s_ps;
         dma4(lds0 + kRing + op * 4096 + (quad & 3) * 1024 + (wave & 3) * 256, s_voff,
              (const unsigned char*)(op == 0 ? p.S : p.Z) + (size_t)quad * 4);
       }
@@ -622,7 +628,7 @@ __global__ __launch_bounds__(64 * kWavesM * (8 / kNBW), 32 * kMBW * kWavesM == 1
       // fragment order: block row / 32 of the tile, then the lanes as the matrix instruction numbers them
       if constexpr (kBFrag) b_off[nb][h] = (row >> 5) * 1024 + lane * 16;
     }
-    s_off[nb] = kRing + row * 4 + (P::kScaleDma == 1 ? g : 0);
+    s_off[nb] = kRing + row * 4 + (P::kScaleDma == 1 ? g : (P::kScaleDma >= 2 && s_gshift == 5 ? 2 * g : 0));
   }
   using frag_t = typename P::frag_t;
   auto read_a1 = [&](const unsigned char* base, int j, int mb) -> frag_t {
@@ -647,7 +653,8 @@ __global__ __launch_bounds__(64 * kWavesM * (8 / kNBW), 32 * kMBW * kWavesM == 1
   };
   auto read_scale1 = [&](int kb, int nb) -> typename P::Scale {
     if constexpr (P::kScaleDma >= 2) {
-      const unsigned char* at = smem + s_off[0] + ((kb >> 2) & 3) * 1024 + ((kb >> 1) & 1) * 2 + nb * 128;
+      // which of the dword's two groups: with groups of 32 k the lane's half of the tile (in s_off), else the tile's
+      const unsigned char* at = smem + s_off[0] + ((kb >> s_ps) & 3) * 1024 + (s_gshift == 5 ? 0 : (((kb << 6) >> s_gshift) & 1) * 2) + nb * 128;
       return P::ring_scale(at, at + 4096);
     } else {
       return P::prep_scale(read_scale_byte(kb, nb), p);
@@ -994,7 +1001,10 @@ bool dma_eligible(const Params& p) {
   // 32-bit lane offsets: A rows are 128 bytes per K block, packed B rows kBRowBytes
   const size_t a_bytes = (size_t)p.M * (p.ldk / P::kKPerBlock) * kARowBytes;
   const size_t b_bytes = (size_t)p.N * (p.ldk / P::kKPerBlock) * P::kBRowBytes;
-  return P::dma_ok(p) && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && a_bytes < (1ull << 32) && b_bytes < (1ull << 32);
+  // fp16 scales of groups of 32 k go with every tile: not with the pairwise issue of the 32-byte-row form of this tile
+  const bool scales_per_tile = P::kScaleDma >= 2 && P::kBRowBytes == 32 && p.p0 == 5;
+  return P::dma_ok(p) && !scales_per_tile && (p.K % (2 * P::kKPerBlock) == 0) && tiles >= 192 && a_bytes < (1ull << 32) &&
+         b_bytes < (1ull << 32);
 }
 
 // Problems with too few 256 x 256 tiles for the kernel above but at least `min_tiles` tiles of 128 x 256: the same

@@ -29,10 +29,11 @@ struct W4F16Policy : F16Mfma {
   using out_t = half_t;
   struct ScaleRaw { half_t s, z; };
   struct Scale { half_t s, addend; };  // what the decoder multiplies by and adds (w4_cvt_addend)
-  // direct-to-LDS kernel: with one scale (and zero) per 128 k the fp16 values travel by DMA, a dword per row
-  // (two groups = four tiles of 64 k) at a time; other group sizes stay on the register-staged kernel
+  // direct-to-LDS kernel: the fp16 scales (and zeros) of groups of 32 .. 4096 k travel by DMA, a dword per row (two
+  // groups: four tiles of 64 k at group 128) at a time; (groups of 32 k on the 128 x 256 tile only); one group per row
+  // and odd group counts stay on the register-staged kernel
   static constexpr int kScaleDma = MODE >= W4_ZEROS_ORIGINAL ? 3 : (MODE >= W4_SCALE ? 2 : 0);
-  static bool dma_ok(const Params& p) { return kScaleDma == 0 || (p.p0 == 7 && p.K % 256 == 0); }
+  static bool dma_ok(const Params& p) { return kScaleDma == 0 || (p.p0 >= 5 && p.p0 <= 12 && p.K % (2 << p.p0) == 0); }
   __device__ static __forceinline__ Scale ring_scale(const unsigned char* s_at, const unsigned char* z_at) {
     ScaleRaw r{(half_t)1.f, (half_t)0.f};
     r.s = *reinterpret_cast<const half_t*>(s_at);
