@@ -89,6 +89,20 @@ enum dq_w4_layout {
 int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M,
                                int N, int K, int group, int mode, int layout, int variant, dq_stream_t stream);
 
+/* The same product with a workspace the kernels may use for partial sums.  The reference's counterpart is the
+ * split-K form of its dequantize GEMM (examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:130-186, SplitC
+ * allocated inside the kernel function); here the caller brings the buffer.  A matrix with few rows and a long K
+ * (N = 4096, K = 14336: 64 workgroups of 64 rows for 256 CUs) leaves most of the chip idle at 2 <= M <= 128; with a
+ * workspace of dq_w4a16_workspace_bytes(M, N, K, group, mode) bytes the default dispatch (`variant` < 0) cuts K into
+ * up to 16 slices, one workgroup each, writes their fp32 sums to the workspace and adds them in slice order in a
+ * second kernel: results do not depend on timing and stay within rounding of the unsplit kernel's.  A smaller
+ * workspace lowers the slice count, NULL / 0 bytes is call_dequantize_gemv_w4a16.  Workspace: 16-byte aligned,
+ * contents undefined afterwards, not to be shared by calls that overlap in time. */
+size_t dq_w4a16_workspace_bytes(int M, int N, int K, int group, int mode);
+int call_dequantize_gemv_w4a16_ws(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
+                                  void* Workspace, size_t workspace_bytes, int M, int N, int K, int group, int mode,
+                                  int layout, int variant, dq_stream_t stream);
+
 /* W[N,K] fp16 = dequant(B, Scale, Zeros): the dequantised weight tile with the same
  * device decoder the GEMV/GEMM kernels use.  Replaces the `_convert_test`-style kernels
  * of the examples (examples/dequantize_gemm/example_dequant_gemm_w4a8.py:36-65). */

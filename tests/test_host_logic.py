@@ -20,7 +20,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "dqgemm.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"^\s*(?:int|const char\*)\s+(\w+)\s*\(", text, flags=re.M)))
+    return sorted(set(re.findall(r"^\s*(?:int|size_t|const char\*)\s+(\w+)\s*\(", text, flags=re.M)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -30,8 +30,24 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert getattr(lib, n) is not None
     # every declared entry point has a bound signature, and nothing undeclared is bound
-    assert sorted(set(_lib.SIGNATURES) | {"get_last_error"}) == names
+    assert sorted(set(_lib.SIGNATURES) | set(_lib.SIZE_QUERIES) | {"get_last_error"}) == names
     assert lib.get_last_error().decode() == "" or isinstance(lib.get_last_error(), bytes)
+
+
+def test_w4a16_workspace_query():
+    """How much room the small-batch kernel asks for to cut K over workgroups: nothing where the rows alone fill the
+    chip, where there is one row or K is short; otherwise a whole number of [M, N] fp32 slices, at most 16."""
+    q = _lib.load_library().dq_w4a16_workspace_bytes
+    assert q(16, 28672, 8192, 128, 5) == 0          # 448 workgroups of 64 rows
+    assert q(1, 4096, 14336, 128, 5) == 0           # the GEMV takes one row
+    assert q(16, 1536, 1024, 128, 5) == 0           # four steps of 256 k: nothing to cut
+    assert q(3, 1023, 8192, 128, 5) == 0            # M * N not a multiple of four: the slices' rows would be misaligned
+    assert q(2048, 4096, 14336, 128, 5) == 0        # the tiled GEMM's
+    for (M, N, K, group, mode) in ((4, 4096, 14336, 128, 5), (64, 4096, 11008, 128, 5), (256, 4096, 14336, 128, 5),
+                                   (32, 512, 8192, 32, 3), (16, 1024, 4096, 4096, 5), (24, 1024, 6144, 128, 0)):
+        nbytes = q(M, N, K, group, mode)
+        assert nbytes > 0 and nbytes % (M * N * 4) == 0 and 2 <= nbytes // (M * N * 4) <= 16
+        assert K // 256 // (nbytes // (M * N * 4)) >= 4  # every slice at least 1024 k long
 
 
 def test_entry_points_reject_bad_arguments_before_any_launch():

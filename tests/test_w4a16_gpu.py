@@ -364,6 +364,88 @@ def test_fragment_ordered_weights_are_refused_where_no_kernel_reads_them(cuda):
         kern(A, B, S, C)
 
 
+def _workspace_bytes(M, N, K, group, mode):
+    from tilelang_amd import _lib
+
+    return int(_lib.load_library().dq_w4a16_workspace_bytes(M, N, K, K if group == -1 else group, mode))
+
+
+@pytest.mark.parametrize("M", [2, 4, 16, 24, 40, 64, 128])
+@pytest.mark.parametrize("N,K,group,mode", [
+    (1024, 11008, 128, "original"),   # 43 steps of 256 k: slices of unequal length
+    (1024, 14336, 64, "original"),
+    (512, 8192, 32, "scale"),
+    (512, 16384, 1024, "original"),   # 16 bytes of a row's scales cover 32 steps: slices start there
+    (1024, 4096, -1, "original"),     # one group per row
+    (640, 4096, 2048, "rescale"),     # two groups per row: the whole row's scales travel once
+    (1024, 6144, 128, "unsigned"),    # no scales
+])
+def test_split_k_few_rows_long_k(cuda, M, N, K, group, mode):
+    """Few weight rows and a long K: the default dispatch cuts K over workgroups (fp32 partial sums in a workspace
+    the factory adds, summed in slice order) and still meets the oracle."""
+    group = K if group == -1 else group
+    assert _workspace_bytes(M, N, K, group, {"original": 5, "scale": 3, "rescale": 6, "unsigned": 0}[mode]) > 0
+    _run_gemv(cuda, M, N, K, group, mode, seed=M, scale_range=(0.002, 0.01))
+
+
+@pytest.mark.parametrize("M", [4, 32, 64])
+def test_split_k_llm_shape(cuda, M):
+    """N = 4096, K = 11008 (a 7B model's down projection): 64 workgroups without the split."""
+    _run_gemv(cuda, M, 4096, 11008, 128, "original", seed=3, scale_range=(0.002, 0.01))
+
+
+@pytest.mark.parametrize("M,N,K", [(200, 1024, 4096), (256, 4096, 4096), (384, 2048, 8192), (1000, 1000, 2048), (130, 520, 11008)])
+def test_few_hundred_rows_against_few_tiles(cuda, M, N, K):
+    """Above 128 rows the default dispatch keeps the streaming kernel (passes of 64 rows, K split where that fills
+    the chip) while the matrix gives the tiled GEMM at most 64 tiles of 256 x 256."""
+    _run_gemv(cuda, M, N, K, 128, "original", seed=M, scale_range=(0.002, 0.01))
+    _run_gemv(cuda, M, N, K, 64, "scale", seed=M + 1, interleaved=True, scale_range=(0.002, 0.01))
+
+
+def test_split_k_deterministic_and_close_to_unsplit(cuda):
+    M, N, K, group = 24, 1024, 14336, 128
+    a = _run_gemv(cuda, M, N, K, group, "original", seed=9, scale_range=(0.002, 0.01))
+    b = _run_gemv(cuda, M, N, K, group, "original", seed=9, scale_range=(0.002, 0.01))
+    np.testing.assert_array_equal(a.view(np.uint16), b.view(np.uint16))
+    # the same kernel without the split (configuration 4 named outright, folded zero point as the default runs it)
+    c = _run_gemv(cuda, M, N, K, group, "original", seed=9, variant=74, scale_range=(0.002, 0.01), oracle_mode="folded")
+    # only the order of the fp32 additions differs: a unit or two in the last place of the fp16 result
+    assert np.abs(a.astype(np.float32) - c.astype(np.float32)).max() <= 2 * np.spacing(np.abs(c).max().astype(np.float16)).astype(np.float32)
+
+
+def test_split_k_workspace_through_c_abi(cuda):
+    """The entry point with a workspace: a smaller workspace lowers the slice count, none is the plain entry point;
+    a workspace pointer that is NULL or misaligned is refused."""
+    from tilelang_amd import _lib
+    from tilelang_amd.kernels import LAYOUT_PLAIN
+
+    lib = _lib.get_library()
+    M, N, K, group, mode = 16, 1024, 8192, 128, 5
+    d = workloads.w4a16(M, N, K, group, seed=11, scale_range=(0.002, 0.01), zeros_range=(6, 10))
+    A, B, S, Z = (_dev(d[k], cuda) for k in ("A", "B", "Scale", "Zeros"))
+    W = orc.dequant_u4_scale_zeros(d["B"], d["Scale"], d["Zeros"], group, "original")
+    ref = (d["A"].astype(np.float32) @ W.astype(np.float32).T).astype(np.float16).astype(np.float32)
+    full = int(lib.dq_w4a16_workspace_bytes(M, N, K, group, mode))
+    assert full > 0 and full % (M * N * 4) == 0 and full // (M * N * 4) >= 2
+    stream = torch.cuda.current_stream().cuda_stream
+    ws = torch.empty(full + 16, dtype=torch.uint8, device=cuda)
+    for nbytes in (full, 2 * M * N * 4, M * N * 4, 0):
+        C = torch.full((M, N), float("nan"), dtype=torch.float16, device=cuda)
+        rc = lib.call_dequantize_gemv_w4a16_ws(A.data_ptr(), B.data_ptr(), S.data_ptr(), Z.data_ptr(), C.data_ptr(),
+                                               ws.data_ptr() if nbytes else None, nbytes, M, N, K, group, mode, LAYOUT_PLAIN, -1,
+                                               stream)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(C.cpu().numpy().astype(np.float32), ref, rtol=RTOL, atol=ATOL)
+    C = torch.zeros((M, N), dtype=torch.float16, device=cuda)
+    rc = lib.call_dequantize_gemv_w4a16_ws(A.data_ptr(), B.data_ptr(), S.data_ptr(), Z.data_ptr(), C.data_ptr(), None, full, M, N,
+                                           K, group, mode, LAYOUT_PLAIN, -1, stream)
+    assert rc == -1 and "Workspace is expected to have non-NULL data pointer" in _lib.last_error()
+    rc = lib.call_dequantize_gemv_w4a16_ws(A.data_ptr(), B.data_ptr(), S.data_ptr(), Z.data_ptr(), C.data_ptr(), ws.data_ptr() + 4,
+                                           full, M, N, K, group, mode, LAYOUT_PLAIN, -1, stream)
+    assert rc == -1 and "16-byte aligned" in _lib.last_error()
+
+
 def test_multi_tile_k(cuda):
     """K large enough that the activations are staged in several LDS tiles."""
     _run_gemv(cuda, 16, 256, 8192, 128, "scale")

@@ -23,10 +23,11 @@ _initialised_devices: set = set()
 
 _vp, _i = ctypes.c_void_p, ctypes.c_int
 
-#: name -> argtypes; every entry point returns int (0 ok / -1 error) except get_last_error
+#: name -> argtypes; every entry point returns int (0 ok / -1 error) except get_last_error and SIZE_QUERIES
 SIGNATURES = {
     "init": [],
     "call_dequantize_gemv_w4a16": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "call_dequantize_gemv_w4a16_ws": [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_dequantize_gemv_lowbit": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_unpack_qzeros": [_vp, _vp, _i, _i, _i, _vp],
     "call_dequantize_w4": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -44,6 +45,11 @@ SIGNATURES = {
     "call_gemm_plain": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "call_mfma_rate": [_vp, _vp, _i, _i, _i, _vp],
     "call_gemm_mxfp4_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+}
+
+#: name -> argtypes of the functions that return a byte count (size_t) and launch nothing
+SIZE_QUERIES = {
+    "dq_w4a16_workspace_bytes": [_i, _i, _i, _i, _i],
 }
 
 
@@ -77,6 +83,10 @@ def load_library() -> ctypes.CDLL:
             for name, argtypes in SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.restype = ctypes.c_int
+                fn.argtypes = argtypes
+            for name, argtypes in SIZE_QUERIES.items():
+                fn = getattr(lib, name)
+                fn.restype = ctypes.c_size_t
                 fn.argtypes = argtypes
             _lib = lib
     return _lib

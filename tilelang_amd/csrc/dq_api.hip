@@ -25,7 +25,7 @@ int largest_lds_request() { return g_largest_lds_request; }
 int w4a16_regres(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int fast, hipStream_t stream);
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
-                 int mode, int layout, int config, hipStream_t stream);
+                 int mode, int layout, int config, int split, void* parts, hipStream_t stream);
 int w4a16_skinny(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int variant, hipStream_t stream);
 int w4_dequant(const void* B, const void* S, const void* Z, void* W, int N, int K, int group, int mode, int layout,
@@ -137,10 +137,60 @@ extern "C" int init(void) {
   return 0;
 }
 
-extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
-                                          int M, int N, int K, int group, int mode, int layout, int variant,
-                                          dq_stream_t stream) {
-  const char* fn = "call_dequantize_gemv_w4a16";
+// ---- the streaming small-batch kernel's default configuration and K split ------------------------------
+// Which configuration the default dispatch runs at M rows (see w4a16_stream for the numbering).
+static int w4a16_stream_config(int M, int N) {
+  // up to 16 rows: 64 weight rows per workgroup and a ring of four stages, whatever N and the group size (N = 28672,
+  // K = 6144, 4 rows: 22.8 us against 23.8 with 128 weight rows and six stages, which has no room for the scale
+  // slots of groups of 32; K = 8192, group 256: 26.9 against 28.9)
+  if (M <= 16) return 3;
+  // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
+  const bool wide = N >= 128 * 200;
+  // 33 to 48 rows: three blocks of 16 activation rows (40.9 us at N = 28672, K = 8192 against 45.3 us with four)
+  return M <= 32 ? (wide ? 1 : 4) : (M <= 48 ? 7 : 6);
+}
+
+// Into how many slices of K the streaming kernel's workgroups are split when the matrix has too few rows to give
+// every CU a workgroup (N = 4096: 64 workgroups of 64 rows for 256 CUs) and the caller brought a workspace: the
+// count that fills the last round of workgroups best, every slice at least 1024 k long.  1: no split.
+static int w4a16_stream_split(int M, int N, int K, int group, int mode, int config) {
+  if (K % 256 != 0 || ((size_t)M * N) % 4 != 0) return 1;
+  const int rows = (config >= 3 && config <= 5) ? 64 : 128;
+  const int pass = (config == 0 || config == 3 || config == 5) ? 16 : (config == 1 || config == 4) ? 32 : (config == 7 ? 48 : 64);
+  const long wgs = (long)((N + rows - 1) / rows) * ((M + pass - 1) / pass);
+  constexpr int kCus = 256;
+  if (wgs >= kCus * 5 / 8) return 1;
+  // slices start where a chunk of scales (16 bytes of a row: eight groups) starts
+  const int steps = K / 256;
+  const int unit = (mode >= W4_SCALE && group != K && K / group >= 8 && group > 32) ? group / 32 : 1;
+  const int units = (steps + unit - 1) / unit;
+  int best = 1;
+  double best_fill = (double)wgs / kCus;
+  for (int split = 2; split <= 16 && split <= units && steps / split >= 4; ++split) {
+    const long total = wgs * split;
+    const double fill = (double)total / (double)(kCus * ((total + kCus - 1) / kCus));
+    if (fill > best_fill * 1.04) best = split, best_fill = fill;
+  }
+  return best;
+}
+
+// A few hundred activation rows against a matrix that gives the tiled GEMM at most 64 tiles of 256 x 256: the GEMM
+// then runs one round of workgroups on a quarter of the CUs at the latency of its ring (about 12 ns per k: N = 4096,
+// K = 14336 takes 171 us from 129 to 512 rows), and the streaming kernel in passes of 64 rows is ahead of it (58 us at
+// 256 rows, 42 us with K cut in two; N = 8192, K = 8192 at 512 rows: 81 against 114 us; the two meet near 128 tiles).
+static bool w4a16_few_tiles(int M, int N, int K) {
+  return M <= 1024 && K % 256 == 0 && (long)((M + 255) / 256) * ((N + 255) / 256) <= 64;
+}
+
+extern "C" size_t dq_w4a16_workspace_bytes(int M, int N, int K, int group, int mode) {
+  if (M < 2 || N <= 0 || K <= 0 || group <= 0 || (M > 128 && !w4a16_few_tiles(M, N, K))) return 0;
+  const int split = w4a16_stream_split(M, N, K, group, mode, w4a16_stream_config(M, N));
+  return split > 1 ? (size_t)split * M * N * sizeof(float) : 0;
+}
+
+static int gemv_w4a16(const char* fn, const void* A, const void* B, const void* Scale, const void* Zeros, void* C, int M, int N,
+                      int K, int group, int mode, int layout, int variant, void* workspace, size_t workspace_bytes,
+                      dq_stream_t stream) {
   if (!A) DQ_FAIL("%s: A is expected to have non-NULL data pointer", fn);
   if (!C) DQ_FAIL("%s: C is expected to have non-NULL data pointer", fn);
   if (M <= 0) DQ_FAIL("%s: M must be positive (got %d)", fn, M);
@@ -162,12 +212,12 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
               "but \"rescale\" only (got M=%d N=%d K=%d group=%d mode=%d)", fn, M, N, K, group, mode);
     return rc;
   }
-  // prefill-sized M: the tiled MFMA GEMM (same tile-exact decoders); up to 128 rows the streaming kernel
-  // below (two passes over the weights) is still the faster one.  50: the GEMM whatever M.
-  if ((variant < 0 && M > 128) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, (hipStream_t)stream);
+  // prefill-sized M: the tiled MFMA GEMM (same tile-exact decoders); up to 128 rows, and beyond that against a
+  // matrix of few tiles, the streaming kernel below (passes of 64 rows over the weights) is still the faster one.
+  // 50: the GEMM whatever M.
+  if ((variant == -1 && M > 128 && !w4a16_few_tiles(M, N, K)) || variant == 50) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, (hipStream_t)stream);
   // variant < 0: heuristic.  100 + r: the dot2 GEMV kernel with r rows in flight per thread (r = 0: its own
-  // choice).  30..36: a configuration of the direct-to-LDS small-batch kernel.  60, 61: the K-sliced batch kernel
-  // (M <= 64, N >= 22400) with two / more pairs of activation loads in flight.  40: the kernel with
+  // choice).  30..37: a configuration of the direct-to-LDS small-batch kernel.  40: the kernel with
   // register-resident activations (M <= 16).  0, 4, 5, 10: a configuration of the tiled MFMA fallback kernel
   // (covers every shape).
   if ((variant >= 40 && variant <= 43) || (variant < 0 && M >= 2 && M <= 16)) {
@@ -185,39 +235,59 @@ extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const vo
   // above 16 rows
   const int folded_mode = mode == W4_ZEROS_ORIGINAL ? W4_ZEROS_FOLDED : mode;
   if (variant >= 70 && variant < 80) {
-    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, folded_mode, layout, variant - 70, (hipStream_t)stream);
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, folded_mode, layout, variant - 70, 1, nullptr, (hipStream_t)stream);
     if (rc > 0) DQ_FAIL("%s: the streaming small-batch kernel does not cover N=%d K=%d group=%d", fn, N, K, group);
     return rc;
   }
   if (variant >= 30 && variant < 40) {
-    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, variant - 30, (hipStream_t)stream);
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, variant - 30, 1, nullptr, (hipStream_t)stream);
     if (rc > 0) DQ_FAIL("%s: the streaming small-batch kernel does not cover N=%d K=%d group=%d", fn, N, K, group);
     return rc;
   }
-  if (variant < 0 || variant >= 100) {
+  // one and two rows: the dot2 GEMV (it takes up to four, but from three rows on the streaming kernel below is ahead
+  // of it: N = 13824, K = 5120 at 4 rows 13.0 against 19.4 us; N = 28672, K = 6144 22.8 against 32.3)
+  if ((variant < 0 && M <= 2) || variant >= 100) {
     const int rc = w4a16_gemv_dot2(A, B, Scale, Zeros, C, M, N, K, group, mode, layout,
                                    variant >= 100 ? variant - 100 : 0, (hipStream_t)stream);
     if (rc <= 0) return rc;
     if (variant >= 100) DQ_FAIL("%s: the dot2 GEMV kernel does not cover M=%d K=%d", fn, M, K);
   }
-  if (variant < 0 && M > 4) {
-    // 128 weight rows per workgroup when that still gives every CU a workgroup, else 64
-    const bool wide = N >= 128 * 200;
-    // 33 to 48 rows: three blocks of 16 activation rows (40.9 us at N = 28672, K = 8192 against 45.3 us with four)
-    // up to 16 rows with another group size than 128: the 32-row form (the six-stage ring of the 16-row form leaves
-    // no room for the scale slots of small groups)
-    const bool rows16 = M <= 16 && (group == 128 || mode < W4_SCALE);
-    const int config = rows16 ? (wide ? 0 : 3) : (M <= 32 ? (wide ? 1 : 4) : (M <= 48 ? 7 : 6));
+  if (variant < 0 && M >= 2) {
+    const int config = w4a16_stream_config(M, N);
     // the folded zero point shares one rounding of z * s among a group's weights: up to 128 k per group the sum stays
     // well inside the tolerance around the reference's tile, with groups of thousands it need not
     const int stream_mode = group <= 128 ? folded_mode : asked_mode;
-    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, stream_mode, layout, config, (hipStream_t)stream);
+    // with a workspace: K split over workgroups where the rows alone leave CUs idle
+    // (variant -2, -3, ...: that many slices whatever the heuristic says, for measurements and tests)
+    int split = !workspace ? 1 : (variant <= -2 ? -variant : w4a16_stream_split(M, N, K, group, mode, config));
+    while (split > 1 && (size_t)split * M * N * sizeof(float) > workspace_bytes) --split;
+    const int rc = w4a16_stream(A, B, Scale, Zeros, C, M, N, K, group, stream_mode, layout, config, split, workspace, (hipStream_t)stream);
     if (rc <= 0) return rc;
     // a shape the streaming kernel does not take (K % 256, a group size that is no power of two ...): from 64 rows on
     // the tiled GEMM is ahead of the general fallback (N = 28672, K = 8192, group 64: 142 against 285 us at M = 128)
     if (M >= 64 && K % 64 == 0) return w4_f16_gemm(A, B, Scale, Zeros, C, M, N, K, group, asked_mode, layout, (hipStream_t)stream);
   }
+  if (variant < 0 && M > 2 && M <= 4) {  // three and four rows of a shape the streaming kernel does not take
+    const int rc = w4a16_gemv_dot2(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, 0, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
   return w4a16_skinny(A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, (hipStream_t)stream);
+}
+
+extern "C" int call_dequantize_gemv_w4a16(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
+                                          int M, int N, int K, int group, int mode, int layout, int variant,
+                                          dq_stream_t stream) {
+  return gemv_w4a16("call_dequantize_gemv_w4a16", A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, nullptr, 0, stream);
+}
+
+extern "C" int call_dequantize_gemv_w4a16_ws(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,
+                                             void* Workspace, size_t workspace_bytes, int M, int N, int K, int group,
+                                             int mode, int layout, int variant, dq_stream_t stream) {
+  const char* fn = "call_dequantize_gemv_w4a16_ws";
+  if (workspace_bytes && !Workspace) DQ_FAIL("%s: Workspace is expected to have non-NULL data pointer", fn);
+  if (Workspace && !aligned16(Workspace)) DQ_FAIL("%s: Workspace must be 16-byte aligned", fn);
+  return gemv_w4a16(fn, A, B, Scale, Zeros, C, M, N, K, group, mode, layout, variant, workspace_bytes ? Workspace : nullptr,
+                    workspace_bytes, stream);
 }
 
 extern "C" int call_dequantize_gemv_lowbit(const void* A, const void* B, const void* Scale, const void* Zeros, void* C,

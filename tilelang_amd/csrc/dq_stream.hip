@@ -64,11 +64,12 @@ struct StreamGeom {
 // LDS traffic and the decode work per workgroup are those of KSPLIT = 1; what the second wave per
 // SIMD buys is that one wave's MFMAs run under the other's decode and waits.
 template <int MB, int RBW, int NST, int KSPLIT, int MODE, bool APERM>
-__global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t* __restrict__ A,
-                                                                     const uint8_t* __restrict__ B,
+__global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t* __restrict__ A_all,
+                                                                     const uint8_t* __restrict__ B_all,
                                                                      const half_t* __restrict__ S,
                                                                      const half_t* __restrict__ Z, half_t* __restrict__ C,
-                                                                     int M, int N, int K, int gshift, int pshift, int scale_slot_mask) {
+                                                                     float* __restrict__ Parts, int M, int N, int K, int gshift,
+                                                                     int pshift, int scale_slot_mask) {
   extern __shared__ __align__(16) unsigned char smem[];
   using G = StreamGeom<MB, RBW>;
   static_assert(KSPLIT == 1 || KSPLIT == 2, "one or two waves per SIMD");
@@ -98,7 +99,20 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   const int n0 = blockIdx.x * kRowsPerWg;
   const int m0 = blockIdx.y * (16 * MB);
   const int mrows = min(M - m0, 16 * MB);
-  const int KS = K / kStepK;
+  // K split across workgroups (gridDim.z slices): slice z takes a run of whole steps that starts where a chunk of
+  // scales starts, and leaves its fp32 sums in Parts[z][M][N]; w4a16_splitk_sum_kernel adds the slices up in a fixed
+  // order.  For matrices with too few rows to give every CU a workgroup.
+  int s0 = 0, KS = K / kStepK;
+  if (gridDim.z > 1) {
+    const int unit = (K >> gshift) < 8 ? 1 : (1 << pshift);  // steps per chunk of scales (short rows: one chunk for all)
+    const int units = (KS + unit - 1) / unit;
+    const int u0 = units * (int)blockIdx.z / (int)gridDim.z, u1 = units * ((int)blockIdx.z + 1) / (int)gridDim.z;
+    s0 = u0 * unit;
+    KS = min(u1 * unit, KS) - s0;
+  }
+  const int k0 = s0 * kStepK;
+  const half_t* const A = A_all + k0;
+  const uint8_t* const B = B_all + (k0 >> 1);
   // Group size 2^gshift (32 .. K): a row's 16 bytes of scales (eight groups) cover 2^pshift steps of 256 k, travel
   // once per that many steps and live in a ring of scale_slot_mask + 1 slots (the launcher sizes it).
   const int groups_per_row = max(K >> gshift, 1);  // one group per row: any shift that maps every k to group 0
@@ -134,10 +148,12 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
   const unsigned char* s_src = reinterpret_cast<const unsigned char*>((wn >= 2 && kZeros) ? Z : S);
   // the last chunk of a row whose scales are not a multiple of 16 bytes reads the row's last 16 bytes instead of
   // running past its end, and the readers shift their offset by the same amount
-  auto scale_src_off = [&](int g4) { return short_rows ? 0 : min(g4 * 16, row_bytes - 16); };
+  // (positions inside a row count from the row's first scale, wherever the workgroup's K slice starts)
+  const int slice_off = (k0 >> gshift) << 1;
+  auto scale_src_off = [&](int g4) { return short_rows ? 0 : min(slice_off + g4 * 16, row_bytes - 16); };
   auto scale_base = [&](int step) -> const unsigned char* {
     const int g4 = step >> pshift;
-    return smem + kRing + (g4 & scale_slot_mask) * G::kScaleSlot + ((((step * 256) >> gshift) << 1) - scale_src_off(g4));
+    return smem + kRing + (g4 & scale_slot_mask) * G::kScaleSlot + ((((k0 + step * 256) >> gshift) << 1) - scale_src_off(g4));
   };
 
   // DMA instruction `op` of the stage of `step`, into ring slot `slot`: the weights, the activations, and (op == kOps,
@@ -368,6 +384,17 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
       const int n = n0 + wn * (16 * RBW) + rb * 16 + g * 4;
       if (m >= mrows || n >= N) continue;
       const float4_t v = acc[rb][mb];
+      if (gridDim.z > 1) {  // a K slice: fp32, summed up afterwards
+        float* dst = Parts + ((size_t)blockIdx.z * M + (m0 + m)) * N + n;
+        if (((N & 3) == 0) && n + 3 < N) {
+          *reinterpret_cast<float4_t*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) dst[i] = v[i];
+        }
+        continue;
+      }
       half_t* dst = C + (size_t)(m0 + m) * N + n;
       if (((N & 3) == 0) && n + 3 < N) {
         typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
@@ -381,9 +408,28 @@ __global__ __launch_bounds__(256 * KSPLIT) void w4a16_stream_kernel(const half_t
     }
 }
 
+// C[i] = fp16(Parts[0][i] + Parts[1][i] + ...), in that order
+__global__ __launch_bounds__(256) void w4a16_splitk_sum_kernel(const float* __restrict__ parts, half_t* __restrict__ C, size_t count,
+                                                                int split) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i + 3 < count) {
+    float4_t v = *reinterpret_cast<const float4_t*>(parts + i);
+    for (int z = 1; z < split; ++z) v = v + *reinterpret_cast<const float4_t*>(parts + (size_t)z * count + i);
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    const half4_t o = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+    *reinterpret_cast<half4_t*>(C + i) = o;
+  } else {
+    for (size_t j = i; j < count; ++j) {
+      float v = parts[j];
+      for (int z = 1; z < split; ++z) v += parts[(size_t)z * count + j];
+      C[j] = (half_t)v;
+    }
+  }
+}
+
 template <int MB, int RBW, int NST, int KSPLIT>
 int launch_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group, int mode,
-                  int layout, hipStream_t stream) {
+                  int layout, int split, void* parts, hipStream_t stream) {
   constexpr int kRingBytes = NST * StreamGeom<MB, RBW>::kStage;
   constexpr int kRowsPerWg = StreamGeom<MB, RBW>::kRowsPerWg;
   constexpr int kMaxLds = 160 * 1024;
@@ -407,15 +453,19 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
     mask = slots - 1;
   }
   const int lds = kRingBytes + (mask + 1) * StreamGeom<MB, RBW>::kScaleSlot;
-  const dim3 grid((N + kRowsPerWg - 1) / kRowsPerWg, (M + 16 * MB - 1) / (16 * MB));
+  const dim3 grid((N + kRowsPerWg - 1) / kRowsPerWg, (M + 16 * MB - 1) / (16 * MB), split);
   const dim3 block(256 * KSPLIT);
+  if (split > 1) {  // every slice needs a step, and a slice's 4-element rows of fp32 must be 16-byte aligned
+    const int unit = (K >> gshift) < 8 ? 1 : (1 << pshift);  // as the kernel cuts K
+    if ((K / kStepK + unit - 1) / unit < split || ((size_t)M * N) % 4 != 0 || !parts) return 1;
+  }
 #define DQ_LAUNCH2(MODE_, APERM_)                                                                                    \
   do {                                                                                                               \
     auto kern = w4a16_stream_kernel<MB, RBW, NST, KSPLIT, MODE_, APERM_>;                                            \
     static bool lds_limit_raised[kMaxDevices];                                                                       \
     if (raise_lds_limit<kMaxLds>(kern, lds_limit_raised)) return -1;                                                 \
     hipLaunchKernelGGL(kern, grid, block, lds, stream, (const half_t*)A, (const uint8_t*)B, (const half_t*)S,        \
-                       (const half_t*)Z, (half_t*)C, M, N, K, gshift, pshift, mask);                                         \
+                       (const half_t*)Z, (half_t*)C, (float*)parts, M, N, K, gshift, pshift, mask);                                         \
   } while (0)
 #define DQ_LAUNCH_MODE(MODE_)                              \
   do {                                                     \
@@ -436,6 +486,12 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 #undef DQ_LAUNCH_MODE
 #undef DQ_LAUNCH2
   DQ_CHECK_HIP(hipGetLastError());
+  if (split > 1) {
+    const size_t count = (size_t)M * N;
+    hipLaunchKernelGGL(w4a16_splitk_sum_kernel, dim3((unsigned)((count + 1023) / 1024)), dim3(256), 0, stream, (const float*)parts,
+                       (half_t*)C, count, split);
+    DQ_CHECK_HIP(hipGetLastError());
+  }
   return 0;
 }
 
@@ -449,20 +505,20 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 // 128 when the mode reads scales, K a multiple of 256, and every operand below 4 GiB (32-bit
 // lane offsets).
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
-                 int mode, int layout, int config, hipStream_t stream) {
+                 int mode, int layout, int config, int split, void* parts, hipStream_t stream) {
   if (K % kStepK != 0 || N < 1 || M < 1) return 1;
   // scales travel 16 bytes of a row at a time: group sizes 32, 64, ... (powers of two that divide K), or one group per row
   if (mode >= W4_SCALE && group != K && (group < 32 || group > K || (group & (group - 1)) != 0 || K % group != 0)) return 1;
   if ((size_t)N * K / 2 >= (1ull << 32) || (size_t)M * K * 2 >= (1ull << 32)) return 1;
   switch (config) {
-    case 0: return launch_stream<1, 2, 6, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 1: return launch_stream<2, 2, 4, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 2: return launch_stream<4, 2, 3, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 3: return launch_stream<1, 1, 4, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 4: return launch_stream<2, 1, 3, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 5: return launch_stream<1, 1, 6, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 6: return launch_stream<4, 2, 3, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
-    case 7: return launch_stream<3, 2, 3, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, stream);
+    case 0: return launch_stream<1, 2, 6, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 1: return launch_stream<2, 2, 4, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 2: return launch_stream<4, 2, 3, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 3: return launch_stream<1, 1, 4, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 4: return launch_stream<2, 1, 3, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 5: return launch_stream<1, 1, 6, 1>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 6: return launch_stream<4, 2, 3, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
+    case 7: return launch_stream<3, 2, 3, 2>(A, B, S, Z, C, M, N, K, group, mode, layout, split, parts, stream);
     default: DQ_FAIL("w4a16 stream kernel: unknown configuration %d", config);
   }
 }

@@ -181,7 +181,18 @@ def dequantize_gemv(
         params.append(zparam)
     c_idx = len(params)
     params.append(KernelParam("C", torch.float16, (M, N)))
+    # Few rows and a long K: the library cuts K over workgroups when it is given room for the slices' fp32 sums (the
+    # reference's split-K kernels allocate theirs inside the kernel function,
+    # examples/dequantize_gemm/example_dequant_gemm_fp4_hopper.py:141).
+    ws_bytes = 0
+    if variant < 0 and not weight_fragments:
+        ws_bytes = int(_lib.load_library().dq_w4a16_workspace_bytes(M, N, K, group_size, mode))
+    workspace_idx = []
+    if ws_bytes:
+        workspace_idx.append(len(params))
+        params.append(KernelParam("Workspace", torch.uint8, (ws_bytes,)))
     if zwork is not None:
+        workspace_idx.append(len(params))
         params.append(zwork)
 
     def launch(ptrs, stream):
@@ -193,9 +204,12 @@ def dequantize_gemv(
             if lib.call_unpack_qzeros(z, ptrs[-1], N, groups, zfmt, stream) != 0:
                 return -1
             z = ptrs[-1]
+        if ws_bytes:
+            return lib.call_dequantize_gemv_w4a16_ws(a, b, s, z, ptrs[c_idx], ptrs[c_idx + 1], ws_bytes, M, N, K, group_size,
+                                                     mode, layout, variant, stream)
         return lib.call_dequantize_gemv_w4a16(a, b, s, z, ptrs[c_idx], M, N, K, group_size, mode, layout, variant, stream)
 
-    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error, workspace_idx=[-1] if zwork is not None else [])
+    return KernelAdapter("dequantize_gemv", params, [], launch, _lib.last_error, workspace_idx=workspace_idx)
 
 
 def _dequantize_gemv_int8(M, N, K, out_dtype, accum_dtype, num_bits, storage_dtype, source_format, fast_decoding,
