@@ -26,7 +26,9 @@
 //     (two sub-steps deep, across the step boundary), so that a wave's MFMAs issue among the VALU work
 //     of its next sub-step.
 //
-// K is not split: every wave owns its output tile, results are bit-identical from run to run.
+// Every wave owns its output tile.  Asked for by the launcher (matrices with too few rows to give every CU a
+// workgroup), K is cut into gridDim.z slices whose fp32 sums a second kernel adds in slice order: with or without
+// the split no atomics, and results bit-identical from run to run.
 #include <type_traits>
 
 #include "dq_common.h"
@@ -500,10 +502,10 @@ int launch_stream(const void* A, const void* B, const void* S, const void* Z, vo
 // config 0, 1, 2: 16, 32, 64 activation rows and 128 weight rows per workgroup; 3, 4, 5: 16, 32, 16
 // activation rows and 64 weight rows; 6: as 2 with eight waves (measured at N = 28672, K = 8192, M = 64:
 // 60 us against 63 us; the eight-wave forms of 0 and 1 were slower than the four-wave ones and are
-// not built).  Returns 1 when the shape is not
-// covered (the caller falls back to a kernel without these restrictions): the group size must be
-// 128 when the mode reads scales, K a multiple of 256, and every operand below 4 GiB (32-bit
-// lane offsets).
+// not built); 7: as 6 on three blocks of 16 activation rows.  `split` > 1: K in that many slices, fp32 partial
+// sums in parts[split][M][N].  Returns 1 when the shape is not covered (the caller falls back to a kernel without
+// these restrictions): the group size must be a power of two from 32 on or K when the mode reads scales, K a
+// multiple of 256, every operand below 4 GiB (32-bit lane offsets), every slice at least a chunk of scales long.
 int w4a16_stream(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
                  int mode, int layout, int config, int split, void* parts, hipStream_t stream) {
   if (K % kStepK != 0 || N < 1 || M < 1) return 1;
