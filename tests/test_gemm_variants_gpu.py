@@ -458,6 +458,59 @@ def test_bitnet_fragment_ordered_weights_where_no_kernel_reads_them(cuda):
     assert "the tiled kernel reads fragment-ordered weights from" in tl._lib.last_error()
 
 
+@pytest.mark.parametrize("convention", ["unsigned", "offset", "twos"])
+@pytest.mark.parametrize("M,N,K", [(5, 128, 4096), (32, 300, 8192), (17, 1001, 2048), (8, 33, 256), (31, 64, 1280), (16, 4100, 6912),
+                                   (1, 8, 512), (24, 9000, 2560), (32, 8300, 6144),
+                                   # three and four blocks of 32 weight rows per workgroup: both sets of weight registers
+                                   (9, 20000, 1024), (32, 28677, 8192)])
+@pytest.mark.parametrize("interleaved", [True, False])
+def test_bitnet_register_resident_kernel_exact(cuda, convention, M, N, K, interleaved):
+    """The small-batch kernel that keeps the activations in registers (the library's choice from 5 to 32 rows up to
+    K = 8192), named explicitly so that one row and ragged shapes reach it: K slices of unequal length over the eight
+    waves (K = 1280: five pairs of 128-k blocks for eight waves; 256: one), every int32 entry against the
+    integer oracle, all codes, the int8 range of A including -128; the fused BitLinear epilogue against the tiled
+    kernel's bits; fragment-ordered weights where the factory takes them."""
+    rng = np.random.default_rng(M + K + 2)
+    A = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    B = rng.integers(0, 256, size=(N, K // 4), dtype=np.uint8)
+    s_a = torch.tensor(rng.uniform(0.5, 3.0, size=M).astype(np.float32), device=cuda)
+    C = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+    Bdev = _dev(B, cuda).view(torch.int8)
+    if interleaved:
+        Bdev = quantize.interleave_weight(Bdev, 2, "int8")
+    print(f"bitnet register-resident: M={M} N={N} K={K} {convention} interleaved={interleaved}", flush=True)
+    tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention=convention, kernel="resident")(_dev(A, cuda), Bdev, C)
+    out = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="resident")(_dev(A, cuda), Bdev, s_a)
+    out_tiled = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="tiled")(_dev(A, cuda), Bdev, s_a)
+    torch.cuda.synchronize()
+    ft = np.float32 if K * 384 < (1 << 24) else np.float64  # exact in floating point, see the fragment test above
+    ref = (A.astype(ft) @ orc.decode_i2(B, convention).astype(ft).T).astype(np.int64)
+    rows, cols = np.arange(0, M, max(1, M // 5)), np.arange(0, N, max(1, N // 11))
+    np.testing.assert_array_equal(ref[np.ix_(rows, cols)], A[rows].astype(np.int64) @ orc.decode_i2(B[cols], convention).astype(np.int64).T)
+    np.testing.assert_array_equal(C.cpu().numpy().astype(np.int64), ref)
+    assert torch.equal(out.view(torch.int16), out_tiled.view(torch.int16))
+    if K % 2048 == 0:
+        Bfrag = quantize.prepack_i2_fragments(Bdev)
+        Cf = torch.full((M, N), -7, dtype=torch.int32, device=cuda)
+        tl.bitnet_158_int8xint2_prefill(M, N, K, fast_decoding=interleaved, convention=convention, kernel="resident",
+                                        weight_fragments=True)(_dev(A, cuda), Bfrag, Cf)
+        out_f = tl.bitlinear_int8xint2(M, N, K, 1.7, convention=convention, interleaved=interleaved, kernel="resident",
+                                       weight_fragments=True)(_dev(A, cuda), Bfrag, s_a)
+        torch.cuda.synchronize()
+        assert torch.equal(Cf, C)
+        assert torch.equal(out_f.view(torch.int16), out.view(torch.int16))
+
+
+def test_bitnet_register_resident_kernel_refuses_what_does_not_fit_its_registers(cuda):
+    A = torch.zeros((33, 16384), dtype=torch.int8, device=cuda)
+    B = torch.zeros((128, 4096), dtype=torch.int8, device=cuda)
+    C = torch.zeros((33, 128), dtype=torch.int32, device=cuda)
+    with pytest.raises(RuntimeError, match="register-resident kernel needs"):
+        tl.bitnet_158_int8xint2_prefill(33, 128, 4096, convention="offset", kernel="resident")(A[:, :4096].contiguous(), B[:, :1024].contiguous(), C)
+    with pytest.raises(RuntimeError, match="register-resident kernel needs"):
+        tl.bitnet_158_int8xint2_prefill(32, 128, 16384, convention="offset", kernel="resident")(A[:32].contiguous(), B, C[:32].contiguous())
+
+
 def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):
     A = torch.zeros((64, 1024), dtype=torch.int8, device=cuda)
     B = torch.zeros((128, 256), dtype=torch.int8, device=cuda)

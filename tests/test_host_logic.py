@@ -235,9 +235,9 @@ def test_kernels_refuse_cpu_tensors_and_bad_factory_arguments():
     assert kern.params[1].shape == (32, 64)
     with pytest.raises(AssertionError):
         tl.dequantize_gemv(1, 64, 256, trans_A=True)
-    with pytest.raises(ValueError, match="kernel must be None, 'ksliced' or 'tiled'"):
+    with pytest.raises(ValueError, match="kernel must be None, 'ksliced', 'tiled' or 'resident'"):
         tl.bitnet_158_int8xint2_prefill(256, 8192, 8192, kernel="sliced")
-    with pytest.raises(ValueError, match="kernel must be None, 'ksliced' or 'tiled'"):
+    with pytest.raises(ValueError, match="kernel must be None, 'ksliced', 'tiled' or 'resident'"):
         tl.bitlinear_int8xint2(256, 8192, 8192, 1.0, kernel="both")
 
 

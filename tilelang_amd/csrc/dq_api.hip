@@ -46,6 +46,8 @@ int wlow_gemv(const void* A, const void* B, const void* Scale, const void* Zeros
               int bits, int convention, int layout, int zeros_rescale, hipStream_t stream);
 int i2_gemm_kslice(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
                    float s_w, int bitnet_epilogue, int force, hipStream_t stream);
+int i2_gemm_regres(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
+                   float s_w, int bitnet_epilogue, hipStream_t stream);
 int i2_gemv(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
             float s_w, int out_kind, hipStream_t stream);
 int i4_gemv(const void* A, const void* B, void* C, int M, int N, int K, int decode, hipStream_t stream);
@@ -434,10 +436,11 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   const int word_layout = layout & ~LAYOUT_FRAGMENTS;
   if (word_layout != LAYOUT_PLAIN && word_layout != LAYOUT_INTERLEAVED) DQ_FAIL("%s: unknown weight layout %d", fn, layout);
   // bits 4 and 5 of out_kind name a kernel (tests and measurements): K sliced over the waves / the tiled GEMM
-  int kernel_choice = out_kind & (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
-  out_kind &= ~(DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED);
+  constexpr int kChoices = DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED | DQ_I2_KERNEL_RESIDENT;
+  int kernel_choice = out_kind & kChoices;
+  out_kind &= ~kChoices;
   if (out_kind != 0 && out_kind != 1) DQ_FAIL("%s: out_kind must be 0 (int32) or 1 (fp16 BitLinear epilogue)", fn);
-  if (kernel_choice == (DQ_I2_KERNEL_KSLICED | DQ_I2_KERNEL_TILED)) DQ_FAIL("%s: out_kind names two kernels", fn);
+  if (kernel_choice & (kernel_choice - 1)) DQ_FAIL("%s: out_kind names two kernels", fn);
   if (out_kind == 1 && !s_a) DQ_FAIL("%s: s_a is expected to have non-NULL data pointer", fn);
   if (out_kind == 1 && !(s_w != 0.f)) DQ_FAIL("%s: s_w must be non-zero", fn);
   const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
@@ -446,8 +449,23 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
     if (rc > 0) DQ_FAIL("%s: the K-sliced kernel needs K %% 2048 == 0, K < 131072 and operands below 4 GiB (got M=%d N=%d K=%d)", fn, M, N, K);
     return rc;
   }
+  if (kernel_choice == DQ_I2_KERNEL_RESIDENT) {
+    const int rc = i2_gemm_regres(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+    if (rc > 0) DQ_FAIL("%s: the register-resident kernel needs M <= 32, K %% 256 == 0 and K <= 8192 (got M=%d N=%d K=%d)", fn, M, N, K);
+    return rc;
+  }
+  // 4 to 32 rows: activations resident in registers, weights streamed once (at 4 rows already ahead of the dot-product
+  // kernel: N = 28672, K = 8192 18.4 against 19.5 us, fragment-ordered 14.8 against 25.2)
+  if (M >= 4 && M <= 32 && !kernel_choice) {
+    const int rc = i2_gemm_regres(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
   if (M <= 4 && !kernel_choice) {  // decode: the streaming dot4 kernel (row-major or fragment-ordered weights)
     const int rc = i2_gemv(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
+  if (M < 4 && !kernel_choice) {  // one to three rows of a shape the dot-product kernel does not take
+    const int rc = i2_gemm_regres(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
   if (!kernel_choice) {  // a few hundred rows: K sliced over the waves of a workgroup

@@ -46,6 +46,7 @@
 #include <utility>
 
 #include "dq_common.h"
+#include "dq_i2_codes.h"
 
 namespace dq {
 
@@ -91,44 +92,6 @@ __device__ __forceinline__ void wait_loads(uint4_t (&w)[2][kWOps]) {
                : "n"(N)
                : "memory");
 }
-
-template <int CONV>
-struct Codes {
-  static constexpr int kShift = CONV == I2_UNSIGNED ? 0 : 6;  // the accumulators hold 2^kShift x the sum
-};
-
-// One packed dword (16 codes; interleaved words: the codes of elements 4 i .. 4 i + 3 at bit 2 i of bytes 0 .. 3) ->
-// dword i of the operand.
-template <int CONV>
-__device__ __forceinline__ int4_t decode16(uint32_t w) {
-  int4_t o;
-  if constexpr (CONV == I2_UNSIGNED) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = (int)((w >> (2 * i)) & 0x03030303u);
-  } else {
-    // offset binary: flipping the code's top bit after the mask is one three-input bit operation with it
-    constexpr uint32_t flip = CONV == I2_OFFSET ? 0x80808080u : 0u;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = (int)(((w << (6 - 2 * i)) & 0xC0C0C0C0u) ^ flip);
-  }
-  return o;
-}
-
-struct BitnetFinish {
-  using out_t = half_t;
-  const float* s_a;
-  float s_w;
-  __device__ __forceinline__ out_t operator()(int acc, int m) const {
-    float v = (float)acc;
-    v = v / s_a[m];
-    v = v / s_w;
-    return (half_t)v;
-  }
-};
-struct Int32Finish {
-  using out_t = int32_t;
-  __device__ __forceinline__ out_t operator()(int acc, int) const { return acc; }
-};
 
 template <int CONV, bool IL, bool FRAG, class FIN>
 __global__ __launch_bounds__(64 * kWaves, 1) void i2_kslice_kernel(const int8_t* __restrict__ A, const uint8_t* __restrict__ B,

@@ -841,7 +841,7 @@ def bitnet_158_int8xint2_prefill(
     return KernelAdapter("bitnet_158_int8xint2_prefill", params, [], launch, _lib.last_error)
 
 
-_I2_KERNELS = {None: 0, "ksliced": 16, "tiled": 32}  # DQ_I2_KERNEL_* of include/dqgemm.h
+_I2_KERNELS = {None: 0, "ksliced": 16, "tiled": 32, "resident": 64}  # DQ_I2_KERNEL_* of include/dqgemm.h
 
 
 def _i2_fragments_ok(fn: str, K: int, kernel: str | None) -> None:
@@ -853,7 +853,7 @@ def _i2_fragments_ok(fn: str, K: int, kernel: str | None) -> None:
 
 def _i2_kernel_choice(fn: str, kernel: str | None) -> int:
     if kernel not in _I2_KERNELS:
-        raise ValueError(f"{fn}: kernel must be None, 'ksliced' or 'tiled' (got {kernel!r})")
+        raise ValueError(f"{fn}: kernel must be None, 'ksliced', 'tiled' or 'resident' (got {kernel!r})")
     return _I2_KERNELS[kernel]
 
 
