@@ -218,7 +218,7 @@ enum dq_i2_convention {
  * (examples/bitnet-1.58b/kernel_benchmark/tilelang_bitnet_158_int8xint2_decode.py:196-234,249-251).
  * Replaces `call(A, B, C, stream)` of tilelang_bitnet_158_int8xint2_prefill.py:188-296 and
  * tilelang_bitnet_158_int8xint2_decode.py:66-175.  Requires K % 128 == 0.
- * The library picks the kernel by shape (M <= 4: a streaming dot-product kernel; up to 32 rows with K <= 8192: the
+ * The library picks the kernel by shape (M <= 4: a streaming dot-product kernel; up to 32 rows with K % 256 == 0: the
  * activations resident in registers and the weights streamed once; a few hundred rows on a long K:
  * K sliced over the waves of a workgroup; else the tiled GEMM).  All four read DQ_LAYOUT_FRAGMENTS; where the
  * tiled GEMM does not take a fragment-ordered problem (too few tiles) the K-sliced kernel runs it whatever its size.  For tests and measurements out_kind may carry one
@@ -226,7 +226,7 @@ enum dq_i2_convention {
 enum dq_i2_kernel {
   DQ_I2_KERNEL_KSLICED = 16, /* needs K % 2048 == 0, K < 131072; -1 where it cannot run */
   DQ_I2_KERNEL_TILED = 32,
-  DQ_I2_KERNEL_RESIDENT = 64 /* activations resident in registers: M <= 32, K % 256 == 0, K <= 8192 */
+  DQ_I2_KERNEL_RESIDENT = 64 /* activations resident in registers: M <= 32 (128 on matrices of few rows), K % 256 == 0 */
 };
 int call_gemm_int8xint2(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout,
                         const void* s_a, float s_w, int out_kind, dq_stream_t stream);

@@ -448,11 +448,11 @@ def test_bitnet_fragment_ordered_weights_where_no_kernel_reads_them(cuda):
     """Through the C-ABI: a K that neither the K-sliced nor (for want of tiles) the tiled kernel takes, and the tiled
     kernel named on a problem with too few tiles for it."""
     lib = tl._lib.get_library()
-    A = torch.zeros((64, 4096), dtype=torch.int8, device=cuda)
+    A = torch.zeros((200, 4096), dtype=torch.int8, device=cuda)
     B = torch.zeros((4, 32, 64, 16), dtype=torch.int8, device=cuda)
-    C = torch.zeros((64, 128), dtype=torch.int32, device=cuda)
+    C = torch.zeros((200, 128), dtype=torch.int32, device=cuda)
     stream = torch.cuda.current_stream().cuda_stream
-    assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 1024, 1, 2, None, 1.0, 0, stream) == -1
+    assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 200, 128, 1024, 1, 2, None, 1.0, 0, stream) == -1
     assert "no kernel takes" in tl._lib.last_error()
     assert lib.call_gemm_int8xint2(A.data_ptr(), B.data_ptr(), C.data_ptr(), 64, 128, 4096, 1, 2, None, 1.0, 32, stream) == -1
     assert "the tiled kernel reads fragment-ordered weights from" in tl._lib.last_error()
@@ -462,7 +462,11 @@ def test_bitnet_fragment_ordered_weights_where_no_kernel_reads_them(cuda):
 @pytest.mark.parametrize("M,N,K", [(5, 128, 4096), (32, 300, 8192), (17, 1001, 2048), (8, 33, 256), (31, 64, 1280), (16, 4100, 6912),
                                    (1, 8, 512), (24, 9000, 2560), (32, 8300, 6144),
                                    # three and four blocks of 32 weight rows per workgroup: both sets of weight registers
-                                   (9, 20000, 1024), (32, 28677, 8192)])
+                                   (9, 20000, 1024), (32, 28677, 8192),
+                                   # more than 32 activation rows on a matrix of few rows: passes of 32
+                                   (64, 300, 4096), (100, 1001, 2048), (128, 2560, 1280), (33, 5000, 512),
+                                   # K beyond what the registers hold: chunks of K, running sums in LDS
+                                   (8, 300, 11008), (32, 1001, 16384), (5, 9000, 28672), (17, 64, 8448), (64, 200, 12288)])
 @pytest.mark.parametrize("interleaved", [True, False])
 def test_bitnet_register_resident_kernel_exact(cuda, convention, M, N, K, interleaved):
     """The small-batch kernel that keeps the activations in registers (the library's choice from 5 to 32 rows up to
@@ -502,13 +506,20 @@ def test_bitnet_register_resident_kernel_exact(cuda, convention, M, N, K, interl
 
 
 def test_bitnet_register_resident_kernel_refuses_what_does_not_fit_its_registers(cuda):
-    A = torch.zeros((33, 16384), dtype=torch.int8, device=cuda)
+    A = torch.zeros((129, 16384), dtype=torch.int8, device=cuda)
     B = torch.zeros((128, 4096), dtype=torch.int8, device=cuda)
-    C = torch.zeros((33, 128), dtype=torch.int32, device=cuda)
+    C = torch.zeros((129, 128), dtype=torch.int32, device=cuda)
     with pytest.raises(RuntimeError, match="register-resident kernel needs"):
-        tl.bitnet_158_int8xint2_prefill(33, 128, 4096, convention="offset", kernel="resident")(A[:, :4096].contiguous(), B[:, :1024].contiguous(), C)
+        tl.bitnet_158_int8xint2_prefill(129, 128, 4096, convention="offset", kernel="resident")(A[:, :4096].contiguous(), B[:, :1024].contiguous(), C)
+    with pytest.raises(RuntimeError, match="register-resident kernel needs"):  # K % 256
+        tl.bitnet_158_int8xint2_prefill(32, 128, 8320, convention="offset", kernel="resident")(
+            A[:32, :8320].contiguous(), B[:, :2080].contiguous(), C[:32].contiguous())
+    # 64 rows against 28672 weight rows: 1792 workgroup-blocks, far beyond two rounds
+    A2 = torch.zeros((64, 256), dtype=torch.int8, device=cuda)
+    B2 = torch.zeros((28672, 64), dtype=torch.int8, device=cuda)
+    C2 = torch.zeros((64, 28672), dtype=torch.int32, device=cuda)
     with pytest.raises(RuntimeError, match="register-resident kernel needs"):
-        tl.bitnet_158_int8xint2_prefill(32, 128, 16384, convention="offset", kernel="resident")(A[:32].contiguous(), B, C[:32].contiguous())
+        tl.bitnet_158_int8xint2_prefill(64, 28672, 256, convention="offset", kernel="resident")(A2, B2, C2)
 
 
 def test_bitnet_k_sliced_kernel_refuses_what_it_cannot_slice(cuda):

@@ -451,12 +451,14 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
   }
   if (kernel_choice == DQ_I2_KERNEL_RESIDENT) {
     const int rc = i2_gemm_regres(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
-    if (rc > 0) DQ_FAIL("%s: the register-resident kernel needs M <= 32, K %% 256 == 0 and K <= 8192 (got M=%d N=%d K=%d)", fn, M, N, K);
+    if (rc > 0) DQ_FAIL("%s: the register-resident kernel needs M <= 32 (on matrices of few rows M <= 128) and K %% 256 == 0 (got M=%d N=%d K=%d)", fn, M, N, K);
     return rc;
   }
-  // 4 to 32 rows: activations resident in registers, weights streamed once (at 4 rows already ahead of the dot-product
-  // kernel: N = 28672, K = 8192 18.4 against 19.5 us, fragment-ordered 14.8 against 25.2)
-  if (M >= 4 && M <= 32 && !kernel_choice) {
+  // 4 to 32 rows: activations resident in registers, weights streamed once (at 4 rows ahead of the dot-product kernel
+  // on fragment-ordered weights, N = 28672, K = 8192: 14.8 against 25.2 us, and on row-major ones from about 6000
+  // weight rows on: N = 11008, K = 4096 7.3 against 8.7 us, N = 3072, K = 8192 8.6 against 7.1)
+  const bool four_rows_resident = frag || N >= 6144 || (size_t)M * K > 32768;
+  if ((M > 4 || (M == 4 && four_rows_resident)) && M <= 128 && !kernel_choice) {  // beyond 32 rows: on small matrices only (the kernel says which)
     const int rc = i2_gemm_regres(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
@@ -464,7 +466,7 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
     const int rc = i2_gemv(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
-  if (M < 4 && !kernel_choice) {  // one to three rows of a shape the dot-product kernel does not take
+  if (M <= 4 && !kernel_choice) {  // one to four rows of a shape the dot-product kernel does not take
     const int rc = i2_gemm_regres(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, (hipStream_t)stream);
     if (rc <= 0) return rc;
   }
@@ -480,8 +482,9 @@ extern "C" int call_gemm_int8xint2(const void* A, const void* B, void* C, int M,
     DQ_FAIL("%s: the tiled kernel reads fragment-ordered weights from 160 tiles of 128 x 256 on and K %% 256 == 0 (got M=%d N=%d K=%d)", fn, M, N, K);
   const int rck = i2_gemm_kslice(A, B, C, M, N, K, convention, layout, s_a, s_w, out_kind, 1, (hipStream_t)stream);
   if (rck > 0)
-    DQ_FAIL("%s: fragment-ordered weights: no kernel takes M=%d N=%d K=%d (decode: M <= 4 and M * K <= 32768; K-sliced: K %% 2048 == 0; "
-            "tiled: 160 tiles of 128 x 256 and K %% 256 == 0)", fn, M, N, K);
+    DQ_FAIL("%s: fragment-ordered weights: no kernel takes M=%d N=%d K=%d (decode: M <= 4 and M * K <= 32768; register-resident: "
+            "M <= 32, or 128 on a matrix of few rows, and K %% 256 == 0; K-sliced: K %% 2048 == 0; tiled: 160 tiles of "
+            "128 x 256 and K %% 256 == 0)", fn, M, N, K);
   return rck;
 }
 

@@ -1,4 +1,4 @@
-// BitNet W2A8 small batch (5 .. 32 activation rows) on gfx950: activations resident in registers, weights streamed once.
+// BitNet W2A8 small batch (4 .. 32 activation rows; to 128 on matrices of few rows) on gfx950: activations resident in registers, weights streamed once.
 //
 // Replaces the batched use of the decode kernel of
 // examples/bitnet-1.58b/kernel_benchmark/tilelang_bitnet_158_int8xint2_decode.py:66-176 (decoder
@@ -10,7 +10,8 @@
 //
 //   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of whole pairs of 128-k blocks, at most
 //     four pairs: K <= 8192) and keeps the activations of its slice, in the matrix instruction's operand order, in
-//     registers for the whole kernel: 32 rows x 1024 k = 128 registers per lane;
+//     registers for the whole kernel: 32 rows x 1024 k = 128 registers per lane.  A longer K goes in chunks of at
+//     most 6144, the kernel's body once per chunk, the finishing threads' running sums in LDS in between;
 //   * the workgroups walk the blocks of 32 weight rows (block b, b + gridDim.x, ...).  Per block a wave loads its
 //     slice of the 32 rows (eight 16-byte loads per lane at K = 8192), one block ahead of the arithmetic in a second
 //     set of registers, decodes (7 instructions per 16 weights) and issues 32 matrix instructions of 32 x 32 x 32
@@ -38,28 +39,46 @@ namespace {
 
 constexpr int kWaves = 8;             // K slices
 constexpr int kMaxPairs = 4;          // pairs of 128-k blocks per wave
+constexpr int kChunkPairs = 3;        // the same when K goes in chunks
 constexpr int kPartial = 32 * 32 * 4; // one wave's 32 x 32 sums
 constexpr int kLds = 2 * kWaves * kPartial;
+constexpr int kMaxRunning = 8;       // blocks of a workgroup whose running sums fit behind them (N <= 65536)
 
-template <int CONV, bool FRAG, int NPW, class FIN>
-__global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t* __restrict__ A, const uint8_t* __restrict__ B,
-                                                                   typename FIN::out_t* __restrict__ C, int M, int N, int K,
+template <int CONV, bool FRAG, int NPW, bool CHUNKED, class FIN>
+__global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t* __restrict__ A_all, const uint8_t* __restrict__ B,
+                                                                   typename FIN::out_t* __restrict__ C_all, int M_all, int N, int K,
                                                                    int interleaved, FIN fin) {
   extern __shared__ __align__(16) unsigned char smem[];
+  // more than 32 activation rows (small matrices only, see the launcher): workgroup row blockIdx.y takes rows
+  // 32 blockIdx.y .. + 31 over all of the weights
+  const int m_first = 32 * blockIdx.y;
+  const int8_t* const A = A_all + (size_t)m_first * K;
+  typename FIN::out_t* const C = C_all + (size_t)m_first * N;
+  const int M = min(M_all - m_first, 32);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31;
   const int h = lane >> 5;
 
+  // K beyond what the registers hold (8192): the kernel runs once per chunk of K, chunks of equal length up to a
+  // pair; the finishing threads keep the running sums of the workgroup's blocks in LDS between the chunks.
+  const int npair_all = K >> 8;
+  const int nchunks = CHUNKED ? (npair_all + kWaves * NPW - 1) / (kWaves * NPW) : 1;
+  const int row_blocks = (N + 31) >> 5;
+  const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
+  int it = 0;
+  for (int chunk = 0; chunk < nchunks; ++chunk) {
+  const int it0 = it;
+  if (chunk > 0) __syncthreads();  // the partial sums of the chunk before are read: their place is free
   // the wave's pairs of blocks: [p_lo, p_lo + npw), npw = NPW or NPW - 1
-  const int npair = K >> 8;
-  const int p_lo = wave * npair / kWaves;
-  const int npw = (wave + 1) * npair / kWaves - p_lo;
+  const int c_lo = chunk * npair_all / nchunks;
+  const int npair = (chunk + 1) * npair_all / nchunks - c_lo;
+  const int p_lo = c_lo + wave * npair / kWaves;
+  const int npw = c_lo + (wave + 1) * npair / kWaves - p_lo;
   auto pair_of = [&](int i) { return p_lo + min(i, max(npw - 1, 0)); };  // K < 2048: some waves have no pair at all
 
   // ---- weights: load (pair i, o) of the block of 32 rows nb
-  const int row_blocks = (N + 31) >> 5;
   uint32_t w_off[NPW][2];
 #pragma unroll
   for (int i = 0; i < NPW; ++i)
@@ -85,7 +104,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
   // prologue
   uint4_t w0[NPW][2], w1[NPW][2];
   int nb = blockIdx.x;
-  const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
   load_w(w0, nb);
 
   // ---- activations: fragment (pair i, block b, step s): lane (r, h) holds k = 256 pair + 128 b + 64 h + 16 s .. + 15 of row r.
@@ -152,7 +170,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
   // the thread's share of the final sum: activation row tid / 8, weight rows 4 (tid % 8) .. + 3 of the block
   const int out_m = tid >> 3, out_p = tid & 7;
   const bool finisher = tid < 256 && out_m < M;
-  const typename FIN::row_t out_row = fin.row(finisher ? out_m : 0);
+  const typename FIN::row_t out_row = fin.row(finisher ? m_first + out_m : 0);
 
   auto do_block = [&](uint4_t (&w)[NPW][2], int nb, int it) __attribute__((always_inline)) {
     int16_t_ acc;
@@ -194,10 +212,14 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
       int4_t sum = {0, 0, 0, 0};
 #pragma unroll
       for (int w8 = 0; w8 < kWaves; ++w8) sum += *reinterpret_cast<const int4_t*>(buf + w8 * kPartial + m * 128 + ((p ^ (m & 7)) << 4));
+      // the running sum of this thread's four outputs of the workgroup's block number it - it0, behind the buffers
+      int4_t* const running = reinterpret_cast<int4_t*>(smem + kLds + (it - it0) * kPartial + m * 128 + p * 16);
+      if (chunk > 0) sum += *running;
+      if (chunk + 1 < nchunks) *running = sum;
       using out_t = typename FIN::out_t;
       constexpr int kShift = Codes<CONV>::kShift;
       const int n = 32 * nb + 4 * p;
-      if (n < N) {
+      if (chunk + 1 == nchunks && n < N) {
         out_t o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = fin.finish(sum[e] >> kShift, out_row);
@@ -219,7 +241,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
   // count the loads in flight for the path without it, and wait for the block ahead before it computes.
   // (Asking for block nb + 2 gridDim.x pair by pair as block nb's registers come free needs copies of them that no
   // longer fit the 256 registers: the kernel then spills.)
-  int it = 0;
   for (;;) {
     if (nb + step >= row_blocks) {
       do_block(w0, nb, it);
@@ -238,13 +259,15 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
     nb += step;
     ++it;
   }
+  ++it;  // the last block's
+  }  // chunks of K
 }
 
-template <int CONV, bool FRAG, int NPW, class FIN>
+template <int CONV, bool FRAG, int NPW, bool CHUNKED, class FIN>
 int launch_i2_regres(const void* A, const void* B, void* C, int M, int N, int K, int interleaved, FIN fin, hipStream_t stream) {
-  auto kern = i2_regres_kernel<CONV, FRAG, NPW, FIN>;
+  auto kern = i2_regres_kernel<CONV, FRAG, NPW, CHUNKED, FIN>;
   static bool raised[kMaxDevices] = {};
-  if (raise_lds_limit<kLds>(kern, raised)) return -1;
+  if (raise_lds_limit<kLds + kMaxRunning * kPartial>(kern, raised)) return -1;
   static int cus_of[kMaxDevices] = {};
   int device = 0;
   DQ_CHECK_HIP(hipGetDevice(&device));
@@ -252,8 +275,17 @@ int launch_i2_regres(const void* A, const void* B, void* C, int M, int N, int K,
   if (!cus_of[device]) DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
   const int cus = cus_of[device];
   const int row_blocks = (N + 31) / 32;
+  const int passes = (M + 31) / 32;
+  // see i2_gemm_regres: one round of workgroups, or one and a half when K is short enough for one chunk (N = 3072,
+  // K = 8192 at 128 rows: 17.6 us against 24.6 us of the K-sliced kernel; N = 8192, K = 28672 at 64 rows, two full
+  // rounds of chunked work: 67 against 58 us)
+  if (passes > 1 && (long)row_blocks * passes > (CHUNKED ? 2L : 3L) * cus / 2) return 1;
   const int grid = row_blocks < cus ? row_blocks : cus;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWaves), kLds, stream, (const int8_t*)A, (const uint8_t*)B,
+  // K in chunks: the running sums of a workgroup's blocks live behind the two buffers of partial sums
+  const int mine = (row_blocks + grid - 1) / grid;
+  if (CHUNKED && mine > kMaxRunning) return 1;
+  const int lds = kLds + (CHUNKED ? mine * kPartial : 0);
+  hipLaunchKernelGGL(kern, dim3(grid, passes), dim3(64 * kWaves), lds, stream, (const int8_t*)A, (const uint8_t*)B,
                      (typename FIN::out_t*)C, M, N, K, interleaved, fin);
   DQ_CHECK_HIP(hipGetLastError());
   return 0;
@@ -265,25 +297,34 @@ int launch_i2_regres(const void* A, const void* B, void* C, int M, int N, int K,
 int i2_gemm_regres(const void* A, const void* B, void* C, int M, int N, int K, int convention, int layout, const void* s_a,
                    float s_w, int bitnet_epilogue, hipStream_t stream) {
   // whole pairs of 128-k blocks, at most four per wave; the rows of one block of the matrix instruction
-  if (M < 1 || M > 32 || K % 256 != 0 || K > kWaves * kMaxPairs * 256) return 1;
+  // More than 32 rows: every 32 of them stream the weights again, which pays while the whole of it is about one
+  // round of workgroups, i.e. on matrices of few rows, where the kernels for hundreds of activation rows have a
+  // handful of tiles (N = 4096, K = 4096 at 64 rows: 14.9 us there, 6.5 us here); the launcher returns 1 beyond that.
+  if (M < 1 || M > 128 || K % 256 != 0) return 1;
   if ((uint64_t)(N + 32) * (uint64_t)(K >> 2) >= (1ull << 32)) return 1;  // 32-bit lane offsets inside a row block's loads
-  const int npw = ((K >> 8) + kWaves - 1) / kWaves;
+  // Up to K = 8192 the activations of all of K stay in registers (one to four pairs of blocks per wave).  Beyond, K
+  // goes in chunks of at most 6144, equal up to a pair: three pairs per wave leave the registers that the chunk loop
+  // needs (with four the compiler spilled).
+  const int npair = K >> 8;
+  const bool chunked = npair > kWaves * kMaxPairs;
+  const int npw = chunked ? kChunkPairs : (npair + kWaves - 1) / kWaves;
   const int il = (layout & ~LAYOUT_FRAGMENTS) == LAYOUT_INTERLEAVED;
   const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
-#define DQ_I2R(CONV_, FRAG_, NPW_)                                                                                        \
-  do {                                                                                                                    \
-    if (bitnet_epilogue)                                                                                                  \
-      return launch_i2_regres<CONV_, FRAG_, NPW_>(A, B, C, M, N, K, il, BitnetFinish{(const float*)s_a, s_w}, stream);    \
-    return launch_i2_regres<CONV_, FRAG_, NPW_>(A, B, C, M, N, K, il, Int32Finish{}, stream);                             \
+#define DQ_I2R(CONV_, FRAG_, NPW_, CH_)                                                                                        \
+  do {                                                                                                                         \
+    if (bitnet_epilogue)                                                                                                       \
+      return launch_i2_regres<CONV_, FRAG_, NPW_, CH_>(A, B, C, M, N, K, il, BitnetFinish{(const float*)s_a, s_w}, stream);    \
+    return launch_i2_regres<CONV_, FRAG_, NPW_, CH_>(A, B, C, M, N, K, il, Int32Finish{}, stream);                             \
   } while (0)
-#define DQ_I2RN(CONV_, FRAG_)                  \
-  do {                                         \
-    switch (npw) {                             \
-      case 1: DQ_I2R(CONV_, FRAG_, 1);         \
-      case 2: DQ_I2R(CONV_, FRAG_, 2);         \
-      case 3: DQ_I2R(CONV_, FRAG_, 3);         \
-      default: DQ_I2R(CONV_, FRAG_, 4);        \
-    }                                          \
+#define DQ_I2RN(CONV_, FRAG_)                           \
+  do {                                                  \
+    if (chunked) DQ_I2R(CONV_, FRAG_, kChunkPairs, true); \
+    switch (npw) {                                      \
+      case 1: DQ_I2R(CONV_, FRAG_, 1, false);           \
+      case 2: DQ_I2R(CONV_, FRAG_, 2, false);           \
+      case 3: DQ_I2R(CONV_, FRAG_, 3, false);           \
+      default: DQ_I2R(CONV_, FRAG_, 4, false);          \
+    }                                                   \
   } while (0)
 #define DQ_I2RL(CONV_)                  \
   do {                                  \
