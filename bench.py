@@ -497,6 +497,9 @@ def main():
             row = _row(f"w4a16_zeros M={m} N=28672 K=8192", r, "hbm", MFMA_BF16_PEAK)
             row["frac_mfma"] = r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK
             shapes.append(row)
+        # a matrix of few rows and a long K: K split over workgroups, fp32 partial sums in a workspace
+        r = bench_w4a16(torch, tl, workloads, 16, 4096, 14336, True, S, W, dev)
+        shapes.append(_row("w4a16_zeros M=16 N=4096 K=14336", r, "hbm", MFMA_BF16_PEAK))
         for m in (4, 16):
             r = bench_w4a16(torch, tl, workloads, m, 28672, 8192, True, S, W, dev, fragments=True)
             shapes.append(_row(f"w4a16_zeros M={m} N=28672 K=8192 (weights re-ordered offline into the matrix instruction's operand order)",
@@ -508,9 +511,11 @@ def main():
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
         mx_run = r
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
-        for m in (1, 256, 2048):
-            r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m == 1 else gemm))
-            shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m == 1 else "mfma", MFMA_I8_PEAK))
+        for m in (1, 16, 256, 2048):
+            r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m <= 16 else gemm))
+            shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m <= 16 else "mfma", MFMA_I8_PEAK))
+        r = bench_bitnet(torch, tl, workloads, 16, 28672, 8192, S, W, dev)
+        shapes.append(_row("bitnet_w2a8 M=16 N=28672 K=8192", r, "hbm", MFMA_I8_PEAK))
         r = bench_bitnet(torch, tl, workloads, 256, 8192, 8192, S, W, dev, fragments=True, **gemm)
         shapes.append(_row("bitnet_w2a8 M=256 N=8192 K=8192 (weights re-ordered offline into the matrix instruction's operand order)",
                            r, "mfma", MFMA_I8_PEAK))

@@ -61,6 +61,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
   const int r = lane & 31;
   const int h = lane >> 5;
 
+  // the thread's share of the final sum: activation row tid / 8, weight rows 4 (tid % 8) .. + 3 of the block.  (What
+  // the epilogue needs of the row is fetched here, ahead of the activations: a load that could still be in flight
+  // when the loop over the blocks begins would have the compiler wait for the blocks ahead at its first use.)
+  const int out_m = tid >> 3, out_p = tid & 7;
+  const bool finisher = tid < 256 && out_m < M;
+  const typename FIN::row_t out_row = fin.row(finisher ? m_first + out_m : 0);
+
   // K beyond what the registers hold (8192): the kernel runs once per chunk of K, chunks of equal length up to a
   // pair; the finishing threads keep the running sums of the workgroup's blocks in LDS between the chunks.
   const int npair_all = K >> 8;
@@ -167,11 +174,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
   // w[i][b] is the operand of block b of the pair: lane (r, h) holds k = 64 h .. 64 h + 63 of row r
   const int w_from = ((lane & 15) * 4 + ((lane >> 4) & 1) * 2 + (lane >> 5)) * 4;
 
-  // the thread's share of the final sum: activation row tid / 8, weight rows 4 (tid % 8) .. + 3 of the block
-  const int out_m = tid >> 3, out_p = tid & 7;
-  const bool finisher = tid < 256 && out_m < M;
-  const typename FIN::row_t out_row = fin.row(finisher ? m_first + out_m : 0);
-
   auto do_block = [&](uint4_t (&w)[NPW][2], int nb, int it) __attribute__((always_inline)) {
     int16_t_ acc;
 #pragma unroll
@@ -263,6 +265,180 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres_kernel(const int8_t*
   }  // chunks of K
 }
 
+// ---- up to 16 activation rows -------------------------------------------------------------------------------------
+// The same kernel on the 16 x 16 x 64 matrix instruction: blocks of 16 weight rows (N = 28672 is 1792 blocks, seven
+// per workgroup, where blocks of 32 are three and a half), the activations of a wave's eighth of K in 64 registers,
+// and the registers that frees hold four blocks of weights instead of two: three blocks (96 KiB per CU) are asked for
+// ahead of the one being decoded.  A pair of 128-k blocks of 16 rows is 1 KiB: one load per lane.  Row-major: lane l
+// reads piece l % 4 of row l / 4 (whole 64-byte runs) and one ds_bpermute_b32 per dword hands lane (g, r) piece g of
+// row r; fragment order: lane (g, r) reads entry (block 2 pair + g / 2, lane 32 (g % 2) + 16 (nb % 2) + r) of the
+// 32-row fragment block nb / 2, which is that piece.  Dword s of a lane feeds step s: contraction index
+// k = 256 pair + 64 g + 16 s + e for both operands.
+// The loads of the last three blocks' turns have nothing left to ask for and read block 0 instead (the same 32 KiB
+// for every workgroup, from L2, never used): a load under a condition would make the compiler wait for more than
+// the block it needs.
+constexpr int kDepth16 = 4;               // sets of weight registers
+constexpr int kPartial16 = 16 * 16 * 4;   // one wave's 16 x 16 sums
+constexpr int kLds16 = kWaves * 4096;     // the prologue's parking areas; the two buffers of partial sums reuse them
+
+template <int CONV, bool FRAG, int NPW, class FIN>
+__global__ __launch_bounds__(64 * kWaves, 1) void i2_regres16_kernel(const int8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                                     typename FIN::out_t* __restrict__ C, int M, int N, int K,
+                                                                     int interleaved, FIN fin) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+
+  const int npair = K >> 8;
+  const int p_lo = wave * npair / kWaves;
+  const int npw = (wave + 1) * npair / kWaves - p_lo;
+  auto pair_of = [&](int i) { return p_lo + min(i, max(npw - 1, 0)); };
+
+  const int row_blocks = (N + 15) >> 4;
+  const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
+  const int nb0 = blockIdx.x;
+  const int mine = (row_blocks - nb0 + step - 1) / step;
+
+  uint32_t w_off[NPW];
+#pragma unroll
+  for (int i = 0; i < NPW; ++i)
+    w_off[i] = FRAG ? (uint32_t)((2 * pair_of(i) + (g >> 1)) * 1024 + (32 * (g & 1) + r) * 16) : (uint32_t)(pair_of(i) * 64 + (lane & 3) * 16);
+  const uint32_t row_bytes = (uint32_t)(K >> 2);
+  auto load_w = [&](uint4_t (&w)[NPW], int nb_asked, bool real) __attribute__((always_inline)) {
+    const int nb = real ? nb_asked : 0;
+    const uint8_t* base;
+    if constexpr (FRAG) base = B + (size_t)(nb >> 1) * (size_t)(K >> 7) * 1024 + (nb & 1) * 256;
+    else base = B + (size_t)min(16 * nb + (lane >> 2), N - 1) * row_bytes;
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(base + w_off[i]));
+    __builtin_amdgcn_sched_barrier(0);  // the loads go out here, see load_w of the kernel above
+  };
+  // the thread's share of the final sum: activation row tid / 4, weight rows 4 (tid % 4) .. + 3 of the block (fetched
+  // ahead of the activations, see the kernel above)
+  const int out_m = tid >> 2, out_p = tid & 3;
+  const bool finisher = tid < 64 && out_m < M;
+  const typename FIN::row_t out_row = fin.row(finisher ? out_m : 0);
+  uint4_t w[kDepth16][NPW];
+  load_w(w[0], nb0, true);
+  load_w(w[1], nb0 + step, mine > 1);
+  load_w(w[2], nb0 + 2 * step, mine > 2);
+
+  // ---- activations: fragment (pair i, step s): lane (g, r) holds k = 256 pair + 64 g + 16 s .. + 15 of row r; read as
+  // whole lines (instruction j: rows 4 j .. 4 j + 3, lane l the piece l % 16 of row 4 j + l / 16), parked in the
+  // wave's 4 KiB of LDS (piece q of row m at position q ^ m) and read back in operand order
+  int4_t af[NPW][4];
+  {
+    const int8_t* const a_lane = A + 16 * (lane & 15);
+    uint4_t line[NPW][4];
+#pragma unroll
+    for (int i = 0; i < NPW; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        line[i][j] = *reinterpret_cast<const uint4_t*>(a_lane + (size_t)min(4 * j + (lane >> 4), M - 1) * K + 256 * pair_of(i));
+    unsigned char* const park = smem + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        *reinterpret_cast<uint4_t*>(park + row * 256 + (((lane & 15) ^ row) << 4)) = line[i][j];
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        uint4_t a = *reinterpret_cast<const uint4_t*>(park + r * 256 + (((4 * g + s) ^ r) << 4));
+        if (!interleaved) a = transpose4x4_bytes(a);  // plain packing: the decoder's dword j holds elements j, 4 + j, 8 + j, 12 + j
+        af[i][s] = __builtin_bit_cast(int4_t, i < npw ? a : uint4_t{0u, 0u, 0u, 0u});
+      }
+    }
+    __syncthreads();  // the parking areas are where the partial sums go
+  }
+
+  const int w_from = ((lane & 15) * 4 + (lane >> 4)) * 4;  // lane (g, r) of the regrouped register takes lane 4 r + g
+
+  auto do_block = [&](auto q_tag, int k) __attribute__((always_inline)) {
+    constexpr int q = decltype(q_tag)::value;
+    const int nb = nb0 + k * step;
+    load_w(w[(q + 3) % kDepth16], nb + 3 * step, k + 3 < mine);
+    int4_t acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) {
+      uint4_t x = w[q][i];
+      if constexpr (!FRAG) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(w_from, (int)x[d]);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(decode16<CONV>(x[s]), af[i][s], acc, 0, 0, 0);
+    }
+    // lane (g, r) holds the weight rows 4 g .. 4 g + 3 of activation row r.  A wave's sums in LDS: [16 activation
+    // rows][4 pieces of 4 weight rows], piece p of row m at position p ^ (m & 3).
+    unsigned char* const buf = smem + (k & 1) * (kWaves * kPartial16);
+    if (r < M) *reinterpret_cast<int4_t*>(buf + wave * kPartial16 + r * 64 + ((g ^ (r & 3)) << 4)) = acc;
+    __syncthreads();  // one per block, see the kernel above
+    if (finisher) {
+      const int m = out_m, p = out_p;
+      int4_t sum = {0, 0, 0, 0};
+#pragma unroll
+      for (int w8 = 0; w8 < kWaves; ++w8) sum += *reinterpret_cast<const int4_t*>(buf + w8 * kPartial16 + m * 64 + ((p ^ (m & 3)) << 4));
+      using out_t = typename FIN::out_t;
+      constexpr int kShift = Codes<CONV>::kShift;
+      const int n = 16 * nb + 4 * p;
+      if (n < N) {
+        out_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = fin.finish(sum[e] >> kShift, out_row);
+        out_t* const dst = C + (size_t)m * N + n;
+        if ((N & 3) == 0) {
+          typedef out_t out4_t __attribute__((ext_vector_type(4)));
+          *reinterpret_cast<out4_t*>(dst) = out4_t{o[0], o[1], o[2], o[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) dst[e] = o[e];
+        }
+      }
+    }
+  };
+  // Whole turns of the four register sets in a loop without an exit in its body, the last one to three blocks after
+  // it: an exit between two blocks would share its way out with the loop's way round, and the compiler would count
+  // the loads in flight at the top of the loop as if it could have come from there.
+  int k = 0;
+  for (; k + kDepth16 <= mine; k += kDepth16) {
+    do_block(std::integral_constant<int, 0>{}, k);
+    do_block(std::integral_constant<int, 1>{}, k + 1);
+    do_block(std::integral_constant<int, 2>{}, k + 2);
+    do_block(std::integral_constant<int, 3>{}, k + 3);
+  }
+  if (k < mine) {
+    do_block(std::integral_constant<int, 0>{}, k);
+    if (k + 1 < mine) {
+      do_block(std::integral_constant<int, 1>{}, k + 1);
+      if (k + 2 < mine) do_block(std::integral_constant<int, 2>{}, k + 2);
+    }
+  }
+}
+
+template <int CONV, bool FRAG, int NPW, class FIN>
+int launch_i2_regres16(const void* A, const void* B, void* C, int M, int N, int K, int interleaved, FIN fin, hipStream_t stream) {
+  auto kern = i2_regres16_kernel<CONV, FRAG, NPW, FIN>;
+  static bool raised[kMaxDevices] = {};
+  if (raise_lds_limit<kLds16>(kern, raised)) return -1;
+  static int cus_of[kMaxDevices] = {};
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
+  if (!cus_of[device]) DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
+  const int row_blocks = (N + 15) / 16;
+  const int grid = row_blocks < cus_of[device] ? row_blocks : cus_of[device];
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWaves), kLds16, stream, (const int8_t*)A, (const uint8_t*)B,
+                     (typename FIN::out_t*)C, M, N, K, interleaved, fin);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 template <int CONV, bool FRAG, int NPW, bool CHUNKED, class FIN>
 int launch_i2_regres(const void* A, const void* B, void* C, int M, int N, int K, int interleaved, FIN fin, hipStream_t stream) {
   auto kern = i2_regres_kernel<CONV, FRAG, NPW, CHUNKED, FIN>;
@@ -310,15 +486,33 @@ int i2_gemm_regres(const void* A, const void* B, void* C, int M, int N, int K, i
   const int npw = chunked ? kChunkPairs : (npair + kWaves - 1) / kWaves;
   const int il = (layout & ~LAYOUT_FRAGMENTS) == LAYOUT_INTERLEAVED;
   const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
+  // Up to 16 rows the form on blocks of 16 weight rows, where a workgroup has more than four of them (it holds three
+  // blocks in flight and divides the matrix evenly: N = 28672, K = 8192 16.4 against 19.0 us; with fewer blocks its
+  // longer prologue shows: N = 14336, K = 4096 8.2 against 7.9 us).
+  const bool rows16 = M <= 16 && (N + 15) / 16 > 4 * 256;
 #define DQ_I2R(CONV_, FRAG_, NPW_, CH_)                                                                                        \
   do {                                                                                                                         \
     if (bitnet_epilogue)                                                                                                       \
       return launch_i2_regres<CONV_, FRAG_, NPW_, CH_>(A, B, C, M, N, K, il, BitnetFinish{(const float*)s_a, s_w}, stream);    \
     return launch_i2_regres<CONV_, FRAG_, NPW_, CH_>(A, B, C, M, N, K, il, Int32Finish{}, stream);                             \
   } while (0)
+#define DQ_I2R16(CONV_, FRAG_, NPW_)                                                                                     \
+  do {                                                                                                                   \
+    if (bitnet_epilogue)                                                                                                 \
+      return launch_i2_regres16<CONV_, FRAG_, NPW_>(A, B, C, M, N, K, il, BitnetFinish{(const float*)s_a, s_w}, stream); \
+    return launch_i2_regres16<CONV_, FRAG_, NPW_>(A, B, C, M, N, K, il, Int32Finish{}, stream);                          \
+  } while (0)
 #define DQ_I2RN(CONV_, FRAG_)                           \
   do {                                                  \
     if (chunked) DQ_I2R(CONV_, FRAG_, kChunkPairs, true); \
+    if (rows16) {                                       \
+      switch (npw) {                                    \
+        case 1: DQ_I2R16(CONV_, FRAG_, 1);              \
+        case 2: DQ_I2R16(CONV_, FRAG_, 2);              \
+        case 3: DQ_I2R16(CONV_, FRAG_, 3);              \
+        default: DQ_I2R16(CONV_, FRAG_, 4);             \
+      }                                                 \
+    }                                                   \
     switch (npw) {                                      \
       case 1: DQ_I2R(CONV_, FRAG_, 1, false);           \
       case 2: DQ_I2R(CONV_, FRAG_, 2, false);           \
@@ -339,6 +533,7 @@ int i2_gemm_regres(const void* A, const void* B, void* C, int M, int N, int K, i
   }
 #undef DQ_I2RL
 #undef DQ_I2RN
+#undef DQ_I2R16
 #undef DQ_I2R
 }
 
