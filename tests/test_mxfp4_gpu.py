@@ -74,6 +74,26 @@ def test_many_tiles(cuda, fmt, with_bias):
             _check(cuda, 3584, 3600, K, fmt, scale_bias=127)
 
 
+@pytest.mark.parametrize("fmt", ["e2m1", "twiddling", "simple"])
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 128), (5, 300, 1024), (16, 1001, 2048), (8, 4100, 2176), (3, 64, 8192),
+                                   (16, 9000, 5120), (17, 515, 1280), (40, 130, 4096), (64, 8200, 768), (12, 33, 6144)])
+def test_decode_batches(cuda, fmt, with_bias, M, N, K):
+    """Up to 64 rows with K a multiple of 128 up to 8192: the kernel that keeps the activations in registers and streams
+    weights and scale bytes once per 16 rows.  Ragged N (last block of 16 weight rows, N % 4 != 0), K slices of unequal
+    length over the eight waves (2176 = 17 chunks, 1280 = 10, 128 = 1), the eight-chunk form with parked activations
+    (8192), passes of 16 rows (17, 40, 64), every format, with and without bias."""
+    _check(cuda, M, N, K, fmt, scale_bias=127, seed=M + K, with_bias=with_bias)
+
+
+def test_decode_batch_full_size_and_deterministic(cuda):
+    """N = K = 8192 at 16 rows against the oracle, twice: the partial sums of the eight K slices are added in a
+    fixed order."""
+    a = _check(cuda, 16, 8192, 8192, "e2m1", scale_bias=127, seed=4)
+    b = _check(cuda, 16, 8192, 8192, "e2m1", scale_bias=127, seed=4)
+    np.testing.assert_array_equal(a, b)
+
+
 @pytest.mark.parametrize("fmt", ["e2m1", "simple"])
 def test_bias(cuda, fmt):
     _check(cuda, 384, 512, 256, fmt, scale_bias=127, with_bias=True)
@@ -118,11 +138,19 @@ def test_full_size_properties(cuda):
     ref = orc.bf16_bits_to_f32(orc.f32_to_bf16_bits(Af @ W.T))
     got = C[torch.from_numpy(rows).to(cuda)][:, torch.from_numpy(cols).to(cuda)].float().cpu().numpy()
     np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL)
-    # whole-matrix check against the row sample: rows of C computed by an independent call on A[rows]
+    # whole-matrix check against a row sample: rows of C computed by an independent call on A[rows] (80 rows: the tiled
+    # kernel again, whose sums do not depend on where in the matrix a row lies; up to 64 rows the decode kernel would
+    # take the call and add the same products in another order)
+    rows = rng.choice(M, 80, replace=False)
     kern_small = tl.matmul_bf16_mxfp4(len(rows), N, K, weight_format="e2m1", scale_bias=127)
     C_rows = kern_small(A[torch.from_numpy(rows).to(cuda)].contiguous(), B, S, bias[: len(rows)].contiguous())
     torch.cuda.synchronize()
     assert torch.equal(C_rows, C[torch.from_numpy(rows).to(cuda)])
+    # and the decode kernel on 16 of those rows: within rounding of the same values
+    kern_dec = tl.matmul_bf16_mxfp4(16, N, K, weight_format="e2m1", scale_bias=127)
+    C_dec = kern_dec(A[torch.from_numpy(rows[:16]).to(cuda)].contiguous(), B, S, bias[:16].contiguous())
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(C_dec.float().cpu().numpy(), C_rows[:16].float().cpu().numpy(), rtol=RTOL, atol=ATOL)
     # linearity: C(2A) == 2 C(A) exactly (power-of-two scaling commutes with every rounding)
     C2 = kern((A.float() * 2).to(torch.bfloat16), B, S, bias)
     torch.cuda.synchronize()

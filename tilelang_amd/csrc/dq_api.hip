@@ -36,6 +36,8 @@ int w4a16_gemv_dot2(const void* A, const void* B, const void* S, const void* Z, 
 int mxfp4_gemm(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
                int scale_bias, hipStream_t stream);
 
+int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
+                      int scale_bias, int max_rows, hipStream_t stream);
 int bf16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int fmt, hipStream_t stream);
 int fp16_fp4_gemm(const void* A, const void* B, void* C, int M, int N, int K, int transposed, hipStream_t stream);
 int w4_f16_gemm(const void* A, const void* B, const void* S, const void* Z, void* C, int M, int N, int K, int group,
@@ -356,6 +358,13 @@ extern "C" int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const 
   if (scale_bias < 0 || scale_bias > 255) DQ_FAIL("%s: scale_bias must be in 0..255 (got %d)", fn, scale_bias);
   if (!aligned16(A) || !aligned16(B) || !aligned16(C) || (Bias && !aligned16(Bias)))
     DQ_FAIL("%s: A, B, Bias and C must be 16-byte aligned", fn);
+  // a decode batch: activations resident in registers, the weights streamed once per 16 rows (K % 128 == 0, K <= 8192);
+  // two passes (32 rows) still beat the tiled kernel's one round of N / 256 workgroups (N = K = 8192: 34 against
+  // 60 us), four do not
+  if (M <= 32) {
+    const int rc = mxfp4_gemm_regres(A, B, Scale, Bias, C, M, N, K, fp4_format, scale_bias, 32, (hipStream_t)stream);
+    if (rc <= 0) return rc;
+  }
   return mxfp4_gemm(A, B, Scale, Bias, C, M, N, K, fp4_format, scale_bias, (hipStream_t)stream);
 }
 

@@ -1,0 +1,308 @@
+// MXFP4-weight x bf16 small batch (decode: up to 16 activation rows per pass) on gfx950: activations resident in
+// registers, weights and block scales streamed once.
+//
+// Replaces the kernel of examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:201-244 (formats and
+// scales: example_dequant_gemm_bf16_mxfp4_hopper.py:56-110,272-330) where M is a decode batch.  The tiled GEMM gives
+// such a problem N / 256 workgroups with all of K behind each (N = K = 8192 at 1 to 128 rows: 60 us for 35 MB); here
+// the matrix is cut by weight rows over all CUs and by K over the waves of a workgroup, as in dq_regres_i2.hip:
+//
+//   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of whole 128-k chunks, at most eight:
+//     K <= 8192) and keeps the activations of its slice as operands of v_mfma_f32_16x16x32_bf16 in registers for the
+//     whole kernel (16 rows x 1024 k: 128 registers per lane);
+//   * the workgroups walk the blocks of 16 weight rows.  A chunk of a block is 16 rows x 64 bytes: one 16-byte load
+//     per lane (lane l: piece l % 4 of row l / 4, whole 64-byte runs), then one ds_bpermute_b32 per dword hands lane
+//     (g, r) piece g of row r.  Dword s of a lane feeds step s, contraction index k = 128 chunk + 32 g + 8 s + e for
+//     both operands: a lane's 32 codes are ONE scale block, so the lane applies one E8M0 byte per chunk (a dword of
+//     the row's scale bytes per chunk and lane, byte g of it) through the scale operand of the fp4 -> bf16 conversion;
+//   * two sets of weight registers: a workgroup's first two blocks are asked for at once, every further one when the
+//     set of the block two before it comes free; the eight partial sums of a block meet in LDS in fp32 (two
+//     buffers, one barrier per block) and 64 threads add them in wave order (the same order every run), add the bias,
+//     round to bf16 and store.
+//
+// Every load is unconditional and the last block has its own copy of the code, so that the compiler's count of loads
+// in flight is exact (see dq_regres_i2.hip).  A wave whose slice is shorter than the longest loads its last chunk
+// again against activations of zero.  More than 16 rows: gridDim.y passes of 16, each streaming the weights again.
+#include <type_traits>
+
+#include "dq_common.h"
+#include "dq_fp4_codes.h"
+
+namespace dq {
+
+namespace {
+
+constexpr int kWaves = 8;              // K slices
+constexpr int kMaxChunks = 8;          // 128-k chunks per wave
+constexpr int kPartial = 16 * 16 * 4;  // one wave's 16 x 16 sums
+constexpr int kLds = kWaves * 4096;    // the prologue's parking areas; the two buffers of partial sums reuse them
+// With eight chunks per wave the activations (128 registers), two sets of weights and scales (80) and the arithmetic
+// do not fit 256 registers: the fragments of the wave's last three (four) chunks stay parked in LDS (4 KiB per wave and chunk,
+// behind the areas above) and are read again for every block.
+constexpr int parked_chunks(int ncw, bool svec) { return ncw == 8 ? (svec ? 3 : 4) : 0; }  // dword scale loads: eight more addresses
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+// what a lane applies to its 32 codes of one chunk: the block's power of two as the conversion's scale operand, or,
+// for the "simple" format, the exponent to add to both halves of a dword
+struct LaneScale {
+  float f;
+  uint32_t add;
+};
+template <int FMT>
+__device__ __forceinline__ LaneScale lane_scale(uint32_t e, int off) {
+  LaneScale s;
+  if constexpr (FMT == FP4_SIMPLE) {
+    int ex = 126 + (int)e + off - 127;
+    ex = ex < 0 ? 0 : (ex > 252 ? 252 : ex);  // E adds up to 3
+    s.add = ((uint32_t)ex << 7) * 0x00010001u;
+    s.f = 0.f;
+  } else {
+    s.f = scale_to_f32((int)e, off);
+    s.add = 0;
+  }
+  return s;
+}
+template <int FMT>
+__device__ __forceinline__ bf16x8_t decode8(uint32_t w, const LaneScale& s) {
+  if constexpr (FMT == FP4_E2M1) return cvt_e2m1x8(w, s.f);
+  else if constexpr (FMT == FP4_TWIDDLING) return cvt_e2m1x8(twiddled_to_plain(w), s.f);
+  else return __builtin_bit_cast(bf16x8_t, simple_fp4x8<7>(w, s.add));
+}
+
+template <int FMT, bool HAS_BIAS, int NCW, bool SVEC>
+__global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t* __restrict__ A_all, const uint8_t* __restrict__ B,
+                                                                   const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias_all,
+                                                                   bf16_t* __restrict__ C_all, int M_all, int N, int K, int exp_off) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int m_first = 16 * blockIdx.y;
+  const bf16_t* const A = A_all + (size_t)m_first * K;
+  bf16_t* const C = C_all + (size_t)m_first * N;
+  const bf16_t* const Bias = HAS_BIAS ? Bias_all + (size_t)m_first * N : nullptr;
+  const int M = min(M_all - m_first, 16);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+
+  // the wave's chunks: [c_lo, c_lo + ncw), ncw <= NCW
+  const int nchunk = K >> 7;
+  const int c_lo = wave * nchunk / kWaves;
+  const int ncw = (wave + 1) * nchunk / kWaves - c_lo;
+  auto chunk_of = [&](int i) { return c_lo + min(i, max(ncw - 1, 0)); };  // K < 1024: some waves have no chunk at all
+
+  const int row_blocks = (N + 15) >> 4;
+  const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
+  int nb = blockIdx.x;
+
+  // ---- weights and scales of the block of 16 rows nb
+  // (the chunk numbers are the same for every lane of the wave: scalar registers, not eight offsets per lane)
+  const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)(K >> 5);
+  auto load_w = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk) __attribute__((always_inline)) {
+    const uint8_t* const w_row = B + (size_t)min(16 * blk + (lane >> 2), N - 1) * w_row_bytes + (lane & 3) * 16;
+    const uint8_t* const s_row = S + (size_t)min(16 * blk + r, N - 1) * s_row_bytes;
+#pragma unroll
+    for (int i = 0; i < NCW; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + chunk_of(i) * 64));
+    // A lane's scale bytes of a block: the dword of every chunk (byte g of it is the lane's).  SVEC (K % 4096 == 0: every
+    // wave's run of chunks starts on a multiple of four and is a multiple of four long): 16 bytes, four chunks, per
+    // load.  Dword by dword the eight loads of a lane fetched the same 32 bytes eight times from the L2 (nontemporal
+    // loads leave nothing in the L1): 12 of 48 us at N = 28672, K = 8192.
+    if constexpr (SVEC) {
+#pragma unroll
+      for (int i = 0; i < NCW; i += 4) {
+        const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(s_row + c_lo * 4 + i * 4));
+        sc[i] = v[0], sc[i + 1] = v[1], sc[i + 2] = v[2], sc[i + 3] = v[3];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCW; ++i) sc[i] = *reinterpret_cast<const uint32_t*>(s_row + chunk_of(i) * 4);
+    }
+    // the loads go out here, ahead of the arithmetic of the block before: left to itself the scheduler sinks them
+    // behind it to save registers, and the block ahead is then waited for right after it was asked for
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  uint4_t w0[NCW], w1[NCW];
+  uint32_t sc0[NCW], sc1[NCW];
+  // The workgroup's first two blocks are asked for before the activations: the memory's first answer takes as long as
+  // the prologue, and most matrices give a workgroup two to four blocks, too few for a pipeline that starts one deep.
+  // (A condition on a load is harmless here: the wait for the activations below waits for everything before it.)
+  const int mine = (row_blocks - nb + step - 1) / step;
+  load_w(w0, sc0, nb);
+  if (mine > 1) load_w(w1, sc1, nb + step);
+
+  // ---- activations: fragment (chunk i, step s): lane (g, r) holds k = 128 chunk + 32 g + 8 s .. + 7 of row r.  Read as
+  // whole lines (instruction j: rows 4 j .. 4 j + 3, lane l the 16-byte piece l % 16 of row 4 j + l / 16 of the
+  // chunk's 256 bytes), parked in the wave's 4 KiB of LDS (piece q of row m at position q ^ m), read back in operand
+  // order: fetched in that order a load instruction would touch 32 cache lines for 32 bytes each.
+  constexpr int PARK = parked_chunks(NCW, SVEC), NR = NCW - PARK;
+  unsigned char* const kept = smem + kLds + wave * (PARK * 4096);  // chunk NR + q at kept + 4096 q, laid out as `park`
+  const int kept_rd = r * 256;                                      // piece p of the lane's row: kept_rd + ((p ^ r) << 4)
+  bf16x8_t af[NR][4];
+  {
+    const unsigned char* const a_lane = reinterpret_cast<const unsigned char*>(A) + 16 * (lane & 15);
+    uint4_t line[NCW][4];
+#pragma unroll
+    for (int i = 0; i < NCW; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        line[i][j] = *reinterpret_cast<const uint4_t*>(a_lane + ((size_t)min(4 * j + (lane >> 4), M - 1) * K + 128 * chunk_of(i)) * 2);
+#pragma unroll
+    for (int i = 0; i < NCW; ++i) {
+      unsigned char* const park = i < NR ? smem + wave * 4096 : kept + (i - NR) * 4096;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        // a chunk beyond the wave's slice: zeros
+        *reinterpret_cast<uint4_t*>(park + row * 256 + (((lane & 15) ^ row) << 4)) = i < ncw ? line[i][j] : uint4_t{0u, 0u, 0u, 0u};
+      }
+      // a wave's LDS operations are carried out in the order they were issued
+      if (i < NR) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          af[i < NR ? i : 0][s] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4_t*>(park + kept_rd + (((4 * g + s) ^ r) << 4)));
+      }
+    }
+    __syncthreads();  // the parking areas are where the partial sums go
+  }
+
+  const int w_from = ((lane & 15) * 4 + (lane >> 4)) * 4;  // lane (g, r) of the regrouped register takes lane 4 r + g
+  // the thread's share of the final sum: activation row tid / 4, weight rows 4 (tid % 4) .. + 3 of the block
+  const int out_m = tid >> 2, out_p = tid & 3;
+  const bool finisher = tid < 64 && out_m < M;
+
+  auto do_block = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk, int it) __attribute__((always_inline)) {
+    float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NCW; ++i) {
+      uint4_t x = w[i];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(w_from, (int)x[d]);
+      const LaneScale ls = lane_scale<FMT>((sc[i] >> (8 * g)) & 0xFFu, exp_off);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        bf16x8_t a;
+        if (i < NR) a = af[i < NR ? i : 0][s];
+        else a = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4_t*>(kept + (i - NR) * 4096 + kept_rd + (((4 * g + s) ^ r) << 4)));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(decode8<FMT>(x[s], ls), a, acc, 0, 0, 0);
+      }
+    }
+    // lane (g, r) holds the weight rows 4 g .. 4 g + 3 of activation row r.  A wave's sums in LDS: [16 activation
+    // rows][4 pieces of 4 weight rows], piece p of row m at position p ^ (m & 3).
+    unsigned char* const buf = smem + (it & 1) * (kWaves * kPartial);
+    if (r < M) *reinterpret_cast<float4v*>(buf + wave * kPartial + r * 64 + ((g ^ (r & 3)) << 4)) = acc;
+    // One barrier per block: the buffer written here is read below and written again two blocks later, after the next
+    // block's barrier, which no thread passes before it has finished reading here.
+    __syncthreads();
+    if (finisher) {
+      const int m = out_m, p = out_p;
+      float4v sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w8 = 0; w8 < kWaves; ++w8) sum += *reinterpret_cast<const float4v*>(buf + w8 * kPartial + m * 64 + ((p ^ (m & 3)) << 4));
+      const int n = 16 * blk + 4 * p;
+      if (n < N) {
+        bf16_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = sum[e];
+          // reference: C = bf16(float(acc) + float(Bias))
+          if constexpr (HAS_BIAS) {
+            if (n + e < N) v += (float)Bias[(size_t)m * N + n + e];
+          }
+          o[e] = (bf16_t)v;
+        }
+        bf16_t* const dst = C + (size_t)m * N + n;
+        if ((N & 3) == 0) {
+          typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
+          *reinterpret_cast<bf16x4_t*>(dst) = bf16x4_t{o[0], o[1], o[2], o[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) dst[e] = o[e];
+        }
+      }
+    }
+  };
+
+  // w0 holds the workgroup's block k, w1 block k + 1; a set is asked for again (block k + 2) as soon as its block is
+  // done.  The loop over pairs of blocks that both have a successor has no exit in its body, and the last one to three
+  // blocks follow it in copies of their own: a load under a condition, or an exit that shares its way out with the
+  // loop's way round, would make the compiler count the loads in flight for a path that does not have them, and wait
+  // for everything at the top of the loop.
+  int k = 0;
+  for (; k + 4 <= mine; k += 2) {
+    do_block(w0, sc0, nb, k);
+    load_w(w0, sc0, nb + 2 * step);
+    do_block(w1, sc1, nb + step, k + 1);
+    load_w(w1, sc1, nb + 3 * step);
+    nb += 2 * step;
+  }
+  const int left = mine - k;
+  if (left == 1) {
+    do_block(w0, sc0, nb, k);
+  } else if (left == 2) {
+    do_block(w0, sc0, nb, k);
+    do_block(w1, sc1, nb + step, k + 1);
+  } else {
+    do_block(w0, sc0, nb, k);
+    load_w(w0, sc0, nb + 2 * step);
+    do_block(w1, sc1, nb + step, k + 1);
+    do_block(w0, sc0, nb + 2 * step, k + 2);
+  }
+}
+
+template <int FMT, bool HAS_BIAS, int NCW, bool SVEC>
+int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int exp_off,
+                     hipStream_t stream) {
+  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, SVEC>;
+  static bool raised[kMaxDevices] = {};
+  constexpr int kLdsAll = kLds + kWaves * parked_chunks(NCW, SVEC) * 4096;
+  if (raise_lds_limit<kLdsAll>(kern, raised)) return -1;
+  static int cus_of[kMaxDevices] = {};
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
+  if (!cus_of[device]) DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
+  const int row_blocks = (N + 15) / 16;
+  const int grid = row_blocks < cus_of[device] ? row_blocks : cus_of[device];
+  hipLaunchKernelGGL(kern, dim3(grid, (M + 15) / 16), dim3(64 * kWaves), kLdsAll, stream, (const bf16_t*)A, (const uint8_t*)B,
+                     (const uint8_t*)S, (const bf16_t*)Bias, (bf16_t*)C, M, N, K, exp_off);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace
+
+// 0: launched; 1: this shape is not the kernel's (the caller goes on to the tiled GEMM); -1: error.
+// max_rows: the most activation rows to take (passes of 16, each streaming the weights again).
+int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
+                      int scale_bias, int max_rows, hipStream_t stream) {
+  // whole 128-k chunks, at most eight per wave
+  if (M < 1 || M > max_rows || K % 128 != 0 || K > kWaves * kMaxChunks * 128) return 1;
+  const int ncw = ((K >> 7) + kWaves - 1) / kWaves;
+  const int exp_off = 127 - scale_bias;
+  const bool svec = K % 4096 == 0;
+#define DQ_MXR(FMT_, NCW_, SVEC_)                                                                               \
+  do {                                                                                                          \
+    if (Bias) return launch_mx_regres<FMT_, true, NCW_, SVEC_>(A, B, S, Bias, C, M, N, K, exp_off, stream);     \
+    return launch_mx_regres<FMT_, false, NCW_, SVEC_>(A, B, S, nullptr, C, M, N, K, exp_off, stream);           \
+  } while (0)
+#define DQ_MXRN(FMT_)                              \
+  do {                                             \
+    if (svec && ncw == 4) DQ_MXR(FMT_, 4, true);   \
+    if (svec && ncw == 8) DQ_MXR(FMT_, 8, true);   \
+    if (ncw <= 2) DQ_MXR(FMT_, 2, false);          \
+    if (ncw <= 4) DQ_MXR(FMT_, 4, false);          \
+    if (ncw <= 6) DQ_MXR(FMT_, 6, false);          \
+    DQ_MXR(FMT_, 8, false);                        \
+  } while (0)
+  switch (fmt) {
+    case FP4_E2M1: DQ_MXRN(FP4_E2M1);
+    case FP4_SIMPLE: DQ_MXRN(FP4_SIMPLE);
+    case FP4_TWIDDLING: DQ_MXRN(FP4_TWIDDLING);
+    default: DQ_FAIL("mxfp4 gemm: unknown weight format %d", fmt);
+  }
+#undef DQ_MXRN
+#undef DQ_MXR
+}
+
+}  // namespace dq
