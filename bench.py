@@ -49,6 +49,11 @@ def gemv_hbm_traffic():
     return None, None
 
 
+#: False (--no-graph): time plain back-to-back launches.  For runs under a profiler that collects hardware counters: it
+#: serialises the kernels itself, and a replayed graph whose calls are two dependent kernels did not come back under it.
+USE_GRAPH = True
+
+
 def _time_launches(torch, fns, steps, warmup, min_launches=120, max_launches=None, settle_ms=50.0, replays=30):
     """Median device time per call of fns[i % len(fns)], independent of `steps`.
 
@@ -70,6 +75,8 @@ def _time_launches(torch, fns, steps, warmup, min_launches=120, max_launches=Non
     stream = torch.cuda.Stream()
     graph = None
     try:
+        if not USE_GRAPH:
+            raise RuntimeError("--no-graph")
         with torch.cuda.stream(stream):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
@@ -330,6 +337,9 @@ def _row(config, r, bound, peak):
     sec = r["us"] * 1e-6
     row = {"config": config, "us": r["us"], "us_min": r["timing"]["us_min"], "GB/s": r["bytes"] / sec / 1e9, "TFLOP/s": r["flops"] / sec / 1e12, "bound": bound}
     row["frac"] = (r["bytes"] / sec / HBM_PEAK) if bound == "hbm" else (r["flops"] / sec / peak)
+    # progress on stderr (stdout carries the one JSON line): a row at a time, so that a run under a profiler, which
+    # takes minutes, is seen to be alive
+    print(f"[bench] {config}: {r['us']:.1f} us", file=sys.stderr, flush=True)
     return row
 
 
@@ -447,10 +457,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=12)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="skip the per-configuration table")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="time plain launches instead of replaying a HIP graph (for counter runs under rocprofv3 --pmc)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise copy of 128 MiB a few times: under `rocprofv3 --pmc FETCH_SIZE` / "
                          "`WRITE_SIZE` its counters give the factor that turns counter units into bytes")
     args = ap.parse_args()
+    global USE_GRAPH
+    USE_GRAPH = not args.no_graph
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path would shard by output rows N, "
                  "each GPU holding its rows of the weights and a replica of the activations, with no communication)")
@@ -511,6 +525,9 @@ def main():
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
         mx_run = r
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
+        # the same weights at a decode batch: activations resident in registers, weights streamed once
+        r = bench_mxfp4(torch, tl, workloads, 16, 8192, 8192, S, W, dev)
+        shapes.append(_row("mxfp4_gemm M=16 N=8192 K=8192", r, "hbm", MFMA_BF16_PEAK))
         for m in (1, 16, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m <= 16 else gemm))
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m <= 16 else "mfma", MFMA_I8_PEAK))
