@@ -6,8 +6,8 @@
 // such a problem N / 256 workgroups with all of K behind each (N = K = 8192 at 1 to 128 rows: 60 us for 35 MB); here
 // the matrix is cut by weight rows over all CUs and by K over the waves of a workgroup, as in dq_regres_i2.hip:
 //
-//   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of whole 128-k chunks, at most eight:
-//     K <= 8192) and keeps the activations of its slice as operands of v_mfma_f32_16x16x32_bf16 in registers for the
+//   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of 128-k chunks, at most eight:
+//     K <= 8192; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands of v_mfma_f32_16x16x32_bf16 in registers for the
 //     whole kernel (16 rows x 1024 k: 128 registers per lane);
 //   * the workgroups walk the blocks of 16 weight rows.  A chunk of a block is 16 rows x 64 bytes: one 16-byte load
 //     per lane (lane l: piece l % 4 of row l / 4, whole 64-byte runs), then one ds_bpermute_b32 per dword hands lane
@@ -69,7 +69,7 @@ __device__ __forceinline__ bf16x8_t decode8(uint32_t w, const LaneScale& s) {
   else return __builtin_bit_cast(bf16x8_t, simple_fp4x8<7>(w, s.add));
 }
 
-template <int FMT, bool HAS_BIAS, int NCW, bool SVEC>
+template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF>
 __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t* __restrict__ A_all, const uint8_t* __restrict__ B,
                                                                    const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias_all,
                                                                    bf16_t* __restrict__ C_all, int M_all, int N, int K, int exp_off) {
@@ -86,10 +86,15 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   const int g = lane >> 4;
 
   // the wave's chunks: [c_lo, c_lo + ncw), ncw <= NCW
-  const int nchunk = K >> 7;
+  // HALF: K % 128 == 64, the last chunk has 64 k.  Its lanes of the upper half (pieces 2, 3 of a weight
+  // row's 64 bytes, 8 .. 15 of an activation row's 256) read the lower half's addresses instead, so that nothing is
+  // read beyond a row, and take zeros for codes and activations.
+  const int nchunk = (K + 127) >> 7;
+  constexpr bool half_last = HALF;  // a form of its own: its lane-dependent addresses cost registers
   const int c_lo = wave * nchunk / kWaves;
   const int ncw = (wave + 1) * nchunk / kWaves - c_lo;
   auto chunk_of = [&](int i) { return c_lo + min(i, max(ncw - 1, 0)); };  // K < 1024: some waves have no chunk at all
+  auto is_half = [&](int i) { return half_last && chunk_of(i) == nchunk - 1; };
 
   const int row_blocks = (N + 15) >> 4;
   const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
@@ -99,10 +104,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   // (the chunk numbers are the same for every lane of the wave: scalar registers, not eight offsets per lane)
   const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)(K >> 5);
   auto load_w = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk) __attribute__((always_inline)) {
-    const uint8_t* const w_row = B + (size_t)min(16 * blk + (lane >> 2), N - 1) * w_row_bytes + (lane & 3) * 16;
+    const uint8_t* const w_row = B + (size_t)min(16 * blk + (lane >> 2), N - 1) * w_row_bytes;
     const uint8_t* const s_row = S + (size_t)min(16 * blk + r, N - 1) * s_row_bytes;
 #pragma unroll
-    for (int i = 0; i < NCW; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + chunk_of(i) * 64));
+    for (int i = 0; i < NCW; ++i)
+      w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + chunk_of(i) * 64 + ((lane & 3) & (is_half(i) ? 1 : 3)) * 16));
     // A lane's scale bytes of a block: the dword of every chunk (byte g of it is the lane's).  SVEC (K % 4096 == 0: every
     // wave's run of chunks starts on a multiple of four and is a multiple of four long): 16 bytes, four chunks, per
     // load.  Dword by dword the eight loads of a lane fetched the same 32 bytes eight times from the L2 (nontemporal
@@ -115,7 +121,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < NCW; ++i) sc[i] = *reinterpret_cast<const uint32_t*>(s_row + chunk_of(i) * 4);
+      for (int i = 0; i < NCW; ++i) sc[i] = s_row[chunk_of(i) * 4 + (g & (is_half(i) ? 1 : 3))];  // the lane's own byte
     }
     // the loads go out here, ahead of the arithmetic of the block before: left to itself the scheduler sinks them
     // behind it to save registers, and the block ahead is then waited for right after it was asked for
@@ -139,13 +145,14 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   const int kept_rd = r * 256;                                      // piece p of the lane's row: kept_rd + ((p ^ r) << 4)
   bf16x8_t af[NR][4];
   {
-    const unsigned char* const a_lane = reinterpret_cast<const unsigned char*>(A) + 16 * (lane & 15);
+    const unsigned char* const a_base = reinterpret_cast<const unsigned char*>(A);
     uint4_t line[NCW][4];
 #pragma unroll
     for (int i = 0; i < NCW; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        line[i][j] = *reinterpret_cast<const uint4_t*>(a_lane + ((size_t)min(4 * j + (lane >> 4), M - 1) * K + 128 * chunk_of(i)) * 2);
+        line[i][j] = *reinterpret_cast<const uint4_t*>(a_base + ((size_t)min(4 * j + (lane >> 4), M - 1) * K + 128 * chunk_of(i)) * 2 +
+                                                       16 * ((lane & 15) & (is_half(i) ? 7 : 15)));
 #pragma unroll
     for (int i = 0; i < NCW; ++i) {
       unsigned char* const park = i < NR ? smem + wave * 4096 : kept + (i - NR) * 4096;
@@ -153,7 +160,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
       for (int j = 0; j < 4; ++j) {
         const int row = 4 * j + (lane >> 4);
         // a chunk beyond the wave's slice: zeros
-        *reinterpret_cast<uint4_t*>(park + row * 256 + (((lane & 15) ^ row) << 4)) = i < ncw ? line[i][j] : uint4_t{0u, 0u, 0u, 0u};
+        const bool there = i < ncw && !(is_half(i) && (lane & 15) >= 8);
+        *reinterpret_cast<uint4_t*>(park + row * 256 + (((lane & 15) ^ row) << 4)) = there ? line[i][j] : uint4_t{0u, 0u, 0u, 0u};
       }
       // a wave's LDS operations are carried out in the order they were issued
       if (i < NR) {
@@ -177,7 +185,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
       uint4_t x = w[i];
 #pragma unroll
       for (int d = 0; d < 4; ++d) x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(w_from, (int)x[d]);
-      const LaneScale ls = lane_scale<FMT>((sc[i] >> (8 * g)) & 0xFFu, exp_off);
+      const LaneScale ls = lane_scale<FMT>(SVEC ? (sc[i] >> (8 * g)) & 0xFFu : sc[i], exp_off);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         bf16x8_t a;
@@ -250,10 +258,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   }
 }
 
-template <int FMT, bool HAS_BIAS, int NCW, bool SVEC>
+template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF>
 int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int exp_off,
                      hipStream_t stream) {
-  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, SVEC>;
+  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, SVEC, HALF>;
   static bool raised[kMaxDevices] = {};
   constexpr int kLdsAll = kLds + kWaves * parked_chunks(NCW, SVEC) * 4096;
   if (raise_lds_limit<kLdsAll>(kern, raised)) return -1;
@@ -276,24 +284,42 @@ int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bi
 // max_rows: the most activation rows to take (passes of 16, each streaming the weights again).
 int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
                       int scale_bias, int max_rows, hipStream_t stream) {
-  // whole 128-k chunks, at most eight per wave
-  if (M < 1 || M > max_rows || K % 128 != 0 || K > kWaves * kMaxChunks * 128) return 1;
-  const int ncw = ((K >> 7) + kWaves - 1) / kWaves;
+  // 128-k chunks (the last one may be half: K % 128 == 64), at most eight per wave
+  if (M < 1 || M > max_rows || K % 64 != 0 || K > kWaves * kMaxChunks * 128) return 1;
+  // More than 16 rows run as passes of 16, each streaming the weights again: worth it while that stays ahead of the
+  // tiled kernel, whose time up to 128 rows is one round of workgroups with all of K behind each (60 us at K = 8192,
+  // 92 us from N = 16384 on), against 2.5 us + 4.5 us per 8192 k for every block of 16 weight rows that a workgroup
+  // visits here (measured: N = K = 8192 at 32 / 48 / 64 rows 32 / 46 / 61 us against 61 us; N = K = 2880, where the
+  // passes share a round, 11 / 15 / 16 us and at 128 rows 29 us against 24.6 us).
+  if (M > 16) {
+    const double kfrac = (double)K / 8192.0;
+    const long visits = ((long)((N + 15) / 16) * ((M + 15) / 16) + 255) / 256;
+    const double t_here = (double)visits * (2.5 + 4.5 * kfrac) + 3.0, t_tiled = (N > 16384 ? 92.0 : 60.0) * kfrac + 3.0;
+    if (t_here > 0.9 * t_tiled) return 1;
+  }
+  const int ncw = (((K + 127) >> 7) + kWaves - 1) / kWaves;
   const int exp_off = 127 - scale_bias;
   const bool svec = K % 4096 == 0;
-#define DQ_MXR(FMT_, NCW_, SVEC_)                                                                               \
-  do {                                                                                                          \
-    if (Bias) return launch_mx_regres<FMT_, true, NCW_, SVEC_>(A, B, S, Bias, C, M, N, K, exp_off, stream);     \
-    return launch_mx_regres<FMT_, false, NCW_, SVEC_>(A, B, S, nullptr, C, M, N, K, exp_off, stream);           \
+  const bool half = K % 128 != 0;
+  if (half && ncw > 6) return 1;  // the half chunk's form with eight chunks per wave does not fit the registers
+#define DQ_MXR(FMT_, NCW_, SVEC_, HALF_)                                                                               \
+  do {                                                                                                                 \
+    if (Bias) return launch_mx_regres<FMT_, true, NCW_, SVEC_, HALF_>(A, B, S, Bias, C, M, N, K, exp_off, stream);     \
+    return launch_mx_regres<FMT_, false, NCW_, SVEC_, HALF_>(A, B, S, nullptr, C, M, N, K, exp_off, stream);           \
   } while (0)
-#define DQ_MXRN(FMT_)                              \
-  do {                                             \
-    if (svec && ncw == 4) DQ_MXR(FMT_, 4, true);   \
-    if (svec && ncw == 8) DQ_MXR(FMT_, 8, true);   \
-    if (ncw <= 2) DQ_MXR(FMT_, 2, false);          \
-    if (ncw <= 4) DQ_MXR(FMT_, 4, false);          \
-    if (ncw <= 6) DQ_MXR(FMT_, 6, false);          \
-    DQ_MXR(FMT_, 8, false);                        \
+#define DQ_MXRN(FMT_)                                     \
+  do {                                                    \
+    if (svec && ncw == 4) DQ_MXR(FMT_, 4, true, false);   \
+    if (svec && ncw == 8) DQ_MXR(FMT_, 8, true, false);   \
+    if (half) {                                           \
+      if (ncw <= 2) DQ_MXR(FMT_, 2, false, true);         \
+      if (ncw <= 4) DQ_MXR(FMT_, 4, false, true);         \
+      DQ_MXR(FMT_, 6, false, true);                       \
+    }                                                     \
+    if (ncw <= 2) DQ_MXR(FMT_, 2, false, false);          \
+    if (ncw <= 4) DQ_MXR(FMT_, 4, false, false);          \
+    if (ncw <= 6) DQ_MXR(FMT_, 6, false, false);          \
+    DQ_MXR(FMT_, 8, false, false);                        \
   } while (0)
   switch (fmt) {
     case FP4_E2M1: DQ_MXRN(FP4_E2M1);
