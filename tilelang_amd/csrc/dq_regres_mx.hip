@@ -7,8 +7,8 @@
 // the matrix is cut by weight rows over all CUs and by K over the waves of a workgroup, as in dq_regres_i2.hip:
 //
 //   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of 128-k chunks, at most eight:
-//     K <= 8192; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands of v_mfma_f32_16x16x32_bf16 in registers for the
-//     whole kernel (16 rows x 1024 k: 128 registers per lane);
+//     K <= 8192; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands
+//     of v_mfma_f32_16x16x32_bf16 in registers for the whole kernel (16 rows x 1024 k: 128 registers per lane);
 //   * the workgroups walk the blocks of 16 weight rows.  A chunk of a block is 16 rows x 64 bytes: one 16-byte load
 //     per lane (lane l: piece l % 4 of row l / 4, whole 64-byte runs), then one ds_bpermute_b32 per dword hands lane
 //     (g, r) piece g of row r.  Dword s of a lane feeds step s, contraction index k = 128 chunk + 32 g + 8 s + e for
@@ -36,9 +36,10 @@ constexpr int kMaxChunks = 8;          // 128-k chunks per wave
 constexpr int kPartial = 16 * 16 * 4;  // one wave's 16 x 16 sums
 constexpr int kLds = kWaves * 4096;    // the prologue's parking areas; the two buffers of partial sums reuse them
 // With eight chunks per wave the activations (128 registers), two sets of weights and scales (80) and the arithmetic
-// do not fit 256 registers: the fragments of the wave's last three (four) chunks stay parked in LDS (4 KiB per wave and chunk,
-// behind the areas above) and are read again for every block.
-constexpr int parked_chunks(int ncw, bool svec) { return ncw == 8 ? (svec ? 3 : 4) : 0; }  // dword scale loads: eight more addresses
+// do not fit 256 registers: the fragments of the wave's last three chunks (four where the scale bytes are loaded one
+// by one: eight more addresses) stay parked in LDS, 4 KiB per wave and chunk behind the areas above, and are read
+// again for every block.
+constexpr int parked_chunks(int ncw, bool svec) { return ncw == 8 ? (svec ? 3 : 4) : 0; }
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 
@@ -85,10 +86,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   const int r = lane & 15;
   const int g = lane >> 4;
 
-  // the wave's chunks: [c_lo, c_lo + ncw), ncw <= NCW
-  // HALF: K % 128 == 64, the last chunk has 64 k.  Its lanes of the upper half (pieces 2, 3 of a weight
-  // row's 64 bytes, 8 .. 15 of an activation row's 256) read the lower half's addresses instead, so that nothing is
-  // read beyond a row, and take zeros for codes and activations.
+  // The wave's chunks: [c_lo, c_lo + ncw), ncw <= NCW.  HALF: K % 128 == 64, the last chunk has 64 k.  Its lanes of the
+  // upper half (pieces 2, 3 of a weight row's 64 bytes, 8 .. 15 of an activation row's 256) read the lower half's
+  // addresses instead, so that nothing is read beyond a row, and multiply activations of zero.
   const int nchunk = (K + 127) >> 7;
   constexpr bool half_last = HALF;  // a form of its own: its lane-dependent addresses cost registers
   const int c_lo = wave * nchunk / kWaves;
