@@ -79,10 +79,12 @@ def test_many_tiles(cuda, fmt, with_bias):
 @pytest.mark.parametrize("M,N,K", [(1, 256, 128), (5, 300, 1024), (16, 1001, 2048), (8, 4100, 2176), (3, 64, 8192),
                                    (16, 9000, 5120), (17, 515, 1280), (40, 130, 4096), (64, 8200, 768), (12, 33, 6144),
                                    # K % 128 == 64: the last chunk of 128 k is half empty (2880: a hidden size in use)
-                                   (4, 300, 2880), (16, 5763, 2880), (8, 100, 192), (20, 513, 4160), (3, 2880, 64)])
+                                   (4, 300, 2880), (16, 5763, 2880), (8, 100, 192), (20, 513, 4160), (3, 2880, 64),
+                                   # K beyond 8192: slices of at most 6144 k, running sums in LDS between them
+                                   (8, 300, 14336), (16, 4500, 8320), (5, 130, 28672), (24, 64, 12288)])
 def test_decode_batches(cuda, fmt, with_bias, M, N, K):
-    """Up to 32 rows with K a multiple of 64 up to 8192 (more rows: the tiled kernel): the kernel that keeps the activations in registers and streams
-    weights and scale bytes once per 16 rows.  Ragged N (last block of 16 weight rows, N % 4 != 0), K slices of unequal
+    """Decode batches with K a multiple of 64 (of 128 beyond 8192): the kernel that keeps the activations in registers
+    and streams weights and scale bytes once per 16 rows.  Ragged N (last block of 16 weight rows, N % 4 != 0), K slices of unequal
     length over the eight waves (2176 = 17 chunks, 1280 = 10, 128 = 1), the eight-chunk form with parked activations
     (8192), passes of 16 rows (17, 40, 64), every format, with and without bias."""
     _check(cuda, M, N, K, fmt, scale_bias=127, seed=M + K, with_bias=with_bias)

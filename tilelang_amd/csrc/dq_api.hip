@@ -358,7 +358,7 @@ extern "C" int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const 
   if (scale_bias < 0 || scale_bias > 255) DQ_FAIL("%s: scale_bias must be in 0..255 (got %d)", fn, scale_bias);
   if (!aligned16(A) || !aligned16(B) || !aligned16(C) || (Bias && !aligned16(Bias)))
     DQ_FAIL("%s: A, B, Bias and C must be 16-byte aligned", fn);
-  // a decode batch: activations resident in registers, the weights streamed once per 16 rows (K % 64 == 0, K <= 8192;
+  // a decode batch: activations resident in registers, the weights streamed once per 16 rows (K % 64 == 0, beyond 8192 K % 128 == 0;
   // beyond 16 rows while the passes stay ahead of the tiled kernel: the kernel's launcher decides)
   if (M <= 128) {
     const int rc = mxfp4_gemm_regres(A, B, Scale, Bias, C, M, N, K, fp4_format, scale_bias, 128, (hipStream_t)stream);

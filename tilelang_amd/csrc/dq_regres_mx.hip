@@ -7,7 +7,7 @@
 // the matrix is cut by weight rows over all CUs and by K over the waves of a workgroup, as in dq_regres_i2.hip:
 //
 //   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of 128-k chunks, at most eight:
-//     K <= 8192; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands
+//     K <= 8192, more in slices, see below; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands
 //     of v_mfma_f32_16x16x32_bf16 in registers for the whole kernel (16 rows x 1024 k: 128 registers per lane);
 //   * the workgroups walk the blocks of 16 weight rows.  A chunk of a block is 16 rows x 64 bytes: one 16-byte load
 //     per lane (lane l: piece l % 4 of row l / 4, whole 64-byte runs), then one ds_bpermute_b32 per dword hands lane
@@ -18,6 +18,9 @@
 //     set of the block two before it comes free; the eight partial sums of a block meet in LDS in fp32 (two
 //     buffers, one barrier per block) and 64 threads add them in wave order (the same order every run), add the bias,
 //     round to bf16 and store.
+//
+// K beyond 8192 (K % 128 == 0): slices of at most 6144 k, the kernel's body once per slice with a prologue of its own,
+// the running fp32 sums of the workgroup's blocks kept in LDS between slices (N <= 65536).
 //
 // Every load is unconditional and the last block has its own copy of the code, so that the compiler's count of loads
 // in flight is exact (see dq_regres_i2.hip).  A wave whose slice is shorter than the longest loads its last chunk
@@ -70,7 +73,7 @@ __device__ __forceinline__ bf16x8_t decode8(uint32_t w, const LaneScale& s) {
   else return __builtin_bit_cast(bf16x8_t, simple_fp4x8<7>(w, s.add));
 }
 
-template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF>
+template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF, bool LONGK>
 __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t* __restrict__ A_all, const uint8_t* __restrict__ B,
                                                                    const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias_all,
                                                                    bf16_t* __restrict__ C_all, int M_all, int N, int K, int exp_off) {
@@ -91,13 +94,22 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   // addresses instead, so that nothing is read beyond a row, and multiply activations of zero.
   const int nchunk = (K + 127) >> 7;
   constexpr bool half_last = HALF;  // a form of its own: its lane-dependent addresses cost registers
-  const int c_lo = wave * nchunk / kWaves;
-  const int ncw = (wave + 1) * nchunk / kWaves - c_lo;
+  // LONGK: K beyond what the registers hold goes in slices of at most 8 NCW chunks, equal up to a chunk: the kernel's
+  // body once per slice, with a fresh prologue, the finishing threads' running fp32 sums of the workgroup's blocks in
+  // LDS in between (slice order: the same sums every run).
+  const int nslices = LONGK ? (nchunk + kWaves * NCW - 1) / (kWaves * NCW) : 1;
+  const int row_blocks = (N + 15) >> 4;
+  const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
+  const int mine = (row_blocks - (int)blockIdx.x + step - 1) / step;
+  for (int slice = 0; slice < nslices; ++slice) {
+  if (slice > 0) __syncthreads();  // the partial sums of the slice before are read: their place is free
+  const int sl_lo = slice * nchunk / nslices;
+  const int sl_n = (slice + 1) * nchunk / nslices - sl_lo;
+  const int c_lo = sl_lo + wave * sl_n / kWaves;
+  const int ncw = sl_lo + (wave + 1) * sl_n / kWaves - c_lo;
   auto chunk_of = [&](int i) { return c_lo + min(i, max(ncw - 1, 0)); };  // K < 1024: some waves have no chunk at all
   auto is_half = [&](int i) { return half_last && chunk_of(i) == nchunk - 1; };
 
-  const int row_blocks = (N + 15) >> 4;
-  const int step = gridDim.x;  // at most the number of blocks: every workgroup has one
   int nb = blockIdx.x;
 
   // ---- weights and scales of the block of 16 rows nb
@@ -132,7 +144,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   // The workgroup's first two blocks are asked for before the activations: the memory's first answer takes as long as
   // the prologue, and most matrices give a workgroup two to four blocks, too few for a pipeline that starts one deep.
   // (A condition on a load is harmless here: the wait for the activations below waits for everything before it.)
-  const int mine = (row_blocks - nb + step - 1) / step;
   load_w(w0, sc0, nb);
   if (mine > 1) load_w(w1, sc1, nb + step);
 
@@ -196,7 +207,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     }
     // lane (g, r) holds the weight rows 4 g .. 4 g + 3 of activation row r.  A wave's sums in LDS: [16 activation
     // rows][4 pieces of 4 weight rows], piece p of row m at position p ^ (m & 3).
-    unsigned char* const buf = smem + (it & 1) * (kWaves * kPartial);
+    unsigned char* const buf = smem + ((slice * mine + it) & 1) * (kWaves * kPartial);
     if (r < M) *reinterpret_cast<float4v*>(buf + wave * kPartial + r * 64 + ((g ^ (r & 3)) << 4)) = acc;
     // One barrier per block: the buffer written here is read below and written again two blocks later, after the next
     // block's barrier, which no thread passes before it has finished reading here.
@@ -206,8 +217,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
       float4v sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int w8 = 0; w8 < kWaves; ++w8) sum += *reinterpret_cast<const float4v*>(buf + w8 * kPartial + m * 64 + ((p ^ (m & 3)) << 4));
+      if constexpr (LONGK) {  // this thread's four outputs of the workgroup's block number `it`, behind everything else
+        float4v* const running = reinterpret_cast<float4v*>(smem + kLds + kWaves * PARK * 4096 + it * kPartial + m * 64 + p * 16);
+        if (slice > 0) sum += *running;
+        if (slice + 1 < nslices) *running = sum;
+      }
       const int n = 16 * blk + 4 * p;
-      if (n < N) {
+      if (slice + 1 == nslices && n < N) {
         bf16_t o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -256,15 +272,17 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     do_block(w1, sc1, nb + step, k + 1);
     do_block(w0, sc0, nb + 2 * step, k + 2);
   }
+  }  // slices of K
 }
 
-template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF>
+template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF, bool LONGK>
 int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int exp_off,
                      hipStream_t stream) {
-  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, SVEC, HALF>;
+  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, SVEC, HALF, LONGK>;
   static bool raised[kMaxDevices] = {};
-  constexpr int kLdsAll = kLds + kWaves * parked_chunks(NCW, SVEC) * 4096;
-  if (raise_lds_limit<kLdsAll>(kern, raised)) return -1;
+  constexpr int kMaxRunning = 16;  // blocks of a workgroup whose running sums fit (N <= 65536)
+  constexpr int kLdsFixed = kLds + kWaves * parked_chunks(NCW, SVEC) * 4096;
+  if (raise_lds_limit<kLdsFixed + (LONGK ? kMaxRunning * kPartial : 0)>(kern, raised)) return -1;
   static int cus_of[kMaxDevices] = {};
   int device = 0;
   DQ_CHECK_HIP(hipGetDevice(&device));
@@ -272,6 +290,9 @@ int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bi
   if (!cus_of[device]) DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
   const int row_blocks = (N + 15) / 16;
   const int grid = row_blocks < cus_of[device] ? row_blocks : cus_of[device];
+  const int mine = (row_blocks + grid - 1) / grid;
+  if (LONGK && mine > kMaxRunning) return 1;
+  const int kLdsAll = kLdsFixed + (LONGK ? mine * kPartial : 0);
   hipLaunchKernelGGL(kern, dim3(grid, (M + 15) / 16), dim3(64 * kWaves), kLdsAll, stream, (const bf16_t*)A, (const uint8_t*)B,
                      (const uint8_t*)S, (const bf16_t*)Bias, (bf16_t*)C, M, N, K, exp_off);
   DQ_CHECK_HIP(hipGetLastError());
@@ -285,7 +306,8 @@ int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bi
 int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int fmt,
                       int scale_bias, int max_rows, hipStream_t stream) {
   // 128-k chunks (the last one may be half: K % 128 == 64), at most eight per wave
-  if (M < 1 || M > max_rows || K % 64 != 0 || K > kWaves * kMaxChunks * 128) return 1;
+  const bool longk = K > kWaves * kMaxChunks * 128;
+  if (M < 1 || M > max_rows || K % 64 != 0 || (longk && K % 128 != 0)) return 1;
   // More than 16 rows run as passes of 16, each streaming the weights again: worth it while that stays ahead of the
   // tiled kernel, whose time up to 128 rows is one round of workgroups with all of K behind each (60 us at K = 8192,
   // 92 us from N = 16384 on), against 2.5 us + 4.5 us per 8192 k for every block of 16 weight rows that a workgroup
@@ -295,7 +317,13 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
     const double kfrac = (double)K / 8192.0;
     const long visits = ((long)((N + 15) / 16) * ((M + 15) / 16) + 255) / 256;
     const double t_here = (double)visits * (2.5 + 4.5 * kfrac) + 3.0, t_tiled = (N > 16384 ? 92.0 : 60.0) * kfrac + 3.0;
-    if (t_here > 0.9 * t_tiled) return 1;
+    // K in slices: every slice has a prologue of its own (4.3 us), and the passes of a matrix of many rows come in rounds
+    // (N = 8192, K = 16384 at 16 / 32 / 64 rows 36 / 70 / 136 us against 123 us)
+    const int nslices = ((K >> 7) + kWaves * 6 - 1) / (kWaves * 6);
+    const long grid = (N + 15) / 16 < 256 ? (N + 15) / 16 : 256, blocks_each = ((N + 15) / 16 + grid - 1) / grid;
+    const long rounds = (grid * ((M + 15) / 16) + 255) / 256;
+    const double t_sliced = 3.0 + (double)rounds * (4.3 * nslices + 4.5 * kfrac * (double)blocks_each);
+    if ((longk ? t_sliced : t_here) > 0.9 * t_tiled) return 1;
   }
   const int ncw = (((K + 127) >> 7) + kWaves - 1) / kWaves;
   const int exp_off = 127 - scale_bias;
@@ -304,11 +332,15 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
   if (half && ncw > 6) return 1;  // the half chunk's form with eight chunks per wave does not fit the registers
 #define DQ_MXR(FMT_, NCW_, SVEC_, HALF_)                                                                               \
   do {                                                                                                                 \
-    if (Bias) return launch_mx_regres<FMT_, true, NCW_, SVEC_, HALF_>(A, B, S, Bias, C, M, N, K, exp_off, stream);     \
-    return launch_mx_regres<FMT_, false, NCW_, SVEC_, HALF_>(A, B, S, nullptr, C, M, N, K, exp_off, stream);           \
+    if (Bias) return launch_mx_regres<FMT_, true, NCW_, SVEC_, HALF_, false>(A, B, S, Bias, C, M, N, K, exp_off, stream); \
+    return launch_mx_regres<FMT_, false, NCW_, SVEC_, HALF_, false>(A, B, S, nullptr, C, M, N, K, exp_off, stream);    \
   } while (0)
 #define DQ_MXRN(FMT_)                                     \
   do {                                                    \
+    if (longk) {  /* slices of at most 6144 k: six chunks per wave leave the registers the slice loop needs */        \
+      if (Bias) return launch_mx_regres<FMT_, true, 6, false, false, true>(A, B, S, Bias, C, M, N, K, exp_off, stream);   \
+      return launch_mx_regres<FMT_, false, 6, false, false, true>(A, B, S, nullptr, C, M, N, K, exp_off, stream);         \
+    }                                                     \
     if (svec && ncw == 4) DQ_MXR(FMT_, 4, true, false);   \
     if (svec && ncw == 8) DQ_MXR(FMT_, 8, true, false);   \
     if (half) {                                           \
