@@ -6,7 +6,7 @@
 // such a problem N / 256 workgroups with all of K behind each (N = K = 8192 at 1 to 128 rows: 60 us for 35 MB); here
 // the matrix is cut by weight rows over all CUs and by K over the waves of a workgroup, as in dq_regres_i2.hip:
 //
-//   * one workgroup of eight waves per CU; wave w owns an eighth of K (a run of 128-k chunks, at most eight:
+//   * one workgroup of eight waves per CU; wave w owns an eighth of K (which one turns with the workgroup; a run of 128-k chunks, at most eight:
 //     K <= 8192, more in slices, see below; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands
 //     of v_mfma_f32_16x16x32_bf16 in registers for the whole kernel (16 rows x 1024 k: 128 registers per lane);
 //   * the workgroups walk the blocks of 16 weight rows.  A chunk of a block is 16 rows x 64 bytes: one 16-byte load
@@ -16,7 +16,7 @@
 //     the row's scale bytes per chunk and lane, byte g of it) through the scale operand of the fp4 -> bf16 conversion;
 //   * two sets of weight registers: a workgroup's first two blocks are asked for at once, every further one when the
 //     set of the block two before it comes free; the eight partial sums of a block meet in LDS in fp32 (two
-//     buffers, one barrier per block) and 64 threads add them in wave order (the same order every run), add the bias,
+//     buffers, one barrier per block) and 64 threads add them in slice order (the same order every run), add the bias,
 //     round to bf16 and store.
 //
 // K beyond 8192 (K % 128 == 0): slices of at most 6144 k, the kernel's body once per slice with a prologue of its own,
@@ -105,8 +105,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   if (slice > 0) __syncthreads();  // the partial sums of the slice before are read: their place is free
   const int sl_lo = slice * nchunk / nslices;
   const int sl_n = (slice + 1) * nchunk / nslices - sl_lo;
-  const int c_lo = sl_lo + wave * sl_n / kWaves;
-  const int ncw = sl_lo + (wave + 1) * sl_n / kWaves - c_lo;
+  // Which eighth of K a wave owns turns with the workgroup (the workgroups x, x + 8, ... share an XCD): with wave w on
+  // slice w everywhere, every CU asked the same stretch of every weight row and of the activations at the same time
+  // (N = K = 8192 at 16 rows: 16.0 -> 14.4 us).  The partial sums are still added in slice order.
+  const int kw = (wave + (int)(blockIdx.x >> 3)) & (kWaves - 1);
+  const int c_lo = sl_lo + kw * sl_n / kWaves;
+  const int ncw = sl_lo + (kw + 1) * sl_n / kWaves - c_lo;
   auto chunk_of = [&](int i) { return c_lo + min(i, max(ncw - 1, 0)); };  // K < 1024: some waves have no chunk at all
   auto is_half = [&](int i) { return half_last && chunk_of(i) == nchunk - 1; };
 
@@ -118,9 +122,22 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   auto load_w = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk) __attribute__((always_inline)) {
     const uint8_t* const w_row = B + (size_t)min(16 * blk + (lane >> 2), N - 1) * w_row_bytes;
     const uint8_t* const s_row = S + (size_t)min(16 * blk + r, N - 1) * s_row_bytes;
+    if constexpr (SVEC) {
+      // whole 128-byte lines: a pair of chunks of 8 rows per load (lane l: piece l % 8 of row l / 8), rows 0 .. 7 of the
+      // block into w[2 i], rows 8 .. 15 into w[2 i + 1]; do_block sorts them into chunks.  (16 rows x 64 bytes per load
+      // asks the L2 for every line twice and costs the load unit 16 rows per KiB instead of 8.)
+      const uint8_t* const w_lo = B + (size_t)min(16 * blk + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
+      const uint8_t* const w_hi = B + (size_t)min(16 * blk + 8 + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
 #pragma unroll
-    for (int i = 0; i < NCW; ++i)
-      w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + chunk_of(i) * 64 + ((lane & 3) & (is_half(i) ? 1 : 3)) * 16));
+      for (int i = 0; i < NCW; i += 2) {
+        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_lo + (c_lo + i) * 64));
+        w[i + 1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_hi + (c_lo + i) * 64));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NCW; ++i)
+        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + chunk_of(i) * 64 + ((lane & 3) & (is_half(i) ? 1 : 3)) * 16));
+    }
     // A lane's scale bytes of a block: the dword of every chunk (byte g of it is the lane's).  SVEC (K % 4096 == 0: every
     // wave's run of chunks starts on a multiple of four and is a multiple of four long): 16 bytes, four chunks, per
     // load.  Dword by dword the eight loads of a lane fetched the same 32 bytes eight times from the L2 (nontemporal
@@ -184,7 +201,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     __syncthreads();  // the parking areas are where the partial sums go
   }
 
-  const int w_from = ((lane & 15) * 4 + (lane >> 4)) * 4;  // lane (g, r) of the regrouped register takes lane 4 r + g
+  // lane (g, r) of the regrouped register takes lane 4 r + g.  SVEC: the loaded pair X (rows 0 .. 7), Y (rows 8 .. 15)
+  // becomes the even chunk, X with the upper four lanes of every eight taken from Y's lower four, and the odd chunk, X
+  // with the lower four taken from Y's upper four: row r % 8 + 8 j sits in lanes 8 (r % 8) + 4 j .. + 3 of the even
+  // chunk and in lanes 8 (r % 8) + 4 (1 - j) .. + 3 of the odd one.
+  const int w_from = SVEC ? ((r & 7) * 8 + (r >> 3) * 4 + g) * 4 : ((lane & 15) * 4 + (lane >> 4)) * 4;
   // the thread's share of the final sum: activation row tid / 4, weight rows 4 (tid % 4) .. + 3 of the block
   const int out_m = tid >> 2, out_p = tid & 3;
   const bool finisher = tid < 64 && out_m < M;
@@ -194,8 +215,19 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
 #pragma unroll
     for (int i = 0; i < NCW; ++i) {
       uint4_t x = w[i];
+      if constexpr (SVEC) {
 #pragma unroll
-      for (int d = 0; d < 4; ++d) x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(w_from, (int)x[d]);
+        for (int d = 0; d < 4; ++d) {
+          const int lo8 = (int)w[i & ~1][d], hi8 = (int)w[i | 1][d];
+          // row_shr:4 into lanes 4 .. 7, 12 .. 15 of every 16; row_shl:4 into lanes 0 .. 3, 8 .. 11
+          const int sorted = (i & 1) ? __builtin_amdgcn_update_dpp(lo8, hi8, 0x104, 0xF, 0x5, false)
+                                     : __builtin_amdgcn_update_dpp(lo8, hi8, 0x114, 0xF, 0xA, false);
+          x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute((i & 1) ? (w_from ^ 16) : w_from, sorted);
+        }
+      } else {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(w_from, (int)x[d]);
+      }
       const LaneScale ls = lane_scale<FMT>(SVEC ? (sc[i] >> (8 * g)) & 0xFFu : sc[i], exp_off);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
@@ -208,7 +240,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     // lane (g, r) holds the weight rows 4 g .. 4 g + 3 of activation row r.  A wave's sums in LDS: [16 activation
     // rows][4 pieces of 4 weight rows], piece p of row m at position p ^ (m & 3).
     unsigned char* const buf = smem + ((slice * mine + it) & 1) * (kWaves * kPartial);
-    if (r < M) *reinterpret_cast<float4v*>(buf + wave * kPartial + r * 64 + ((g ^ (r & 3)) << 4)) = acc;
+    if (r < M) *reinterpret_cast<float4v*>(buf + kw * kPartial + r * 64 + ((g ^ (r & 3)) << 4)) = acc;
     // One barrier per block: the buffer written here is read below and written again two blocks later, after the next
     // block's barrier, which no thread passes before it has finished reading here.
     __syncthreads();
