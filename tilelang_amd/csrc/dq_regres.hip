@@ -235,7 +235,10 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
   const int nrb_wg = min(rbn, nrb - rb0);
   const uint32_t row_bytes = (uint32_t)(K >> 1);
   const uint32_t groups_per_row = (uint32_t)(K >> 7);
-  const int chunk0 = wave * NC;
+  // which slice of K a wave owns turns with the workgroup (x, x + 8, ... share an XCD), so that the CUs do not all ask
+  // for the same stretch of the activations and of their weight rows at the same time; sums stay in slice order
+  const int kw = (wave + (int)(blockIdx.x >> 3)) & (WAVES - 1);
+  const int chunk0 = kw * NC;
 
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (uint32_t)N * row_bytes, kBufferFlags);
   const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)S, 0, HAS_SCALE ? (uint32_t)N * groups_per_row * 2u : 0u, kBufferFlags);
@@ -397,7 +400,7 @@ __global__ __launch_bounds__(64 * WAVES) void w4a16_regres_fast_kernel(const hal
     park_scales(rb + 1);
     // total[i] = partial C[m = 4 g + i][(rb0 + rb) * 16 + r] over this wave's K slice
     float* buf = &red[rb & 1][0][0];
-    *reinterpret_cast<float4_t*>(buf + wave * 256 + lane * 4) = total;
+    *reinterpret_cast<float4_t*>(buf + kw * 256 + lane * 4) = total;
     __syncthreads();  // the other buffer is rewritten only after the next barrier
     if (tid < 256 && rb < nrb_wg) {
       float v = buf[tid];

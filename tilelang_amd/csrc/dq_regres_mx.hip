@@ -158,12 +158,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   };
   uint4_t w0[NCW], w1[NCW];
   uint32_t sc0[NCW], sc1[NCW];
-  // The workgroup's first two blocks are asked for before the activations: the memory's first answer takes as long as
-  // the prologue, and most matrices give a workgroup two to four blocks, too few for a pipeline that starts one deep.
-  // (A condition on a load is harmless here: the wait for the activations below waits for everything before it.)
-  load_w(w0, sc0, nb);
-  if (mine > 1) load_w(w1, sc1, nb + step);
-
   // ---- activations: fragment (chunk i, step s): lane (g, r) holds k = 128 chunk + 32 g + 8 s .. + 7 of row r.  Read as
   // whole lines (instruction j: rows 4 j .. 4 j + 3, lane l the 16-byte piece l % 16 of row 4 j + l / 16 of the
   // chunk's 256 bytes), parked in the wave's 4 KiB of LDS (piece q of row m at position q ^ m), read back in operand
@@ -172,7 +166,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   unsigned char* const kept = smem + kLds + wave * (PARK * 4096);  // chunk NR + q at kept + 4096 q, laid out as `park`
   const int kept_rd = r * 256;                                      // piece p of the lane's row: kept_rd + ((p ^ r) << 4)
   bf16x8_t af[NR][4];
+  // The workgroup's first two blocks of weights are asked for in the prologue as well (most matrices give a workgroup
+  // two to four blocks, too few for a pipeline that starts one deep).  Loads come back in the order they went out, and
+  // the first block's arithmetic needs the first block and the activations: so the second block goes out behind the
+  // activations, and their fragments are parked and read back while it is still on its way.
   {
+    load_w(w0, sc0, nb);
     const unsigned char* const a_base = reinterpret_cast<const unsigned char*>(A);
     uint4_t line[NCW][4];
 #pragma unroll
@@ -181,6 +180,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
       for (int j = 0; j < 4; ++j)
         line[i][j] = *reinterpret_cast<const uint4_t*>(a_base + ((size_t)min(4 * j + (lane >> 4), M - 1) * K + 128 * chunk_of(i)) * 2 +
                                                        16 * ((lane & 15) & (is_half(i) ? 7 : 15)));
+    __builtin_amdgcn_sched_barrier(0);
+    if (mine > 1) load_w(w1, sc1, nb + step);
 #pragma unroll
     for (int i = 0; i < NCW; ++i) {
       unsigned char* const park = i < NR ? smem + wave * 4096 : kept + (i - NR) * 4096;
