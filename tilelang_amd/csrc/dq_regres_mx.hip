@@ -119,41 +119,48 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   // ---- weights and scales of the block of 16 rows nb
   // (the chunk numbers are the same for every lane of the wave: scalar registers, not eight offsets per lane)
   const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)(K >> 5);
+  // load_part(.., i): what chunk i's arithmetic leaves free.  Whole 128-byte lines where the wave's run of chunks allows
+  // (SVEC, K % 4096 == 0: every run starts on a multiple of four and is a multiple of four long): a pair of chunks of 8
+  // rows per load (lane l: piece l % 8 of row l / 8), rows 0 .. 7 of the block into w[2 i], rows 8 .. 15 into
+  // w[2 i + 1]; do_block sorts them into chunks.  (16 rows x 64 bytes per load asks the L2 for every line twice and
+  // costs the load unit 16 rows per KiB instead of 8.)  A lane's scale bytes of a block: the dword of every chunk (byte
+  // g of it is the lane's); SVEC: 16 bytes, four chunks, per load.  Dword by dword the eight loads of a lane fetched the
+  // same 32 bytes eight times from the L2 (nontemporal loads leave nothing in the L1): 12 of 48 us at N = 28672,
+  // K = 8192.
+  struct RowPtrs {
+    const uint8_t *w_lo, *w_hi, *s_row;
+  };
+  auto rows_of = [&](int blk) __attribute__((always_inline)) {
+    RowPtrs p;
+    if constexpr (SVEC) {
+      p.w_lo = B + (size_t)min(16 * blk + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
+      p.w_hi = B + (size_t)min(16 * blk + 8 + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
+    } else {
+      p.w_lo = p.w_hi = B + (size_t)min(16 * blk + (lane >> 2), N - 1) * w_row_bytes;
+    }
+    p.s_row = S + (size_t)min(16 * blk + r, N - 1) * s_row_bytes;
+    return p;
+  };
+  auto load_part = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], const RowPtrs& p, int i) __attribute__((always_inline)) {
+    if constexpr (SVEC) {
+      if (i & 1) {
+        w[i - 1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_lo + (c_lo + i - 1) * 64));
+        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_hi + (c_lo + i - 1) * 64));
+      }
+      if ((i & 3) == 3) {
+        const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.s_row + c_lo * 4 + (i - 3) * 4));
+        sc[i - 3] = v[0], sc[i - 2] = v[1], sc[i - 1] = v[2], sc[i] = v[3];
+      }
+    } else {
+      w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_lo + chunk_of(i) * 64 + ((lane & 3) & (is_half(i) ? 1 : 3)) * 16));
+      sc[i] = p.s_row[chunk_of(i) * 4 + (g & (is_half(i) ? 1 : 3))];  // the lane's own byte
+    }
+  };
   auto load_w = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk) __attribute__((always_inline)) {
-    const uint8_t* const w_row = B + (size_t)min(16 * blk + (lane >> 2), N - 1) * w_row_bytes;
-    const uint8_t* const s_row = S + (size_t)min(16 * blk + r, N - 1) * s_row_bytes;
-    if constexpr (SVEC) {
-      // whole 128-byte lines: a pair of chunks of 8 rows per load (lane l: piece l % 8 of row l / 8), rows 0 .. 7 of the
-      // block into w[2 i], rows 8 .. 15 into w[2 i + 1]; do_block sorts them into chunks.  (16 rows x 64 bytes per load
-      // asks the L2 for every line twice and costs the load unit 16 rows per KiB instead of 8.)
-      const uint8_t* const w_lo = B + (size_t)min(16 * blk + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
-      const uint8_t* const w_hi = B + (size_t)min(16 * blk + 8 + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
+    const RowPtrs p = rows_of(blk);
 #pragma unroll
-      for (int i = 0; i < NCW; i += 2) {
-        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_lo + (c_lo + i) * 64));
-        w[i + 1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_hi + (c_lo + i) * 64));
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NCW; ++i)
-        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + chunk_of(i) * 64 + ((lane & 3) & (is_half(i) ? 1 : 3)) * 16));
-    }
-    // A lane's scale bytes of a block: the dword of every chunk (byte g of it is the lane's).  SVEC (K % 4096 == 0: every
-    // wave's run of chunks starts on a multiple of four and is a multiple of four long): 16 bytes, four chunks, per
-    // load.  Dword by dword the eight loads of a lane fetched the same 32 bytes eight times from the L2 (nontemporal
-    // loads leave nothing in the L1): 12 of 48 us at N = 28672, K = 8192.
-    if constexpr (SVEC) {
-#pragma unroll
-      for (int i = 0; i < NCW; i += 4) {
-        const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(s_row + c_lo * 4 + i * 4));
-        sc[i] = v[0], sc[i + 1] = v[1], sc[i + 2] = v[2], sc[i + 3] = v[3];
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NCW; ++i) sc[i] = s_row[chunk_of(i) * 4 + (g & (is_half(i) ? 1 : 3))];  // the lane's own byte
-    }
-    // the loads go out here, ahead of the arithmetic of the block before: left to itself the scheduler sinks them
-    // behind it to save registers, and the block ahead is then waited for right after it was asked for
+    for (int i = 0; i < NCW; ++i) load_part(w, sc, p, i);
+    // the loads go out here, ahead of what follows: left to itself the scheduler sinks them to save registers
     __builtin_amdgcn_sched_barrier(0);
   };
   uint4_t w0[NCW], w1[NCW];
@@ -211,7 +218,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   const int out_m = tid >> 2, out_p = tid & 3;
   const bool finisher = tid < 64 && out_m < M;
 
-  auto do_block = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk, int it) __attribute__((always_inline)) {
+  // next_tag: whether the set takes the workgroup's block after the next (blk + 2 step) as this one is consumed: every
+  // chunk's registers are asked for again as soon as its arithmetic is out, not when the whole block is done (with two
+  // sets of registers that is what keeps close to two blocks per CU in flight).
+  auto do_block = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], int blk, int it, auto next_tag) __attribute__((always_inline)) {
+    constexpr bool reload = decltype(next_tag)::value;
+    const RowPtrs nxt = rows_of(reload ? blk + 2 * step : blk);
     float4v acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < NCW; ++i) {
@@ -236,6 +248,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
         if (i < NR) a = af[i < NR ? i : 0][s];
         else a = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4_t*>(kept + (i - NR) * 4096 + kept_rd + (((4 * g + s) ^ r) << 4)));
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(decode8<FMT>(x[s], ls), a, acc, 0, 0, 0);
+      }
+      if constexpr (reload) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_part(w, sc, nxt, i);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     // lane (g, r) holds the weight rows 4 g .. 4 g + 3 of activation row r.  A wave's sums in LDS: [16 activation
@@ -280,30 +297,28 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     }
   };
 
-  // w0 holds the workgroup's block k, w1 block k + 1; a set is asked for again (block k + 2) as soon as its block is
-  // done.  The loop over pairs of blocks that both have a successor has no exit in its body, and the last one to three
-  // blocks follow it in copies of their own: a load under a condition, or an exit that shares its way out with the
-  // loop's way round, would make the compiler count the loads in flight for a path that does not have them, and wait
-  // for everything at the top of the loop.
+  // w0 holds the workgroup's block k, w1 block k + 1.  The loop over pairs of blocks that both have a successor has no
+  // exit in its body, and the last one to three blocks follow it in copies of their own: a load under a condition, or
+  // an exit that shares its way out with the loop's way round, would make the compiler count the loads in flight for a
+  // path that does not have them, and wait for everything at the top of the loop.
+  constexpr std::true_type more{};
+  constexpr std::false_type last{};
   int k = 0;
   for (; k + 4 <= mine; k += 2) {
-    do_block(w0, sc0, nb, k);
-    load_w(w0, sc0, nb + 2 * step);
-    do_block(w1, sc1, nb + step, k + 1);
-    load_w(w1, sc1, nb + 3 * step);
+    do_block(w0, sc0, nb, k, more);
+    do_block(w1, sc1, nb + step, k + 1, more);
     nb += 2 * step;
   }
   const int left = mine - k;
   if (left == 1) {
-    do_block(w0, sc0, nb, k);
+    do_block(w0, sc0, nb, k, last);
   } else if (left == 2) {
-    do_block(w0, sc0, nb, k);
-    do_block(w1, sc1, nb + step, k + 1);
+    do_block(w0, sc0, nb, k, last);
+    do_block(w1, sc1, nb + step, k + 1, last);
   } else {
-    do_block(w0, sc0, nb, k);
-    load_w(w0, sc0, nb + 2 * step);
-    do_block(w1, sc1, nb + step, k + 1);
-    do_block(w0, sc0, nb + 2 * step, k + 2);
+    do_block(w0, sc0, nb, k, more);
+    do_block(w1, sc1, nb + step, k + 1, last);
+    do_block(w0, sc0, nb + 2 * step, k + 2, last);
   }
   }  // slices of K
 }
