@@ -322,9 +322,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres16_kernel(const int8_
   const bool finisher = tid < 64 && out_m < M;
   const typename FIN::row_t out_row = fin.row(finisher ? out_m : 0);
   uint4_t w[kDepth16][NPW];
+  // Loads come back in the order they went out, and the first block's arithmetic needs the first block and the
+  // activations: the two blocks ahead go out behind the activations.
   load_w(w[0], nb0, true);
-  load_w(w[1], nb0 + step, mine > 1);
-  load_w(w[2], nb0 + 2 * step, mine > 2);
 
   // ---- activations: fragment (pair i, step s): lane (g, r) holds k = 256 pair + 64 g + 16 s .. + 15 of row r; read as
   // whole lines (instruction j: rows 4 j .. 4 j + 3, lane l the piece l % 16 of row 4 j + l / 16), parked in the
@@ -338,6 +338,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void i2_regres16_kernel(const int8_
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         line[i][j] = *reinterpret_cast<const uint4_t*>(a_lane + (size_t)min(4 * j + (lane >> 4), M - 1) * K + 256 * pair_of(i));
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(w[1], nb0 + step, mine > 1);
+    load_w(w[2], nb0 + 2 * step, mine > 2);
     unsigned char* const park = smem + wave * 4096;
 #pragma unroll
     for (int i = 0; i < NPW; ++i) {
