@@ -358,20 +358,18 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
   if (M < 1 || M > max_rows || K % 64 != 0 || (longk && K % 128 != 0)) return 1;
   // More than 16 rows run as passes of 16, each streaming the weights again: worth it while that stays ahead of the
   // tiled kernel, whose time up to 128 rows is one round of workgroups with all of K behind each (60 us at K = 8192,
-  // 92 us from N = 16384 on), against 2.5 us + 4.5 us per 8192 k for every block of 16 weight rows that a workgroup
-  // visits here (measured: N = K = 8192 at 32 / 48 / 64 rows 32 / 46 / 61 us against 61 us; N = K = 2880, where the
-  // passes share a round, 11 / 15 / 16 us and at 128 rows 29 us against 24.6 us).
+  // 92 us from N = 16384 on).  Here the passes' workgroups come in rounds of one per CU, and a workgroup takes its
+  // prologue (2 us + 2.5 us per 8192 k, once per slice of K) and 0.3 us + 2.8 us per 8192 k for every block of 16
+  // weight rows it visits (measured at K = 8192: N = 8192 at 16 / 32 / 48 rows 13 / 24 / 35 us, N = 28672 at 16 rows
+  // 26.6 us; N = K = 2880, where the passes share a round, 16 / 32 / 64 / 128 rows 6.7 / 11 / 16 / 29 us against 24.6 us).
   if (M > 16) {
     const double kfrac = (double)K / 8192.0;
-    const long visits = ((long)((N + 15) / 16) * ((M + 15) / 16) + 255) / 256;
-    const double t_here = (double)visits * (2.5 + 4.5 * kfrac) + 3.0, t_tiled = (N > 16384 ? 92.0 : 60.0) * kfrac + 3.0;
-    // K in slices: every slice has a prologue of its own (4.3 us), and the passes of a matrix of many rows come in rounds
-    // (N = 8192, K = 16384 at 16 / 32 / 64 rows 36 / 70 / 136 us against 123 us)
-    const int nslices = ((K >> 7) + kWaves * 6 - 1) / (kWaves * 6);
+    const int nslices = longk ? ((K >> 7) + kWaves * 6 - 1) / (kWaves * 6) : 1;
     const long grid = (N + 15) / 16 < 256 ? (N + 15) / 16 : 256, blocks_each = ((N + 15) / 16 + grid - 1) / grid;
     const long rounds = (grid * ((M + 15) / 16) + 255) / 256;
-    const double t_sliced = 3.0 + (double)rounds * (4.3 * nslices + 4.5 * kfrac * (double)blocks_each);
-    if ((longk ? t_sliced : t_here) > 0.9 * t_tiled) return 1;
+    const double t_here = 2.0 + 1.1 * (double)rounds * (2.0 * nslices + 2.5 * kfrac + (double)blocks_each * (0.3 * nslices + 2.8 * kfrac));
+    const double t_tiled = (N > 16384 ? 92.0 : 60.0) * kfrac + 3.0;
+    if (t_here > 0.9 * t_tiled) return 1;
   }
   const int ncw = (((K + 127) >> 7) + kWaves - 1) / kWaves;
   const int exp_off = 127 - scale_bias;
