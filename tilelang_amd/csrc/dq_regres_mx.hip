@@ -42,7 +42,7 @@ constexpr int kLds = kWaves * 4096;    // the prologue's parking areas; the two 
 // do not fit 256 registers: the fragments of the wave's last three chunks (four where the scale bytes are loaded one
 // by one: eight more addresses) stay parked in LDS, 4 KiB per wave and chunk behind the areas above, and are read
 // again for every block.
-constexpr int parked_chunks(int ncw, bool svec) { return ncw == 8 ? (svec ? 3 : 4) : 0; }
+constexpr int parked_chunks(int ncw, int lines) { return ncw == 8 ? (lines ? 3 : 4) : 0; }
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 
@@ -73,7 +73,10 @@ __device__ __forceinline__ bf16x8_t decode8(uint32_t w, const LaneScale& s) {
   else return __builtin_bit_cast(bf16x8_t, simple_fp4x8<7>(w, s.add));
 }
 
-template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF, bool LONGK>
+// LINES: 0: K % 64 == 0, a load per chunk of 16 rows x 64 bytes and a byte of scale per chunk and lane; 1: K % 256 == 0,
+// the waves' runs are whole pairs of chunks, weights fetched as whole 128-byte lines and scales 8 bytes (a pair) at a
+// time; 2: K % 4096 == 0, every run starts on a multiple of four chunks and is as long: scales 16 bytes at a time.
+template <int FMT, bool HAS_BIAS, int NCW, int LINES, bool HALF, bool LONGK>
 __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t* __restrict__ A_all, const uint8_t* __restrict__ B,
                                                                    const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias_all,
                                                                    bf16_t* __restrict__ C_all, int M_all, int N, int K, int exp_off) {
@@ -83,6 +86,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   bf16_t* const C = C_all + (size_t)m_first * N;
   const bf16_t* const Bias = HAS_BIAS ? Bias_all + (size_t)m_first * N : nullptr;
   const int M = min(M_all - m_first, 16);
+  constexpr bool PAIR = LINES >= 1, SVEC = LINES == 2;
+  static_assert(!PAIR || (NCW % 2 == 0 && !HALF), "whole pairs of whole chunks");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -103,15 +108,20 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   const int mine = (row_blocks - (int)blockIdx.x + step - 1) / step;
   for (int slice = 0; slice < nslices; ++slice) {
   if (slice > 0) __syncthreads();  // the partial sums of the slice before are read: their place is free
-  const int sl_lo = slice * nchunk / nslices;
-  const int sl_n = (slice + 1) * nchunk / nslices - sl_lo;
+  // (PAIR: slices and runs are cut in whole pairs of chunks)
+  constexpr int U = PAIR ? 2 : 1;
+  const int nunit = nchunk / U;
+  const int sl_lo = slice * nunit / nslices;
+  const int sl_n = (slice + 1) * nunit / nslices - sl_lo;
   // Which eighth of K a wave owns turns with the workgroup (the workgroups x, x + 8, ... share an XCD): with wave w on
   // slice w everywhere, every CU asked the same stretch of every weight row and of the activations at the same time
   // (N = K = 8192 at 16 rows: 16.0 -> 14.4 us).  The partial sums are still added in slice order.
   const int kw = (wave + (int)(blockIdx.x >> 3)) & (kWaves - 1);
-  const int c_lo = sl_lo + kw * sl_n / kWaves;
-  const int ncw = sl_lo + (kw + 1) * sl_n / kWaves - c_lo;
-  auto chunk_of = [&](int i) { return c_lo + min(i, max(ncw - 1, 0)); };  // K < 1024: some waves have no chunk at all
+  const int u_lo = sl_lo + kw * sl_n / kWaves;
+  const int nuw = sl_lo + (kw + 1) * sl_n / kWaves - u_lo;
+  const int c_lo = U * u_lo, ncw = U * nuw;
+  // K < 1024: some waves have no chunk at all
+  auto chunk_of = [&](int i) { return c_lo + U * min(i / U, max(nuw - 1, 0)) + i % U; };
   auto is_half = [&](int i) { return half_last && chunk_of(i) == nchunk - 1; };
 
   int nb = blockIdx.x;
@@ -119,20 +129,19 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   // ---- weights and scales of the block of 16 rows nb
   // (the chunk numbers are the same for every lane of the wave: scalar registers, not eight offsets per lane)
   const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)(K >> 5);
-  // load_part(.., i): what chunk i's arithmetic leaves free.  Whole 128-byte lines where the wave's run of chunks allows
-  // (SVEC, K % 4096 == 0: every run starts on a multiple of four and is a multiple of four long): a pair of chunks of 8
-  // rows per load (lane l: piece l % 8 of row l / 8), rows 0 .. 7 of the block into w[2 i], rows 8 .. 15 into
-  // w[2 i + 1]; do_block sorts them into chunks.  (16 rows x 64 bytes per load asks the L2 for every line twice and
-  // costs the load unit 16 rows per KiB instead of 8.)  A lane's scale bytes of a block: the dword of every chunk (byte
-  // g of it is the lane's); SVEC: 16 bytes, four chunks, per load.  Dword by dword the eight loads of a lane fetched the
-  // same 32 bytes eight times from the L2 (nontemporal loads leave nothing in the L1): 12 of 48 us at N = 28672,
-  // K = 8192.
+  // load_part(.., i): what chunk i's arithmetic leaves free.  Whole 128-byte lines where K allows (PAIR): a pair of
+  // chunks of 8 rows per load (lane l: piece l % 8 of row l / 8), rows 0 .. 7 of the block into w[2 j], rows 8 .. 15
+  // into w[2 j + 1]; do_block sorts them into chunks.  (16 rows x 64 bytes per load asks the L2 for every line twice
+  // and costs the load unit 16 rows per KiB instead of 8.)  A lane's scale bytes of a block: the dword of every chunk
+  // (byte g of it is the lane's), 8 bytes (a pair) or 16 bytes (four chunks, SVEC) per load; without PAIR the lane's own
+  // byte.  Dword by dword the eight loads of a lane fetched the same 32 bytes eight times from the L2 (nontemporal
+  // loads leave nothing in the L1): 12 of 48 us at N = 28672, K = 8192.
   struct RowPtrs {
     const uint8_t *w_lo, *w_hi, *s_row;
   };
   auto rows_of = [&](int blk) __attribute__((always_inline)) {
     RowPtrs p;
-    if constexpr (SVEC) {
+    if constexpr (PAIR) {
       p.w_lo = B + (size_t)min(16 * blk + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
       p.w_hi = B + (size_t)min(16 * blk + 8 + (lane >> 3), N - 1) * w_row_bytes + (lane & 7) * 16;
     } else {
@@ -142,14 +151,21 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     return p;
   };
   auto load_part = [&](uint4_t (&w)[NCW], uint32_t (&sc)[NCW], const RowPtrs& p, int i) __attribute__((always_inline)) {
-    if constexpr (SVEC) {
+    if constexpr (PAIR) {
       if (i & 1) {
-        w[i - 1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_lo + (c_lo + i - 1) * 64));
-        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_hi + (c_lo + i - 1) * 64));
+        w[i - 1] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_lo + chunk_of(i - 1) * 64));
+        w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_hi + chunk_of(i - 1) * 64));
+        if constexpr (!SVEC) {
+          typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+          const uint2v v = __builtin_nontemporal_load(reinterpret_cast<const uint2v*>(p.s_row + chunk_of(i - 1) * 4));
+          sc[i - 1] = v[0], sc[i] = v[1];
+        }
       }
-      if ((i & 3) == 3) {
-        const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.s_row + c_lo * 4 + (i - 3) * 4));
-        sc[i - 3] = v[0], sc[i - 2] = v[1], sc[i - 1] = v[2], sc[i] = v[3];
+      if constexpr (SVEC) {
+        if ((i & 3) == 3) {
+          const uint4_t v = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.s_row + c_lo * 4 + (i - 3) * 4));
+          sc[i - 3] = v[0], sc[i - 2] = v[1], sc[i - 1] = v[2], sc[i] = v[3];
+        }
       }
     } else {
       w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p.w_lo + chunk_of(i) * 64 + ((lane & 3) & (is_half(i) ? 1 : 3)) * 16));
@@ -169,7 +185,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   // whole lines (instruction j: rows 4 j .. 4 j + 3, lane l the 16-byte piece l % 16 of row 4 j + l / 16 of the
   // chunk's 256 bytes), parked in the wave's 4 KiB of LDS (piece q of row m at position q ^ m), read back in operand
   // order: fetched in that order a load instruction would touch 32 cache lines for 32 bytes each.
-  constexpr int PARK = parked_chunks(NCW, SVEC), NR = NCW - PARK;
+  constexpr int PARK = parked_chunks(NCW, LINES), NR = NCW - PARK;
   unsigned char* const kept = smem + kLds + wave * (PARK * 4096);  // chunk NR + q at kept + 4096 q, laid out as `park`
   const int kept_rd = r * 256;                                      // piece p of the lane's row: kept_rd + ((p ^ r) << 4)
   bf16x8_t af[NR][4];
@@ -209,11 +225,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
     __syncthreads();  // the parking areas are where the partial sums go
   }
 
-  // lane (g, r) of the regrouped register takes lane 4 r + g.  SVEC: the loaded pair X (rows 0 .. 7), Y (rows 8 .. 15)
+  // lane (g, r) of the regrouped register takes lane 4 r + g.  PAIR: the loaded pair X (rows 0 .. 7), Y (rows 8 .. 15)
   // becomes the even chunk, X with the upper four lanes of every eight taken from Y's lower four, and the odd chunk, X
   // with the lower four taken from Y's upper four: row r % 8 + 8 j sits in lanes 8 (r % 8) + 4 j .. + 3 of the even
   // chunk and in lanes 8 (r % 8) + 4 (1 - j) .. + 3 of the odd one.
-  const int w_from = SVEC ? ((r & 7) * 8 + (r >> 3) * 4 + g) * 4 : ((lane & 15) * 4 + (lane >> 4)) * 4;
+  const int w_from = PAIR ? ((r & 7) * 8 + (r >> 3) * 4 + g) * 4 : ((lane & 15) * 4 + (lane >> 4)) * 4;
   // the thread's share of the final sum: activation row tid / 4, weight rows 4 (tid % 4) .. + 3 of the block
   const int out_m = tid >> 2, out_p = tid & 3;
   const bool finisher = tid < 64 && out_m < M;
@@ -228,7 +244,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
 #pragma unroll
     for (int i = 0; i < NCW; ++i) {
       uint4_t x = w[i];
-      if constexpr (SVEC) {
+      if constexpr (PAIR) {
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
           const int lo8 = (int)w[i & ~1][d], hi8 = (int)w[i | 1][d];
@@ -241,7 +257,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
 #pragma unroll
         for (int d = 0; d < 4; ++d) x[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(w_from, (int)x[d]);
       }
-      const LaneScale ls = lane_scale<FMT>(SVEC ? (sc[i] >> (8 * g)) & 0xFFu : sc[i], exp_off);
+      const LaneScale ls = lane_scale<FMT>(PAIR ? (sc[i] >> (8 * g)) & 0xFFu : sc[i], exp_off);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         bf16x8_t a;
@@ -323,13 +339,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void mx_regres_kernel(const bf16_t*
   }  // slices of K
 }
 
-template <int FMT, bool HAS_BIAS, int NCW, bool SVEC, bool HALF, bool LONGK>
+template <int FMT, bool HAS_BIAS, int NCW, int LINES, bool HALF, bool LONGK>
 int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K, int exp_off,
                      hipStream_t stream) {
-  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, SVEC, HALF, LONGK>;
+  auto kern = mx_regres_kernel<FMT, HAS_BIAS, NCW, LINES, HALF, LONGK>;
   static bool raised[kMaxDevices] = {};
   constexpr int kMaxRunning = 16;  // blocks of a workgroup whose running sums fit (N <= 65536)
-  constexpr int kLdsFixed = kLds + kWaves * parked_chunks(NCW, SVEC) * 4096;
+  constexpr int kLdsFixed = kLds + kWaves * parked_chunks(NCW, LINES) * 4096;
   if (raise_lds_limit<kLdsFixed + (LONGK ? kMaxRunning * kPartial : 0)>(kern, raised)) return -1;
   static int cus_of[kMaxDevices] = {};
   int device = 0;
@@ -371,33 +387,41 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
     const double t_tiled = (N > 16384 ? 92.0 : 60.0) * kfrac + 3.0;
     if (t_here > 0.9 * t_tiled) return 1;
   }
-  const int ncw = (((K + 127) >> 7) + kWaves - 1) / kWaves;
   const int exp_off = 127 - scale_bias;
-  const bool svec = K % 4096 == 0;
   const bool half = K % 128 != 0;
+  const int lines = K % 4096 == 0 ? 2 : (K % 256 == 0 ? 1 : 0);
+  // chunks per wave: the longest run (with lines, whole pairs)
+  const int nchunk = (K + 127) >> 7;
+  const int ncw = lines ? 2 * ((nchunk / 2 + kWaves - 1) / kWaves) : (nchunk + kWaves - 1) / kWaves;
   if (half && ncw > 6) return 1;  // the half chunk's form with eight chunks per wave does not fit the registers
-#define DQ_MXR(FMT_, NCW_, SVEC_, HALF_)                                                                               \
-  do {                                                                                                                 \
-    if (Bias) return launch_mx_regres<FMT_, true, NCW_, SVEC_, HALF_, false>(A, B, S, Bias, C, M, N, K, exp_off, stream); \
-    return launch_mx_regres<FMT_, false, NCW_, SVEC_, HALF_, false>(A, B, S, nullptr, C, M, N, K, exp_off, stream);    \
+#define DQ_MXR(FMT_, NCW_, LINES_, HALF_, LONGK_)                                                                            \
+  do {                                                                                                                       \
+    if (Bias) return launch_mx_regres<FMT_, true, NCW_, LINES_, HALF_, LONGK_>(A, B, S, Bias, C, M, N, K, exp_off, stream); \
+    return launch_mx_regres<FMT_, false, NCW_, LINES_, HALF_, LONGK_>(A, B, S, nullptr, C, M, N, K, exp_off, stream);       \
   } while (0)
-#define DQ_MXRN(FMT_)                                     \
-  do {                                                    \
-    if (longk) {  /* slices of at most 6144 k: six chunks per wave leave the registers the slice loop needs */        \
-      if (Bias) return launch_mx_regres<FMT_, true, 6, false, false, true>(A, B, S, Bias, C, M, N, K, exp_off, stream);   \
-      return launch_mx_regres<FMT_, false, 6, false, false, true>(A, B, S, nullptr, C, M, N, K, exp_off, stream);         \
-    }                                                     \
-    if (svec && ncw == 4) DQ_MXR(FMT_, 4, true, false);   \
-    if (svec && ncw == 8) DQ_MXR(FMT_, 8, true, false);   \
-    if (half) {                                           \
-      if (ncw <= 2) DQ_MXR(FMT_, 2, false, true);         \
-      if (ncw <= 4) DQ_MXR(FMT_, 4, false, true);         \
-      DQ_MXR(FMT_, 6, false, true);                       \
-    }                                                     \
-    if (ncw <= 2) DQ_MXR(FMT_, 2, false, false);          \
-    if (ncw <= 4) DQ_MXR(FMT_, 4, false, false);          \
-    if (ncw <= 6) DQ_MXR(FMT_, 6, false, false);          \
-    DQ_MXR(FMT_, 8, false, false);                        \
+#define DQ_MXRN(FMT_)                                                                                          \
+  do {                                                                                                         \
+    if (longk) { /* slices of at most 6144 k: six chunks per wave leave the registers the slice loop needs */ \
+      if (lines) DQ_MXR(FMT_, 6, 1, false, true);                                                              \
+      DQ_MXR(FMT_, 6, 0, false, true);                                                                         \
+    }                                                                                                          \
+    if (lines == 2 && ncw == 4) DQ_MXR(FMT_, 4, 2, false, false);                                              \
+    if (lines == 2 && ncw == 8) DQ_MXR(FMT_, 8, 2, false, false);                                              \
+    if (lines) {                                                                                               \
+      if (ncw <= 2) DQ_MXR(FMT_, 2, 1, false, false);                                                          \
+      if (ncw <= 4) DQ_MXR(FMT_, 4, 1, false, false);                                                          \
+      if (ncw <= 6) DQ_MXR(FMT_, 6, 1, false, false);                                                          \
+      DQ_MXR(FMT_, 8, 1, false, false);                                                                        \
+    }                                                                                                          \
+    if (half) {                                                                                                \
+      if (ncw <= 2) DQ_MXR(FMT_, 2, 0, true, false);                                                           \
+      if (ncw <= 4) DQ_MXR(FMT_, 4, 0, true, false);                                                           \
+      DQ_MXR(FMT_, 6, 0, true, false);                                                                         \
+    }                                                                                                          \
+    if (ncw <= 2) DQ_MXR(FMT_, 2, 0, false, false);                                                            \
+    if (ncw <= 4) DQ_MXR(FMT_, 4, 0, false, false);                                                            \
+    if (ncw <= 6) DQ_MXR(FMT_, 6, 0, false, false);                                                            \
+    DQ_MXR(FMT_, 8, 0, false, false);                                                                          \
   } while (0)
   switch (fmt) {
     case FP4_E2M1: DQ_MXRN(FP4_E2M1);
