@@ -50,7 +50,8 @@ def gemv_hbm_traffic():
 
 
 #: False (--no-graph): time plain back-to-back launches.  For runs under a profiler that collects hardware counters: it
-#: serialises the kernels itself, and a replayed graph whose calls are two dependent kernels did not come back under it.
+#: serialises the kernels itself, and a replayed graph whose calls are two dependent kernels did not come back under it
+#: (that row, the K split over workgroups, is left out of such runs altogether).
 USE_GRAPH = True
 
 
@@ -511,9 +512,12 @@ def main():
             row = _row(f"w4a16_zeros M={m} N=28672 K=8192", r, "hbm", MFMA_BF16_PEAK)
             row["frac_mfma"] = r["flops"] / (r["us"] * 1e-6) / MFMA_BF16_PEAK
             shapes.append(row)
-        # a matrix of few rows and a long K: K split over workgroups, fp32 partial sums in a workspace
-        r = bench_w4a16(torch, tl, workloads, 16, 4096, 14336, True, S, W, dev)
-        shapes.append(_row("w4a16_zeros M=16 N=4096 K=14336", r, "hbm", MFMA_BF16_PEAK))
+        # a matrix of few rows and a long K: K split over workgroups, fp32 partial sums in a workspace.  Left out of
+        # counter runs (--no-graph): under `rocprofv3 --pmc` this row's pair of dependent kernels has stalled, as a
+        # replayed graph and once as plain launches, while tests, timing and the kernel trace run it without trouble.
+        if USE_GRAPH:
+            r = bench_w4a16(torch, tl, workloads, 16, 4096, 14336, True, S, W, dev)
+            shapes.append(_row("w4a16_zeros M=16 N=4096 K=14336", r, "hbm", MFMA_BF16_PEAK))
         for m in (4, 16):
             r = bench_w4a16(torch, tl, workloads, m, 28672, 8192, True, S, W, dev, fragments=True)
             shapes.append(_row(f"w4a16_zeros M={m} N=28672 K=8192 (weights re-ordered offline into the matrix instruction's operand order)",
