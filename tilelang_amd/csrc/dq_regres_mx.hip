@@ -6,25 +6,30 @@
 // such a problem N / 256 workgroups with all of K behind each (N = K = 8192 at 1 to 128 rows: 60 us for 35 MB); here
 // the matrix is cut by weight rows over all CUs and by K over the waves of a workgroup, as in dq_regres_i2.hip:
 //
-//   * one workgroup of eight waves per CU; wave w owns an eighth of K (which one turns with the workgroup; a run of 128-k chunks, at most eight:
-//     K <= 8192, more in slices, see below; K % 128 == 64 leaves the last chunk half empty) and keeps the activations of its slice as operands
-//     of v_mfma_f32_16x16x32_bf16 in registers for the whole kernel (16 rows x 1024 k: 128 registers per lane);
-//   * the workgroups walk the blocks of 16 weight rows.  A chunk of a block is 16 rows x 64 bytes: one 16-byte load
-//     per lane (lane l: piece l % 4 of row l / 4, whole 64-byte runs), then one ds_bpermute_b32 per dword hands lane
-//     (g, r) piece g of row r.  Dword s of a lane feeds step s, contraction index k = 128 chunk + 32 g + 8 s + e for
-//     both operands: a lane's 32 codes are ONE scale block, so the lane applies one E8M0 byte per chunk (a dword of
-//     the row's scale bytes per chunk and lane, byte g of it) through the scale operand of the fp4 -> bf16 conversion;
-//   * two sets of weight registers: a workgroup's first two blocks are asked for at once, every further one when the
-//     set of the block two before it comes free; the eight partial sums of a block meet in LDS in fp32 (two
-//     buffers, one barrier per block) and 64 threads add them in slice order (the same order every run), add the bias,
-//     round to bf16 and store.
+//   * one workgroup of eight waves per CU; a wave owns an eighth of K (which one turns with the workgroup): a run of
+//     128-k chunks, at most eight (K <= 8192; more in slices, see below; K % 128 == 64 leaves the last chunk half
+//     empty), and keeps the activations of its slice as operands of v_mfma_f32_16x16x32_bf16 in registers for the
+//     whole kernel (16 rows x 1024 k: 128 registers per lane);
+//   * the workgroups walk the blocks of 16 weight rows.  With K % 256 == 0 the runs are whole pairs of chunks and a
+//     load takes 8 rows x 128 bytes (whole cache lines; lane l: piece l % 8 of row l / 8), two DPP moves sort a pair
+//     of loads (rows 0 .. 7, rows 8 .. 15) into the even and the odd chunk; otherwise a load is a chunk of 16 rows x
+//     64 bytes.  One ds_bpermute_b32 per dword then hands lane (g, r) piece g of row r of the chunk.  Dword s of a
+//     lane feeds step s, contraction index k = 128 chunk + 32 g + 8 s + e for both operands: a lane's 32 codes are
+//     ONE scale block, so the lane applies one E8M0 byte per chunk (byte g of the row's dword of scale bytes for the
+//     chunk; 8 or 16 bytes of them per load) through the scale operand of the fp4 -> bf16 conversion;
+//   * two sets of weight registers.  The workgroup's first block is asked for ahead of the activations and its
+//     second behind them (loads come back in the order they went out); after that every chunk's registers are asked
+//     for again, for the block after the next, as soon as the chunk's arithmetic is out.  The eight partial sums of
+//     a block meet in LDS in fp32 (two buffers, one barrier per block) and 64 threads add them in slice order (the
+//     same order every run), add the bias, round to bf16 and store.
 //
 // K beyond 8192 (K % 128 == 0): slices of at most 6144 k, the kernel's body once per slice with a prologue of its own,
 // the running fp32 sums of the workgroup's blocks kept in LDS between slices (N <= 65536).
 //
-// Every load is unconditional and the last block has its own copy of the code, so that the compiler's count of loads
-// in flight is exact (see dq_regres_i2.hip).  A wave whose slice is shorter than the longest loads its last chunk
-// again against activations of zero.  More than 16 rows: gridDim.y passes of 16, each streaming the weights again.
+// Every load is unconditional and the last blocks have their own copies of the code, so that the compiler's count of
+// loads in flight is exact (see dq_regres_i2.hip).  A wave whose run is shorter than the longest loads its last chunk
+// (pair) again against activations of zero.  More than 16 rows: gridDim.y passes of 16, each streaming the weights
+// again.
 #include <type_traits>
 
 #include "dq_common.h"
