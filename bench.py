@@ -535,8 +535,9 @@ def main():
         for m in (1, 16, 256, 2048):
             r = bench_bitnet(torch, tl, workloads, m, 8192, 8192, S, W, dev, **({} if m <= 16 else gemm))
             shapes.append(_row(f"bitnet_w2a8 M={m} N=8192 K=8192", r, "hbm" if m <= 16 else "mfma", MFMA_I8_PEAK))
-        r = bench_bitnet(torch, tl, workloads, 16, 28672, 8192, S, W, dev)
-        shapes.append(_row("bitnet_w2a8 M=16 N=28672 K=8192", r, "hbm", MFMA_I8_PEAK))
+        # 17 to 32 rows: the register-resident form on blocks of 32 weight rows (up to 16 rows: blocks of 16, the row above)
+        r = bench_bitnet(torch, tl, workloads, 32, 28672, 8192, S, W, dev)
+        shapes.append(_row("bitnet_w2a8 M=32 N=28672 K=8192", r, "hbm", MFMA_I8_PEAK))
         r = bench_bitnet(torch, tl, workloads, 256, 8192, 8192, S, W, dev, fragments=True, **gemm)
         shapes.append(_row("bitnet_w2a8 M=256 N=8192 K=8192 (weights re-ordered offline into the matrix instruction's operand order)",
                            r, "mfma", MFMA_I8_PEAK))

@@ -489,10 +489,11 @@ int i2_gemm_regres(const void* A, const void* B, void* C, int M, int N, int K, i
   const int npw = chunked ? kChunkPairs : (npair + kWaves - 1) / kWaves;
   const int il = (layout & ~LAYOUT_FRAGMENTS) == LAYOUT_INTERLEAVED;
   const bool frag = (layout & LAYOUT_FRAGMENTS) != 0;
-  // Up to 16 rows the form on blocks of 16 weight rows, where a workgroup has more than four of them (it holds three
-  // blocks in flight and divides the matrix evenly: N = 28672, K = 8192 16.4 against 19.0 us; with fewer blocks its
-  // longer prologue shows: N = 14336, K = 4096 8.2 against 7.9 us).
-  const bool rows16 = M <= 16 && (N + 15) / 16 > 4 * 256;
+  // Up to 16 rows the form on blocks of 16 weight rows: it divides the matrix over more workgroups and holds three
+  // blocks in flight (N = 28672, K = 8192: 15.8 against 19.0 us; N = K = 8192 at 16 rows 9.1 against 10.5 us; N = 2048,
+  // K = 8192: 7.6 against 9.8 us; N = K = 4096: 5.3 against 6.6 us).  With K below 4096 only where a workgroup has more
+  // than four of them: its longer prologue shows (N = 8192, K = 2048 at 4 and 8 rows: 4.8 against 4.5 us).
+  const bool rows16 = M <= 16 && (K >= 4096 || (N + 15) / 16 > 4 * 256);
 #define DQ_I2R(CONV_, FRAG_, NPW_, CH_)                                                                                        \
   do {                                                                                                                         \
     if (bitnet_epilogue)                                                                                                       \
