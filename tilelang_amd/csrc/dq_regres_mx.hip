@@ -368,6 +368,110 @@ int launch_mx_regres(const void* A, const void* B, const void* S, const void* Bi
   return 0;
 }
 
+// ---- one activation row: a dot-product kernel (the memory-bound decode GEMV; no matrix instruction) --------------------
+// A wave owns whole weight rows.  Lane l of step s holds the 32 codes k = 2048 s + 32 l .. + 31 of a row: 16 bytes, ONE
+// scale block, so a wave's load instruction reads 1 KiB contiguous and a lane applies one E8M0 byte per load through
+// the conversion's scale operand.  The lane's 32 activations of every step stay in registers for the whole kernel
+// (16 per step), the products are summed in fp32 with v_dot2c_f32_bf16, a row's 64 partial sums by a butterfly over
+// the lanes (fixed order).  kGemvRows rows are in flight per wave, and as many waves per SIMD as the registers allow
+// hide the rest of the latency; the waves walk the batches of rows with a stride of the whole grid.  K % 64 == 0 up to
+// 2048 STEPS: the lanes beyond a row's end read its last 16 bytes again against activations of zero.
+constexpr int kGemvRows = 4;
+
+template <int FMT, bool HAS_BIAS, int STEPS>
+__global__ __launch_bounds__(256) void mx_gemv_kernel(const bf16_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                      const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias,
+                                                      bf16_t* __restrict__ C, int N, int K, int exp_off) {
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6), nwaves = gridDim.x * 4;
+  const int nblk = K >> 5;  // scale blocks (16 bytes of codes) per row
+  const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)nblk;
+  // the lane's block of every step, and its activations (zeros beyond the row's end)
+  uint32_t blk[STEPS];
+  uint4_t a[STEPS][4];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int c = s * 64 + lane;
+    blk[s] = (uint32_t)min(c, nblk - 1);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint4_t v = *reinterpret_cast<const uint4_t*>(reinterpret_cast<const unsigned char*>(A) + (size_t)blk[s] * 64 + q * 16);
+      a[s][q] = c < nblk ? v : uint4_t{0u, 0u, 0u, 0u};
+    }
+  }
+  const int nbatch = (N + kGemvRows - 1) / kGemvRows;
+  for (int b = gw; b < nbatch; b += nwaves) {
+    uint4_t w[kGemvRows][STEPS];
+    uint32_t sc[kGemvRows][STEPS];
+#pragma unroll
+    for (int j = 0; j < kGemvRows; ++j) {
+      const int n = min(b * kGemvRows + j, N - 1);
+      const uint8_t* const w_row = B + (size_t)n * w_row_bytes;
+      const uint8_t* const s_row = S + (size_t)n * s_row_bytes;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        w[j][s] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + blk[s] * 16));
+        sc[j][s] = __builtin_nontemporal_load(s_row + blk[s]);
+      }
+    }
+    float sum[kGemvRows];
+#pragma unroll
+    for (int j = 0; j < kGemvRows; ++j) {
+      float acc = 0.f;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        const LaneScale ls = lane_scale<FMT>(sc[j][s], exp_off);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const bf16x8_t wv = decode8<FMT>(w[j][s][q], ls);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t pair = a[s][q][e];  // a value first: a bit cast of the element expression itself reads element 0
+            acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2_t{wv[2 * e], wv[2 * e + 1]}, __builtin_bit_cast(bf16x2_t, pair), acc, false);
+          }
+        }
+      }
+      sum[j] = acc;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+#pragma unroll
+      for (int j = 0; j < kGemvRows; ++j) sum[j] += __shfl_xor(sum[j], off);
+    // lane j of the first kGemvRows stores row j of the batch
+    float mine = sum[0];
+#pragma unroll
+    for (int j = 1; j < kGemvRows; ++j) mine = lane == j ? sum[j] : mine;
+    const int n = b * kGemvRows + lane;
+    if (lane < kGemvRows && n < N) {
+      // reference: C = bf16(float(acc) + float(Bias))
+      if constexpr (HAS_BIAS) mine += (float)Bias[n];
+      C[n] = (bf16_t)mine;
+    }
+  }
+}
+
+template <int FMT, bool HAS_BIAS, int STEPS>
+int launch_mx_gemv(const void* A, const void* B, const void* S, const void* Bias, void* C, int N, int K, int exp_off,
+                   hipStream_t stream) {
+  auto kern = mx_gemv_kernel<FMT, HAS_BIAS, STEPS>;
+  static int cus_of[kMaxDevices] = {}, per_cu[kMaxDevices] = {};
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
+  if (!cus_of[device]) {
+    DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
+    DQ_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[device], kern, 256, 0));
+    if (per_cu[device] < 1) per_cu[device] = 1;
+  }
+  // every workgroup resident at once; no more waves than batches of rows
+  const int nbatch = (N + kGemvRows - 1) / kGemvRows;
+  const int want = (nbatch + 3) / 4, room = cus_of[device] * per_cu[device];
+  hipLaunchKernelGGL(kern, dim3(want < room ? want : room), dim3(256), 0, stream, (const bf16_t*)A, (const uint8_t*)B,
+                     (const uint8_t*)S, (const bf16_t*)Bias, (bf16_t*)C, N, K, exp_off);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 }  // namespace
 
 // 0: launched; 1: this shape is not the kernel's (the caller goes on to the tiled GEMM); -1: error.
@@ -393,6 +497,30 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
     if (t_here > 0.9 * t_tiled) return 1;
   }
   const int exp_off = 127 - scale_bias;
+  if (M == 1 && K <= 8192) {  // one row: the dot-product kernel
+#define DQ_MXV(FMT_, STEPS_)                                                                                  \
+  do {                                                                                                        \
+    if (Bias) return launch_mx_gemv<FMT_, true, STEPS_>(A, B, S, Bias, C, N, K, exp_off, stream);             \
+    return launch_mx_gemv<FMT_, false, STEPS_>(A, B, S, nullptr, C, N, K, exp_off, stream);                   \
+  } while (0)
+#define DQ_MXVN(FMT_)                 \
+  do {                                \
+    switch ((K + 2047) / 2048) {      \
+      case 1: DQ_MXV(FMT_, 1);        \
+      case 2: DQ_MXV(FMT_, 2);        \
+      case 3: DQ_MXV(FMT_, 3);        \
+      default: DQ_MXV(FMT_, 4);       \
+    }                                 \
+  } while (0)
+    switch (fmt) {
+      case FP4_E2M1: DQ_MXVN(FP4_E2M1);
+      case FP4_SIMPLE: DQ_MXVN(FP4_SIMPLE);
+      case FP4_TWIDDLING: DQ_MXVN(FP4_TWIDDLING);
+      default: DQ_FAIL("mxfp4 gemm: unknown weight format %d", fmt);
+    }
+#undef DQ_MXVN
+#undef DQ_MXV
+  }
   const bool half = K % 128 != 0;
   const int lines = K % 4096 == 0 ? 2 : (K % 256 == 0 ? 1 : 0);
   // chunks per wave: the longest run (with lines, whole pairs)
