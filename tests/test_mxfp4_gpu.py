@@ -85,7 +85,9 @@ def test_many_tiles(cuda, fmt, with_bias):
                                    # K % 256 == 0: whole pairs of chunks per wave, runs of unequal length (7168 = 28 pairs, 256 = 1)
                                    (9, 700, 7168), (16, 130, 256), (2, 48, 3584),
                                    # one row up to K = 8192: the dot-product kernel (whole rows per wave, lanes beyond a row's end idle)
-                                   (1, 300, 1024), (1, 1001, 2880), (1, 4100, 8192), (1, 513, 5120), (1, 5, 64), (1, 9000, 7168), (1, 31, 4160)])
+                                   (1, 300, 1024), (1, 1001, 2880), (1, 4100, 8192), (1, 513, 5120), (1, 5, 64), (1, 9000, 7168), (1, 31, 4160),
+                                   # two rows: the same with the activations in LDS
+                                   (2, 4100, 8192), (2, 1001, 5120), (2, 515, 1024), (2, 9000, 7168), (2, 7, 64)])
 def test_decode_batches(cuda, fmt, with_bias, M, N, K):
     """Decode batches with K a multiple of 64 (of 128 beyond 8192): the kernel that keeps the activations in registers
     and streams weights and scale bytes once per 16 rows.  Ragged N (last block of 16 weight rows, N % 4 != 0), K slices of unequal

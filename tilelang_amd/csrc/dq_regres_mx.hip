@@ -472,6 +472,114 @@ int launch_mx_gemv(const void* A, const void* B, const void* S, const void* Bias
   return 0;
 }
 
+// ---- two activation rows (the kernel takes up to four): the same dot-product kernel with the activations in LDS -----------
+// MR rows of 32 activations per lane and step would not fit the registers beside the weights in flight: the workgroup
+// copies the rows to LDS once ([row][step][piece of 16 bytes][lane]: a wave's read is 1 KiB contiguous), and a step's
+// fragments of all rows are read once per batch of kGemvRows weight rows; every weight dword is converted once and
+// multiplied into all rows.  The MR x kGemvRows sums of a batch are added over the lanes by the halving reduction
+// (RowReduce over each 16 lanes, then two butterflies): lane 4 m + j ends up with row m of the batch's weight row j.
+template <int FMT, bool HAS_BIAS, int STEPS, int MR>
+__global__ __launch_bounds__(256) void mx_gemv_rows_kernel(const bf16_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                           const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias,
+                                                           bf16_t* __restrict__ C, int M, int N, int K, int exp_off) {
+  static_assert(MR * kGemvRows <= 16, "one value per lane of a DPP row");
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int gw = blockIdx.x * 4 + (tid >> 6), nwaves = gridDim.x * 4;
+  const int nblk = K >> 5;  // scale blocks (16 bytes of codes, 64 bytes of activations) per row
+  const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)nblk;
+  for (int p = tid; p < MR * STEPS * 256; p += 256) {  // source order: piece q of block 64 s + l of row m at p = ((m STEPS + s) 64 + l) 4 + q
+    const int q = p & 3, l = (p >> 2) & 63, ms = p >> 8;
+    const int m = ms / STEPS, c = (ms % STEPS) * 64 + l;
+    uint4_t v = {0u, 0u, 0u, 0u};  // rows beyond M, blocks beyond the row's end
+    if (m < M && c < nblk) v = *reinterpret_cast<const uint4_t*>(reinterpret_cast<const unsigned char*>(A) + (size_t)m * K * 2 + (size_t)c * 64 + q * 16);
+    *reinterpret_cast<uint4_t*>(smem + ((ms * 4 + q) * 64 + l) * 16) = v;
+  }
+  __syncthreads();
+  uint32_t blk[STEPS];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) blk[s] = (uint32_t)min(s * 64 + lane, nblk - 1);
+  const int nbatch = (N + kGemvRows - 1) / kGemvRows;
+  for (int b = gw; b < nbatch; b += nwaves) {
+    uint4_t w[kGemvRows][STEPS];
+    uint32_t sc[kGemvRows][STEPS];
+#pragma unroll
+    for (int j = 0; j < kGemvRows; ++j) {
+      const int n = min(b * kGemvRows + j, N - 1);
+      const uint8_t* const w_row = B + (size_t)n * w_row_bytes;
+      const uint8_t* const s_row = S + (size_t)n * s_row_bytes;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        w[j][s] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + blk[s] * 16));
+        sc[j][s] = __builtin_nontemporal_load(s_row + blk[s]);
+      }
+    }
+    float acc[16];  // [m][j]
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      uint4_t af[MR][4];
+#pragma unroll
+      for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) af[m][q] = *reinterpret_cast<const uint4_t*>(smem + (((m * STEPS + s) * 4 + q) * 64 + lane) * 16);
+#pragma unroll
+      for (int j = 0; j < kGemvRows; ++j) {
+        const LaneScale ls = lane_scale<FMT>(sc[j][s], exp_off);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const bf16x8_t wv = decode8<FMT>(w[j][s][q], ls);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bf16x2_t wp = {wv[2 * e], wv[2 * e + 1]};
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+              const uint32_t pair = af[m][q][e];  // a value first (see mx_gemv_kernel)
+              acc[m * kGemvRows + j] = __builtin_amdgcn_fdot2_f32_bf16(wp, __builtin_bit_cast(bf16x2_t, pair), acc[m * kGemvRows + j], false);
+            }
+          }
+        }
+      }
+      // a step's fragments are read when the step before is done: hoisted, the fragments of all steps are live at once
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    float t = RowReduce<16, 0>::run(acc, lane);
+    t += __shfl_xor(t, 16);
+    t += __shfl_xor(t, 32);
+    const int m = (lane >> 2) & 3, n = b * kGemvRows + (lane & 3);
+    if (lane < 16 && m < M && n < N) {
+      // reference: C = bf16(float(acc) + float(Bias))
+      if constexpr (HAS_BIAS) t += (float)Bias[(size_t)m * N + n];
+      C[(size_t)m * N + n] = (bf16_t)t;
+    }
+  }
+}
+
+template <int FMT, bool HAS_BIAS, int STEPS, int MR>
+int launch_mx_gemv_rows(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K,
+                        int exp_off, hipStream_t stream) {
+  auto kern = mx_gemv_rows_kernel<FMT, HAS_BIAS, STEPS, MR>;
+  constexpr int kLdsA = MR * STEPS * 4096;
+  static bool raised[kMaxDevices] = {};
+  if (raise_lds_limit<kLdsA>(kern, raised)) return -1;
+  static int cus_of[kMaxDevices] = {}, per_cu[kMaxDevices] = {};
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
+  if (!cus_of[device]) {
+    DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
+    DQ_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[device], kern, 256, kLdsA));
+    if (per_cu[device] < 1) per_cu[device] = 1;
+  }
+  const int nbatch = (N + kGemvRows - 1) / kGemvRows;
+  const int want = (nbatch + 3) / 4, room = cus_of[device] * per_cu[device];
+  hipLaunchKernelGGL(kern, dim3(want < room ? want : room), dim3(256), kLdsA, stream, (const bf16_t*)A, (const uint8_t*)B,
+                     (const uint8_t*)S, (const bf16_t*)Bias, (bf16_t*)C, M, N, K, exp_off);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 }  // namespace
 
 // 0: launched; 1: this shape is not the kernel's (the caller goes on to the tiled GEMM); -1: error.
@@ -520,6 +628,33 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
     }
 #undef DQ_MXVN
 #undef DQ_MXV
+  }
+  // Two rows: the dot-product kernel with the activations in LDS (N = K = 8192: 10.1 against 12.7 us; N = 28672: level).
+  // With four rows its 64 dot products per 16 bytes of weights are what binds (N = 28672, K = 8192: 31 against 25.5 us):
+  // three and more rows go to the matrix-instruction kernel below.
+  if (M == 2 && K <= 8192) {
+#define DQ_MXW(FMT_, STEPS_)                                                                                   \
+  do {                                                                                                         \
+    if (Bias) return launch_mx_gemv_rows<FMT_, true, STEPS_, 2>(A, B, S, Bias, C, M, N, K, exp_off, stream);   \
+    return launch_mx_gemv_rows<FMT_, false, STEPS_, 2>(A, B, S, nullptr, C, M, N, K, exp_off, stream);         \
+  } while (0)
+#define DQ_MXWN(FMT_)                 \
+  do {                                \
+    switch ((K + 2047) / 2048) {      \
+      case 1: DQ_MXW(FMT_, 1);        \
+      case 2: DQ_MXW(FMT_, 2);        \
+      case 3: DQ_MXW(FMT_, 3);        \
+      default: DQ_MXW(FMT_, 4);       \
+    }                                 \
+  } while (0)
+    switch (fmt) {
+      case FP4_E2M1: DQ_MXWN(FP4_E2M1);
+      case FP4_SIMPLE: DQ_MXWN(FP4_SIMPLE);
+      case FP4_TWIDDLING: DQ_MXWN(FP4_TWIDDLING);
+      default: DQ_FAIL("mxfp4 gemm: unknown weight format %d", fmt);
+    }
+#undef DQ_MXWN
+#undef DQ_MXW
   }
   const bool half = K % 128 != 0;
   const int lines = K % 4096 == 0 ? 2 : (K % 256 == 0 ? 1 : 0);
