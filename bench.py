@@ -529,6 +529,9 @@ def main():
         r = bench_mxfp4(torch, tl, workloads, 4096, 8192, 8192, S, W, dev, **gemm)
         mx_run = r
         shapes.append(_row("mxfp4_gemm M=4096 N=8192 K=8192", r, "mfma", MFMA_BF16_PEAK))
+        # MXFP4 weights at one row, the headline matrix's shape: the dot-product kernel (no matrix instruction)
+        r = bench_mxfp4(torch, tl, workloads, 1, 28672, 8192, S, W, dev)
+        shapes.append(_row("mxfp4_gemv M=1 N=28672 K=8192", r, "hbm", MFMA_BF16_PEAK))
         # the same weights at a decode batch: activations resident in registers, weights streamed once
         r = bench_mxfp4(torch, tl, workloads, 16, 8192, 8192, S, W, dev)
         shapes.append(_row("mxfp4_gemm M=16 N=8192 K=8192", r, "hbm", MFMA_BF16_PEAK))
