@@ -87,7 +87,10 @@ def test_many_tiles(cuda, fmt, with_bias):
                                    # one row up to K = 8192: the dot-product kernel (whole rows per wave, lanes beyond a row's end idle)
                                    (1, 300, 1024), (1, 1001, 2880), (1, 4100, 8192), (1, 513, 5120), (1, 5, 64), (1, 9000, 7168), (1, 31, 4160),
                                    # two rows: the same with the activations in LDS
-                                   (2, 4100, 8192), (2, 1001, 5120), (2, 515, 1024), (2, 9000, 7168), (2, 7, 64)])
+                                   (2, 4100, 8192), (2, 1001, 5120), (2, 515, 1024), (2, 9000, 7168), (2, 7, 64),
+                                   # one and two rows beyond K = 8192: chunks of four steps, activations padded to whole chunks in LDS
+                                   (1, 300, 14336), (2, 1001, 16384), (1, 64, 28672), (2, 130, 8320), (1, 4100, 12288), (2, 33, 32768),
+                                   (1, 40, 40960)])
 def test_decode_batches(cuda, fmt, with_bias, M, N, K):
     """Decode batches with K a multiple of 64 (of 128 beyond 8192): the kernel that keeps the activations in registers
     and streams weights and scale bytes once per 16 rows.  Ragged N (last block of 16 weight rows, N % 4 != 0), K slices of unequal

@@ -580,6 +580,114 @@ int launch_mx_gemv_rows(const void* A, const void* B, const void* S, const void*
   return 0;
 }
 
+// ---- one and two activation rows with K beyond 8192: the dot-product kernel over chunks of four steps ---------------------
+// As mx_gemv_rows_kernel (activations in LDS, padded with zeros to whole chunks), the loop over K in chunks of four
+// steps (8192 k): a chunk's 16 loads of a batch of four weight rows are asked for, waited for and multiplied, the
+// sums carried from chunk to chunk; the other waves of the SIMD cover the wait.
+template <int FMT, bool HAS_BIAS, int MR>
+__global__ __launch_bounds__(256) void mx_gemv_long_kernel(const bf16_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                           const uint8_t* __restrict__ S, const bf16_t* __restrict__ Bias,
+                                                           bf16_t* __restrict__ C, int M, int N, int K, int exp_off) {
+  static_assert(MR * kGemvRows <= 16, "one value per lane of a DPP row");
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int gw = blockIdx.x * 4 + (tid >> 6), nwaves = gridDim.x * 4;
+  const int nblk = K >> 5;
+  const int nchunk = (nblk + 255) >> 8, nsteps = 4 * nchunk;  // steps of 64 blocks, padded to whole chunks
+  const uint32_t w_row_bytes = (uint32_t)(K >> 1), s_row_bytes = (uint32_t)nblk;
+  for (int p = tid; p < MR * nsteps * 256; p += 256) {  // piece q of block 64 s + l of row m at p = ((m nsteps + s) 64 + l) 4 + q
+    const int q = p & 3, l = (p >> 2) & 63, ms = p >> 8;
+    const int m = ms / nsteps, c = (ms % nsteps) * 64 + l;
+    uint4_t v = {0u, 0u, 0u, 0u};  // rows beyond M, blocks beyond the row's end
+    if (m < M && c < nblk) v = *reinterpret_cast<const uint4_t*>(reinterpret_cast<const unsigned char*>(A) + (size_t)m * K * 2 + (size_t)c * 64 + q * 16);
+    *reinterpret_cast<uint4_t*>(smem + ((ms * 4 + q) * 64 + l) * 16) = v;
+  }
+  __syncthreads();
+  const int nbatch = (N + kGemvRows - 1) / kGemvRows;
+  for (int b = gw; b < nbatch; b += nwaves) {
+    float acc[16];  // [m][j]
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    for (int ch = 0; ch < nchunk; ++ch) {
+      uint4_t w[kGemvRows][4];
+      uint32_t sc[kGemvRows][4];
+#pragma unroll
+      for (int j = 0; j < kGemvRows; ++j) {
+        const int n = min(b * kGemvRows + j, N - 1);
+        const uint8_t* const w_row = B + (size_t)n * w_row_bytes;
+        const uint8_t* const s_row = S + (size_t)n * s_row_bytes;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const uint32_t blk = (uint32_t)min((4 * ch + s) * 64 + lane, nblk - 1);
+          w[j][s] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(w_row + blk * 16));
+          sc[j][s] = __builtin_nontemporal_load(s_row + blk);
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        uint4_t af[MR][4];
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) af[m][q] = *reinterpret_cast<const uint4_t*>(smem + (((m * nsteps + 4 * ch + s) * 4 + q) * 64 + lane) * 16);
+#pragma unroll
+        for (int j = 0; j < kGemvRows; ++j) {
+          const LaneScale ls = lane_scale<FMT>(sc[j][s], exp_off);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const bf16x8_t wv = decode8<FMT>(w[j][s][q], ls);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const bf16x2_t wp = {wv[2 * e], wv[2 * e + 1]};
+#pragma unroll
+              for (int m = 0; m < MR; ++m) {
+                const uint32_t pair = af[m][q][e];  // a value first (see mx_gemv_kernel)
+                acc[m * kGemvRows + j] = __builtin_amdgcn_fdot2_f32_bf16(wp, __builtin_bit_cast(bf16x2_t, pair), acc[m * kGemvRows + j], false);
+              }
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // a step's fragments are read when the step before is done
+      }
+    }
+    float t = RowReduce<16, 0>::run(acc, lane);
+    t += __shfl_xor(t, 16);
+    t += __shfl_xor(t, 32);
+    const int m = (lane >> 2) & 3, n = b * kGemvRows + (lane & 3);
+    if (lane < 16 && m < M && n < N) {
+      // reference: C = bf16(float(acc) + float(Bias))
+      if constexpr (HAS_BIAS) t += (float)Bias[(size_t)m * N + n];
+      C[(size_t)m * N + n] = (bf16_t)t;
+    }
+  }
+}
+
+constexpr int kGemvLongMaxK = 32768;  // two rows of activations: 128 KiB of LDS
+
+template <int FMT, bool HAS_BIAS, int MR>
+int launch_mx_gemv_long(const void* A, const void* B, const void* S, const void* Bias, void* C, int M, int N, int K,
+                        int exp_off, hipStream_t stream) {
+  auto kern = mx_gemv_long_kernel<FMT, HAS_BIAS, MR>;
+  static bool raised[kMaxDevices] = {};
+  if (raise_lds_limit<MR * (kGemvLongMaxK / 2048) * 4096>(kern, raised)) return -1;
+  const int nchunk = ((K >> 5) + 255) >> 8;
+  const int lds = MR * 4 * nchunk * 4096;
+  static int cus_of[kMaxDevices] = {};
+  int device = 0;
+  DQ_CHECK_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
+  if (!cus_of[device]) DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
+  int per_cu = 0;  // depends on K through the LDS a workgroup takes
+  DQ_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds));
+  if (per_cu < 1) per_cu = 1;
+  const int nbatch = (N + kGemvRows - 1) / kGemvRows;
+  const int want = (nbatch + 3) / 4, room = cus_of[device] * per_cu;
+  hipLaunchKernelGGL(kern, dim3(want < room ? want : room), dim3(256), lds, stream, (const bf16_t*)A, (const uint8_t*)B,
+                     (const uint8_t*)S, (const bf16_t*)Bias, (bf16_t*)C, M, N, K, exp_off);
+  DQ_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
 }  // namespace
 
 // 0: launched; 1: this shape is not the kernel's (the caller goes on to the tiled GEMM); -1: error.
@@ -655,6 +763,24 @@ int mxfp4_gemm_regres(const void* A, const void* B, const void* S, const void* B
     }
 #undef DQ_MXWN
 #undef DQ_MXW
+  }
+  if (M <= 2 && K > 8192 && K <= kGemvLongMaxK) {  // one and two rows, long K: the dot-product kernel over chunks of K
+#define DQ_MXL(FMT_)                                                                                               \
+  do {                                                                                                             \
+    if (M == 1) {                                                                                                  \
+      if (Bias) return launch_mx_gemv_long<FMT_, true, 1>(A, B, S, Bias, C, M, N, K, exp_off, stream);             \
+      return launch_mx_gemv_long<FMT_, false, 1>(A, B, S, nullptr, C, M, N, K, exp_off, stream);                   \
+    }                                                                                                              \
+    if (Bias) return launch_mx_gemv_long<FMT_, true, 2>(A, B, S, Bias, C, M, N, K, exp_off, stream);               \
+    return launch_mx_gemv_long<FMT_, false, 2>(A, B, S, nullptr, C, M, N, K, exp_off, stream);                     \
+  } while (0)
+    switch (fmt) {
+      case FP4_E2M1: DQ_MXL(FP4_E2M1);
+      case FP4_SIMPLE: DQ_MXL(FP4_SIMPLE);
+      case FP4_TWIDDLING: DQ_MXL(FP4_TWIDDLING);
+      default: DQ_FAIL("mxfp4 gemm: unknown weight format %d", fmt);
+    }
+#undef DQ_MXL
   }
   const bool half = K % 128 != 0;
   const int lines = K % 4096 == 0 ? 2 : (K % 256 == 0 ? 1 : 0);
