@@ -187,3 +187,39 @@ def test_graph_replays_match_eager_decode_and_half_tile_kernels(cuda):
         torch.cuda.synchronize()
         for got, want in zip(outs + [c4_g], eager):
             assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+
+
+def test_graph_replays_match_eager_mxfp4_decode_kernels(cuda):
+    """The MXFP4 dot-product kernels (one row; two rows with the activations in LDS; K beyond 8192 in chunks), the
+    register-resident MXFP4 kernel at 16 rows and the 16-row BitNet form on a small matrix, under capture."""
+    cases = [(1, 1001, 4096), (2, 515, 8192), (1, 300, 16384), (2, 130, 12288), (16, 1000, 8192)]
+    runs = []
+    for i, (M, N, K) in enumerate(cases):
+        d = workloads.mxfp4(M, N, K, seed=30 + i, scale_bias=127)
+        kern = tl.matmul_bf16_mxfp4(M, N, K, weight_format="e2m1", scale_bias=127)
+        A, B, S = _dev(d["A"], cuda).view(torch.bfloat16), _dev(d["B"], cuda), _dev(d["Scale"], cuda)
+        bias = torch.empty((M, N), dtype=torch.bfloat16, device=cuda)
+        runs.append((kern, (A, B, S, bias)))
+    M5, N5, K5 = 16, 1000, 4096
+    d5 = workloads.bitnet(M5, N5, K5, seed=40)
+    bl = tl.bitlinear_int8xint2(M5, N5, K5, float(d5["s_w"]))
+    A5, B5, sa5 = _dev(d5["A"], cuda), _dev(d5["B"], cuda).view(torch.int8), _dev(d5["s_a"], cuda)
+
+    def run():
+        return [k(*a) for k, a in runs] + [bl(A5, B5, sa5)]
+
+    eager = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            outs = run()
+    for _ in range(3):
+        for t in outs:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))

@@ -677,9 +677,13 @@ int launch_mx_gemv_long(const void* A, const void* B, const void* S, const void*
   DQ_CHECK_HIP(hipGetDevice(&device));
   if (device < 0 || device >= kMaxDevices) DQ_FAIL("device index %d is beyond the %d this library keeps state for", device, kMaxDevices);
   if (!cus_of[device]) DQ_CHECK_HIP(hipDeviceGetAttribute(&cus_of[device], hipDeviceAttributeMultiprocessorCount, device));
-  int per_cu = 0;  // depends on K through the LDS a workgroup takes
-  DQ_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds));
-  if (per_cu < 1) per_cu = 1;
+  // workgroups per CU: depends on K through the LDS a workgroup takes (asked once per device and chunk count)
+  static int per_cu_of[kMaxDevices][kGemvLongMaxK / 8192 + 1] = {};
+  int& per_cu = per_cu_of[device][nchunk];
+  if (!per_cu) {
+    DQ_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds));
+    if (per_cu < 1) per_cu = 1;
+  }
   const int nbatch = (N + kGemvRows - 1) / kGemvRows;
   const int want = (nbatch + 3) / 4, room = cus_of[device] * per_cu;
   hipLaunchKernelGGL(kern, dim3(want < room ? want : room), dim3(256), lds, stream, (const bf16_t*)A, (const uint8_t*)B,
