@@ -467,6 +467,8 @@ def test_bitnet_fragment_ordered_weights_where_no_kernel_reads_them(cuda):
                                    (64, 300, 4096), (100, 1001, 2048), (128, 2560, 1280), (33, 5000, 512),
                                    # up to 16 rows: blocks of 16 weight rows, four sets of weight registers in turn
                                    (16, 28677, 8192), (3, 9000, 2560), (12, 16 * 256 * 6 + 5, 512), (16, 16 * 256 * 4, 1024),
+                                   # the same form on small and ragged matrices (K >= 4096 at any N): fewer blocks than CUs, one or two per workgroup
+                                   (16, 100, 4352), (7, 1000, 5120), (16, 4097, 7936), (12, 33, 8192), (9, 2048, 6144),
                                    # K beyond what the registers hold: chunks of K, running sums in LDS
                                    (8, 300, 11008), (32, 1001, 16384), (5, 9000, 28672), (17, 64, 8448), (64, 200, 12288)])
 @pytest.mark.parametrize("interleaved", [True, False])
