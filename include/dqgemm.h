@@ -142,7 +142,11 @@ enum dq_fp4_format {
  * fp32 accumulation.  Replaces `call(A, B, Scale, Bias, C, stream)` of the kernel generated from
  * examples/dequantize_gemm/example_dequant_gemm_bf16_mxfp4_cdna4.py:201-244.  The reference
  * multiplies by 2^Scale with the raw byte (:254-267): scale_bias = 0; an E8M0 scale is
- * scale_bias = 127.  Bias may be NULL.  Requires K % 64 == 0, scale_size == 32. */
+ * scale_bias = 127.  Bias may be NULL.  Requires K % 64 == 0, scale_size == 32.
+ * The library picks the kernel by shape (one and two rows up to K = 32768: a dot-product kernel on whole weight
+ * rows; up to 16 rows, more while passes of 16 stay ahead: the activations resident in registers and the weights
+ * streamed once; else the tiled GEMM).  Each adds the same products in fp32 in an order of its own: a row computed
+ * in a small batch and in a large one may differ in the last bf16 bit; every call of one shape returns the same bits. */
 int call_dequant_gemm_bf16_mxfp4(const void* A, const void* B, const void* Scale, const void* Bias, void* C, int M,
                                  int N, int K, int scale_size, int fp4_format, int scale_bias, dq_stream_t stream);
 
